@@ -1,0 +1,157 @@
+/*
+ * strix_mi355.h — C ABI of the MI355X (gfx950) quantized-matmul backend.
+ *
+ * This is the boundary a Strix.rs `WeightAccel` implementation binds to
+ * (trait: crates/strix-core/src/accel.rs:147).  Each entry point names the
+ * trait method / reference function it stands in for.  Plain pointers and
+ * sizes only.
+ *
+ * Return convention (all int-returning calls):
+ *     1   done
+ *     0   declined exactly where the reference declines with `false`/`None`
+ *         because the key/layer is not resident (accel.rs:142-146)
+ *    <0   error (SMX_ERR_*); text via smx_last_error().  There is no CPU
+ *         fallback inside the library.
+ *
+ * One context = one device + one HIP stream.  Calls on one context must be
+ * serialised by the caller (the reference is driven the same way,
+ * crates/strix-backend-rocm/src/decode.rs:559-562); distinct contexts are
+ * independent.  Host-pointer entry points copy in, run, copy out and
+ * synchronise; `_dev` entry points take device pointers, enqueue on the
+ * context's stream and return without synchronising.
+ */
+#ifndef STRIX_MI355_H
+#define STRIX_MI355_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct smx_ctx smx_ctx;
+
+enum {
+    SMX_OK = 1,
+    SMX_NOT_RESIDENT = 0,
+    SMX_ERR_ARG = -1,    /* null pointer, bad size, shape mismatch */
+    SMX_ERR_HIP = -2,    /* a HIP runtime call failed */
+    SMX_ERR_LIMIT = -3,  /* a documented limit exceeded */
+    SMX_ERR_NOMEM = -4   /* device or host allocation failed */
+};
+
+/* ---- context: replaces HipGpu::new + kernel compilation,
+ *      crates/strix-backend-rocm/src/hip.rs:135-160, decode.rs:563-830 ---- */
+int smx_create(int device, smx_ctx** out);
+void smx_destroy(smx_ctx* ctx); /* frees every device buffer the context owns */
+/* Last error text of this context (of the calling thread's last failed
+ * smx_create when ctx is NULL).  Valid until the next call on the context. */
+const char* smx_last_error(const smx_ctx* ctx);
+const char* smx_name(const smx_ctx* ctx);          /* WeightAccel::name, accel.rs:405 */
+size_t smx_resident_count(const smx_ctx* ctx);     /* WeightAccel::resident_count, accel.rs:402 */
+size_t smx_resident_bytes(const smx_ctx* ctx);     /* device bytes held by resident weights */
+
+/* ---- weight upload: raw GGUF block bytes, [out_dim rows][in_dim/QK blocks].
+ *      The bytes are copied; the caller may drop them afterwards.
+ *      Re-uploading a key replaces the previous weight. ---- */
+/* WeightAccel::upload_q4_0, accel.rs:150; decode.rs:2491-2521 */
+int smx_upload_q4_0(smx_ctx* ctx, const char* key, const void* bytes, size_t nbytes,
+                    size_t in_dim, size_t out_dim);
+/* WeightAccel::upload_q8_0, accel.rs:163; decode.rs:2683-2714 */
+int smx_upload_q8_0(smx_ctx* ctx, const char* key, const void* bytes, size_t nbytes,
+                    size_t in_dim, size_t out_dim);
+/* WeightAccel::upload_q6_k, accel.rs:159; decode.rs:2629-2681 */
+int smx_upload_q6_k(smx_ctx* ctx, const char* key, const void* bytes, size_t nbytes,
+                    size_t in_dim, size_t out_dim);
+/* WeightAccel::upload_moe_q8, accel.rs:170-181; decode.rs:2717-2791.
+ * gate/up: ne experts x [eff rows][hidden/32 blocks]; down: ne x [hidden rows][eff/32]. */
+int smx_upload_moe_q8(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_nbytes,
+                      const void* up, size_t up_nbytes, const void* down, size_t down_nbytes,
+                      size_t hidden, size_t eff, size_t ne);
+/* Drop one resident weight (the reference never frees, decode.rs:458-460). */
+int smx_evict(smx_ctx* ctx, const char* key);
+
+/* ---- decode GEMV ---- */
+/* WeightAccel::gemv, accel.rs:391; decode.rs:3827-3898.  y = W.x with x
+ * quantised per 32-block on the device (kernels.rs:75-96) and integer block
+ * dots (kernels.rs:259-287, 894-912).  in_len must equal in_dim, out_cap >= out_dim. */
+int smx_gemv(smx_ctx* ctx, const char* key, const float* x, size_t in_len, float* y,
+             size_t out_cap);
+/* Small-batch GEMV, m <= SMX_GEMV_MAX_M rows against one weight read once
+ * (kernels.rs:1016-1045, the n-gram verify path): xs[m][in_dim] -> y[m][out_dim]. */
+#define SMX_GEMV_MAX_M 8
+int smx_gemv_rows(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim,
+                  float* y, size_t y_cap);
+/* WeightAccel::gemv_batch, accel.rs:397; decode.rs:3227-3255.  n (key, x)
+ * pairs, one device job, one sync.  status[i] receives the per-item code. */
+int smx_gemv_batch(smx_ctx* ctx, size_t n, const char* const* keys, const float* const* xs,
+                   const size_t* in_lens, float* const* ys, const size_t* out_caps, int* status);
+
+/* ---- prefill GEMM ---- */
+/* WeightAccel::prefill_q8_gemm, accel.rs:213; decode.rs:3257-3297 (and the
+ * Q4_0 GEMMs kernels.rs:481-601).  xs[m][in_dim] -> y[m][out_dim], any
+ * resident Q4_0/Q8_0 weight, any m; split-K is chosen internally. */
+int smx_gemm(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim, float* y,
+             size_t y_cap);
+/* WeightAccel::lm_head_argmax_rows, accel.rs:217; decode.rs:3631-3690.
+ * out[t] = argmax_r (W.xs[t])[r], lowest index on ties. */
+int smx_lm_head_argmax_rows(smx_ctx* ctx, const char* key, const float* xs, size_t m,
+                            size_t in_dim, uint32_t* out);
+
+/* ---- MoE ---- */
+/* WeightAccel::moe_ffn, accel.rs:201-210; decode.rs:2833-2870, 1923-2128.
+ * y[hidden] = sum_k wexp[k] * down_k( silu(gate_k x) * (up_k x) ), k routed
+ * experts accumulated in routed order.  sgate must be 0 (no shared expert). */
+int smx_moe_ffn(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
+                const float* x, size_t x_len, float sgate, float* y, size_t y_cap);
+/* WeightAccel::moe_layer_q8_dev, accel.rs:311-321; decode.rs:1608-1739.
+ * xs[m][hidden]; plan[nplan][3] = (expert, slot_off, count); slot_tok[slots],
+ * wslot[slots]; y[m][hidden] = sum over the token's slots (ascending slot
+ * index) of wslot * expert_ffn(xs[token]). */
+int smx_moe_layer(smx_ctx* ctx, size_t layer, const float* xs, size_t m, const size_t* plan,
+                  size_t nplan, const int32_t* slot_tok, const float* wslot, size_t slots,
+                  float* y, size_t y_cap);
+
+/* ---- device-resident variants (async on the context's stream) ---- */
+int smx_dev_alloc(smx_ctx* ctx, size_t nbytes, void** dptr);
+int smx_dev_free(smx_ctx* ctx, void* dptr);
+int smx_h2d(smx_ctx* ctx, void* dst_dev, const void* src_host, size_t nbytes);
+int smx_d2h(smx_ctx* ctx, void* dst_host, const void* src_dev, size_t nbytes); /* syncs */
+int smx_sync(smx_ctx* ctx);
+int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
+int smx_gemm_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
+int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
+                    const float* x_dev, float* y_dev);
+
+/* ---- per-kernel timing: the role of STRIX_PROF, decode.rs:25-69, 2190-2203,
+ *      done with HIP events on the context's stream instead of host syncs ---- */
+int smx_prof_enable(smx_ctx* ctx, int on);   /* on: bracket each matmul kernel with an event pair */
+int smx_prof_reset(smx_ctx* ctx);
+/* Total milliseconds and launch count recorded for kernels whose name starts
+ * with `prefix` (syncs the stream).  Names: smx_prof_names(). */
+int smx_prof_read(smx_ctx* ctx, const char* prefix, double* total_ms, size_t* launches);
+const char* smx_prof_names(smx_ctx* ctx);    /* comma-separated kernel names seen so far */
+/* Stream-level stopwatch: events around whatever is enqueued in between. */
+int smx_timer_begin(smx_ctx* ctx);
+int smx_timer_end(smx_ctx* ctx, float* ms);  /* syncs */
+
+/* ---- parity instrumentation (same device code path, integer results dumped) ---- */
+/* Device activation quantiser: xq[m][k] i8, xd[m][k/32] f32, xs16[m][k/16] i16. */
+int smx_quantize(smx_ctx* ctx, const float* x, size_t m, size_t k, int8_t* xq, float* xd,
+                 int16_t* xs16);
+/* Per-block i32 dots formed by the GEMV kernel: out[out_dim][in_dim/32]
+ * (Q6_K: [out_dim][in_dim/16]). */
+int smx_gemv_block_dots(smx_ctx* ctx, const char* key, const float* x, size_t in_len,
+                        int32_t* out, size_t out_cap);
+/* Per-block i32 accumulators formed by the MFMA GEMM: out[m][out_dim][in_dim/32]. */
+int smx_gemm_block_dots(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim,
+                        int32_t* out, size_t out_cap);
+/* smx_moe_ffn with its intermediate stages: gu[k][2][eff] (gate, up outputs),
+ * aq[k][eff] / ad[k][eff/32] (quantised silu(g)*u).  Any of them may be NULL. */
+int smx_moe_ffn_stages(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
+                       const float* x, size_t x_len, float* y, float* gu, int8_t* aq, float* ad);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

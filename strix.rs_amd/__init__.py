@@ -1,0 +1,321 @@
+"""Python binding of libstrix_mi355.so (ctypes over the C ABI in include/strix_mi355.h).
+
+`Mi355WeightAccel` mirrors the method names, argument meaning and decline
+behaviour of the reference's `WeightAccel` trait
+(crates/strix-core/src/accel.rs:147-405): `upload_*` return True/False, `gemv`
+and friends return a numpy array or None when the key is not resident.  Errors
+the reference would swallow into a decline (bad shapes, HIP failures) raise
+`SmxError` instead, since this backend has no CPU fallback to decline to.
+
+The directory name contains a dot, so load this package by path, e.g.
+    importlib.util.spec_from_file_location("strix_rs_amd", ".../strix.rs_amd/__init__.py",
+                                           submodule_search_locations=[".../strix.rs_amd"])
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libstrix_mi355.so")
+
+SMX_OK, SMX_NOT_RESIDENT = 1, 0
+GEMV_MAX_M = 8
+
+EXPORTS = [
+    "smx_create", "smx_destroy", "smx_last_error", "smx_name", "smx_resident_count",
+    "smx_resident_bytes", "smx_upload_q4_0", "smx_upload_q8_0", "smx_upload_q6_k",
+    "smx_upload_moe_q8", "smx_evict", "smx_gemv", "smx_gemv_rows", "smx_gemv_batch", "smx_gemm",
+    "smx_lm_head_argmax_rows", "smx_moe_ffn", "smx_moe_layer", "smx_dev_alloc", "smx_dev_free",
+    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev",
+    "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
+    "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
+    "smx_moe_ffn_stages",
+]
+
+
+class SmxError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__(f"smx error {code}: {msg}")
+        self.code = code
+
+
+_lib = None
+
+
+def load_library():
+    """Load the built library; fails loudly if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise FileNotFoundError(
+            f"{LIB_PATH} is missing: build it with `python strix.rs_amd/build.py` "
+            "(there is no CPU fallback)")
+    L = C.CDLL(LIB_PATH)
+    vp, sz, i, cp = C.c_void_p, C.c_size_t, C.c_int, C.c_char_p
+    L.smx_create.argtypes = [i, C.POINTER(vp)]
+    L.smx_destroy.argtypes = [vp]
+    L.smx_destroy.restype = None
+    L.smx_last_error.argtypes = [vp]
+    L.smx_last_error.restype = cp
+    L.smx_name.argtypes = [vp]
+    L.smx_name.restype = cp
+    L.smx_resident_count.argtypes = [vp]
+    L.smx_resident_count.restype = sz
+    L.smx_resident_bytes.argtypes = [vp]
+    L.smx_resident_bytes.restype = sz
+    for n in ("smx_upload_q4_0", "smx_upload_q8_0", "smx_upload_q6_k"):
+        getattr(L, n).argtypes = [vp, cp, vp, sz, sz, sz]
+    L.smx_upload_moe_q8.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz, sz, sz, sz]
+    L.smx_evict.argtypes = [vp, cp]
+    L.smx_gemv.argtypes = [vp, cp, vp, sz, vp, sz]
+    L.smx_gemv_rows.argtypes = [vp, cp, vp, sz, sz, vp, sz]
+    L.smx_gemv_batch.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp]
+    L.smx_gemm.argtypes = [vp, cp, vp, sz, sz, vp, sz]
+    L.smx_lm_head_argmax_rows.argtypes = [vp, cp, vp, sz, sz, vp]
+    L.smx_moe_ffn.argtypes = [vp, sz, vp, vp, sz, vp, sz, C.c_float, vp, sz]
+    L.smx_moe_layer.argtypes = [vp, sz, vp, sz, vp, sz, vp, vp, sz, vp, sz]
+    L.smx_dev_alloc.argtypes = [vp, sz, C.POINTER(vp)]
+    L.smx_dev_free.argtypes = [vp, vp]
+    L.smx_h2d.argtypes = [vp, vp, vp, sz]
+    L.smx_d2h.argtypes = [vp, vp, vp, sz]
+    L.smx_sync.argtypes = [vp]
+    L.smx_gemv_dev.argtypes = [vp, cp, vp, sz, vp]
+    L.smx_gemm_dev.argtypes = [vp, cp, vp, sz, vp]
+    L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
+    L.smx_prof_enable.argtypes = [vp, i]
+    L.smx_prof_reset.argtypes = [vp]
+    L.smx_prof_read.argtypes = [vp, cp, C.POINTER(C.c_double), C.POINTER(sz)]
+    L.smx_prof_names.argtypes = [vp]
+    L.smx_prof_names.restype = cp
+    L.smx_timer_begin.argtypes = [vp]
+    L.smx_timer_end.argtypes = [vp, C.POINTER(C.c_float)]
+    L.smx_quantize.argtypes = [vp, vp, sz, sz, vp, vp, vp]
+    L.smx_gemv_block_dots.argtypes = [vp, cp, vp, sz, vp, sz]
+    L.smx_gemm_block_dots.argtypes = [vp, cp, vp, sz, sz, vp, sz]
+    L.smx_moe_ffn_stages.argtypes = [vp, sz, vp, vp, sz, vp, sz, vp, vp, vp, vp]
+    _lib = L
+    return L
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _c(a, dt):
+    return np.ascontiguousarray(a, dtype=dt)
+
+
+class Mi355WeightAccel:
+    """One device, one stream, resident quantized weights (WeightAccel, accel.rs:147)."""
+
+    def __init__(self, device=0):
+        self._L = load_library()
+        h = C.c_void_p()
+        rc = self._L.smx_create(device, C.byref(h))
+        if rc != SMX_OK:
+            raise SmxError(rc, self._L.smx_last_error(None).decode())
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._L.smx_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    # -- helpers
+    def _check(self, rc):
+        """1 -> True, 0 -> False (not resident), <0 -> raise."""
+        if rc < 0:
+            raise SmxError(rc, self._L.smx_last_error(self._h).decode())
+        return rc == SMX_OK
+
+    def last_error(self):
+        return self._L.smx_last_error(self._h).decode()
+
+    # -- WeightAccel surface
+    def name(self):
+        return self._L.smx_name(self._h).decode()
+
+    def resident_count(self):
+        return int(self._L.smx_resident_count(self._h))
+
+    def resident_bytes(self):
+        return int(self._L.smx_resident_bytes(self._h))
+
+    def _upload(self, fn, key, raw, in_dim, out_dim):
+        raw = _c(raw, np.uint8)
+        return self._check(fn(self._h, key.encode(), _p(raw), raw.size, in_dim, out_dim))
+
+    def upload_q4_0(self, key, raw, in_dim, out_dim):
+        return self._upload(self._L.smx_upload_q4_0, key, raw, in_dim, out_dim)
+
+    def upload_q8_0(self, key, raw, in_dim, out_dim):
+        return self._upload(self._L.smx_upload_q8_0, key, raw, in_dim, out_dim)
+
+    def upload_q6_k(self, key, raw, in_dim, out_dim):
+        return self._upload(self._L.smx_upload_q6_k, key, raw, in_dim, out_dim)
+
+    def upload_moe_q8(self, layer, gate, up, down, hidden, eff, ne):
+        gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
+        return self._check(self._L.smx_upload_moe_q8(self._h, layer, _p(gate), gate.size, _p(up), up.size,
+                                                     _p(down), down.size, hidden, eff, ne))
+
+    def evict(self, key):
+        return self._check(self._L.smx_evict(self._h, key.encode()))
+
+    def gemv(self, key, x, out_dim):
+        x = _c(x, np.float32).reshape(-1)
+        y = np.empty(out_dim, np.float32)
+        ok = self._check(self._L.smx_gemv(self._h, key.encode(), _p(x), x.size, _p(y), y.size))
+        return y if ok else None
+
+    def gemv_rows(self, key, xs, out_dim):
+        xs = _c(xs, np.float32)
+        m, k = xs.shape
+        y = np.empty((m, out_dim), np.float32)
+        ok = self._check(self._L.smx_gemv_rows(self._h, key.encode(), _p(xs), m, k, _p(y), y.size))
+        return y if ok else None
+
+    def gemv_batch(self, calls, out_dims):
+        """calls: [(key, x)], out_dims: [out_dim]; returns [array | None] (accel.rs:397)."""
+        n = len(calls)
+        xs = [_c(x, np.float32).reshape(-1) for _, x in calls]
+        ys = [np.empty(d, np.float32) for d in out_dims]
+        keys = (C.c_char_p * n)(*[k.encode() for k, _ in calls])
+        xp = (C.c_void_p * n)(*[x.ctypes.data for x in xs])
+        yp = (C.c_void_p * n)(*[y.ctypes.data for y in ys])
+        il = (C.c_size_t * n)(*[x.size for x in xs])
+        oc = (C.c_size_t * n)(*[y.size for y in ys])
+        st = (C.c_int * n)()
+        self._check(self._L.smx_gemv_batch(self._h, n, keys, xp, il, yp, oc, st))
+        out = []
+        for i in range(n):
+            if st[i] < 0:
+                raise SmxError(st[i], self.last_error())
+            out.append(ys[i] if st[i] == SMX_OK else None)
+        return out
+
+    def prefill_q8_gemm(self, key, xs, m, out_dim):
+        """y[m][out_dim] token-major (accel.rs:213)."""
+        xs = _c(xs, np.float32).reshape(m, -1)
+        y = np.empty((m, out_dim), np.float32)
+        ok = self._check(self._L.smx_gemm(self._h, key.encode(), _p(xs), m, xs.shape[1], _p(y), y.size))
+        return y if ok else None
+
+    def lm_head_argmax_rows(self, key, xs, m):
+        xs = _c(xs, np.float32).reshape(m, -1)
+        out = np.empty(m, np.uint32)
+        ok = self._check(self._L.smx_lm_head_argmax_rows(self._h, key.encode(), _p(xs), m, xs.shape[1], _p(out)))
+        return out if ok else None
+
+    def moe_ffn(self, layer, ids, wexp, x, sgate=0.0):
+        ids, wexp, x = _c(ids, np.int32), _c(wexp, np.float32), _c(x, np.float32).reshape(-1)
+        y = np.empty(x.size, np.float32)
+        ok = self._check(self._L.smx_moe_ffn(self._h, layer, _p(ids), _p(wexp), ids.size, _p(x), x.size,
+                                             sgate, _p(y), y.size))
+        return y if ok else None
+
+    def moe_layer_q8_dev(self, layer, xs, m, plan, slot_tok, wslot):
+        xs = _c(xs, np.float32).reshape(m, -1)
+        plan = _c(plan, np.uint64).reshape(-1, 3)
+        slot_tok, wslot = _c(slot_tok, np.int32), _c(wslot, np.float32)
+        y = np.empty_like(xs)
+        ok = self._check(self._L.smx_moe_layer(self._h, layer, _p(xs), m, _p(plan), plan.shape[0],
+                                               _p(slot_tok), _p(wslot), slot_tok.size, _p(y), y.size))
+        return y if ok else None
+
+    # -- parity instrumentation
+    def quantize(self, x, k):
+        x = _c(x, np.float32).reshape(-1, k)
+        m = x.shape[0]
+        xq = np.empty((m, k), np.int8)
+        xd = np.empty((m, k // 32), np.float32)
+        xs = np.empty((m, k // 16), np.int16)
+        self._check(self._L.smx_quantize(self._h, _p(x), m, k, _p(xq), _p(xd), _p(xs)))
+        return xq, xd, xs
+
+    def gemv_block_dots(self, key, x, out_dim, per_row):
+        x = _c(x, np.float32).reshape(-1)
+        out = np.empty((out_dim, per_row), np.int32)
+        ok = self._check(self._L.smx_gemv_block_dots(self._h, key.encode(), _p(x), x.size, _p(out), out.size))
+        return out if ok else None
+
+    def gemm_block_dots(self, key, xs, m, out_dim, nb):
+        xs = _c(xs, np.float32).reshape(m, -1)
+        out = np.empty((m, out_dim, nb), np.int32)
+        ok = self._check(self._L.smx_gemm_block_dots(self._h, key.encode(), _p(xs), m, xs.shape[1], _p(out), out.size))
+        return out if ok else None
+
+    def moe_ffn_stages(self, layer, ids, wexp, x, eff):
+        ids, wexp, x = _c(ids, np.int32), _c(wexp, np.float32), _c(x, np.float32).reshape(-1)
+        k = ids.size
+        y = np.empty(x.size, np.float32)
+        gu = np.empty((k, 2, eff), np.float32)
+        aq = np.empty((k, eff), np.int8)
+        ad = np.empty((k, eff // 32), np.float32)
+        ok = self._check(self._L.smx_moe_ffn_stages(self._h, layer, _p(ids), _p(wexp), k, _p(x), x.size,
+                                                    _p(y), _p(gu), _p(aq), _p(ad)))
+        return (y, gu, aq, ad) if ok else None
+
+    # -- device-resident + timing (used by the benchmark)
+    def dev_alloc(self, nbytes):
+        d = C.c_void_p()
+        self._check(self._L.smx_dev_alloc(self._h, nbytes, C.byref(d)))
+        return d.value
+
+    def dev_free(self, dptr):
+        self._check(self._L.smx_dev_free(self._h, dptr))
+
+    def h2d(self, dptr, arr):
+        arr = np.ascontiguousarray(arr)
+        self._check(self._L.smx_h2d(self._h, dptr, _p(arr), arr.nbytes))
+
+    def d2h(self, arr, dptr):
+        self._check(self._L.smx_d2h(self._h, _p(arr), dptr, arr.nbytes))
+        return arr
+
+    def sync(self):
+        self._check(self._L.smx_sync(self._h))
+
+    def gemv_dev(self, key, xs_dev, m, y_dev):
+        return self._check(self._L.smx_gemv_dev(self._h, key.encode(), xs_dev, m, y_dev))
+
+    def gemm_dev(self, key, xs_dev, m, y_dev):
+        return self._check(self._L.smx_gemm_dev(self._h, key.encode(), xs_dev, m, y_dev))
+
+    def moe_ffn_dev(self, layer, ids, wexp, x_dev, y_dev):
+        ids, wexp = _c(ids, np.int32), _c(wexp, np.float32)
+        return self._check(self._L.smx_moe_ffn_dev(self._h, layer, _p(ids), _p(wexp), ids.size, x_dev, y_dev))
+
+    def prof_enable(self, on=True):
+        self._check(self._L.smx_prof_enable(self._h, 1 if on else 0))
+
+    def prof_reset(self):
+        self._check(self._L.smx_prof_reset(self._h))
+
+    def prof_read(self, prefix):
+        ms, n = C.c_double(), C.c_size_t()
+        self._check(self._L.smx_prof_read(self._h, prefix.encode(), C.byref(ms), C.byref(n)))
+        return ms.value, n.value
+
+    def prof_names(self):
+        s = self._L.smx_prof_names(self._h).decode()
+        return s.split(",") if s else []
+
+    def timer_begin(self):
+        self._check(self._L.smx_timer_begin(self._h))
+
+    def timer_end(self):
+        ms = C.c_float()
+        self._check(self._L.smx_timer_end(self._h, C.byref(ms)))
+        return ms.value

@@ -1,0 +1,57 @@
+// Activation quantiser: fp32 rows -> per-32-block Q8 (int8 quants + f32 scale + 16-element sums).
+//
+// Arithmetic of the reference's device quantisers (crates/strix-backend-rocm/src/kernels.rs:75-96,
+// 864-876, 1000-1013): d = amax/127, inv = d > 0 ? 1/d : 0, q = clamp(rint(x*inv), -127, 127).
+// Layout differs: quants stay contiguous int8 [m][K]; the block sum the reference keeps per 32
+// (kernels.rs:93) is kept as two 16-element sums packed in one dword, which also serves the
+// 16-wide sub-blocks of Q6_K.
+#include "smx_internal.h"
+
+namespace smx {
+
+// 8 lanes per 32-block, one float4 each: 128-bit loads, 32-bit packed stores.
+__global__ __launch_bounds__(256) void actquant_kernel(const float4* __restrict__ x, int* __restrict__ xq4,
+                                                       float* __restrict__ xd, int* __restrict__ xs,
+                                                       size_t nblocks) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t blk = gid >> 3;
+    const bool live = blk < nblocks;
+    float4 v = live ? x[gid] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    a = fmaxf(a, __shfl_xor(a, 1));
+    a = fmaxf(a, __shfl_xor(a, 2));
+    a = fmaxf(a, __shfl_xor(a, 4));
+    const float d = a / 127.f;
+    const float inv = d > 0.f ? 1.f / d : 0.f;
+    int q0 = max(-127, min(127, (int)rintf(v.x * inv)));
+    int q1 = max(-127, min(127, (int)rintf(v.y * inv)));
+    int q2 = max(-127, min(127, (int)rintf(v.z * inv)));
+    int q3 = max(-127, min(127, (int)rintf(v.w * inv)));
+    int s = q0 + q1 + q2 + q3;
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);                 // sum over this lane's 16-element half
+    const int other = __shfl_xor(s, 4);    // the other half's sum
+    if (live) {
+        xq4[gid] = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+        if ((gid & 7) == 0) {
+            xd[blk] = d;
+            xs[blk] = (s & 0xffff) | (other << 16);
+        }
+    }
+}
+
+int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, float* xd, int32_t* xs) {
+    if (K % 32 != 0) return fail(c, SMX_ERR_ARG, "quantise: row length %zu is not a multiple of 32", K);
+    const size_t nblocks = m * (K / 32);
+    if (nblocks == 0) return SMX_OK;
+    const size_t threads = nblocks * 8;
+    const size_t grid = (threads + 255) / 256;
+    if (grid > 0x7fffffffu) return fail(c, SMX_ERR_LIMIT, "quantise: %zu blocks exceed the grid limit", nblocks);
+    ProfScope ps(c, "actquant");
+    hipLaunchKernelGGL(actquant_kernel, dim3((unsigned)grid), dim3(256), 0, c->stream, (const float4*)x, (int*)xq,
+                       xd, (int*)xs, nblocks);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
+}  // namespace smx

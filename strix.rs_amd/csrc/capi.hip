@@ -1,0 +1,282 @@
+// extern "C" entry points of the matmul path: host-pointer calls (copy in, run, copy out, sync)
+// and device-pointer calls (enqueue only).
+#include <cstring>
+
+#include "smx_internal.h"
+
+using namespace smx;
+
+namespace {
+
+const Weight* find_weight(smx_ctx* c, const char* key) {
+    auto it = c->weights.find(key);
+    return it == c->weights.end() ? nullptr : &it->second;
+}
+
+// Scratch for m quantised rows of length K.
+int ensure_act(smx_ctx* c, size_t m, size_t K) {
+    int rc;
+    if ((rc = ensure(c, c->xq, m * K)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xd, m * (K / 32) * 4)) != SMX_OK) return rc;
+    return ensure(c, c->xs, m * (K / 32) * 4);
+}
+
+// argmax per row of y[m][N], lowest index on ties (strict '>' scan order of decode.rs:3677-3683).
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restrict__ y, size_t N,
+                                                          unsigned* __restrict__ out) {
+    const float* row = y + (size_t)blockIdx.x * N;
+    float best = -INFINITY;
+    size_t bi = 0;
+    bool have = false;
+    for (size_t i = threadIdx.x; i < N; i += 256) {  // ascending i: strict '>' keeps the lowest index
+        const float v = row[i];
+        if (!have || v > best) {
+            best = v;
+            bi = i;
+            have = true;
+        }
+    }
+    __shared__ float sb[256];
+    __shared__ size_t si[256];
+    __shared__ int sh[256];
+    sb[threadIdx.x] = best;
+    si[threadIdx.x] = bi;
+    sh[threadIdx.x] = have ? 1 : 0;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if ((int)threadIdx.x < s) {
+            const int o = threadIdx.x + s;
+            if (sh[o] && (!sh[threadIdx.x] || sb[o] > sb[threadIdx.x] ||
+                          (sb[o] == sb[threadIdx.x] && si[o] < si[threadIdx.x]))) {
+                sb[threadIdx.x] = sb[o];
+                si[threadIdx.x] = si[o];
+                sh[threadIdx.x] = 1;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = (unsigned)si[0];
+}
+
+// quantise m device rows and run the right matmul kernel into y_dev
+int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm,
+                   int32_t* dump) {
+    int rc = ensure_act(c, m, w.K);
+    if (rc != SMX_OK) return rc;
+    rc = launch_actquant(c, xs_dev, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+    if (rc != SMX_OK) return rc;
+    const bool gemv_ok = m <= SMX_GEMV_MAX_M && (w.type != kQ6_K || m == 1);
+    if (gemv_ok && !force_gemm)
+        return launch_gemv(c, w, (const int8_t*)c->xq.p, (const float*)c->xd.p, (const int32_t*)c->xs.p, m, y_dev,
+                           dump);
+    if (w.type == kQ6_K) return fail(c, SMX_ERR_LIMIT, "Q6_K weights are served by the GEMV path only (one row per call)");
+    return launch_gemm(c, w, (const int8_t*)c->xq.p, (const float*)c->xd.p, m, y_dev, dump);
+}
+
+int matmul_host(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, float* y, size_t y_cap,
+                bool force_gemm, const char* who) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !xs || !y) return fail(c, SMX_ERR_ARG, "%s: null argument", who);
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (in_dim != w->K) return fail(c, SMX_ERR_ARG, "%s: activation length %zu, weight in_dim %zu", who, in_dim, w->K);
+    if (m == 0) return fail(c, SMX_ERR_ARG, "%s: zero rows", who);
+    if (y_cap < m * w->N) return fail(c, SMX_ERR_ARG, "%s: output capacity %zu < %zu", who, y_cap, m * w->N);
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, m * w->K * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
+    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, force_gemm, nullptr);
+    if (rc != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, m * w->N * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int smx_gemv(smx_ctx* c, const char* key, const float* x, size_t in_len, float* y, size_t out_cap) {
+    return matmul_host(c, key, x, 1, in_len, y, out_cap, false, "gemv");
+}
+
+int smx_gemv_rows(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, float* y, size_t y_cap) {
+    if (c && m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv_rows: %zu rows (limit %d)", m, SMX_GEMV_MAX_M);
+    return matmul_host(c, key, xs, m, in_dim, y, y_cap, false, "gemv_rows");
+}
+
+int smx_gemm(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, float* y, size_t y_cap) {
+    return matmul_host(c, key, xs, m, in_dim, y, y_cap, true, "gemm");
+}
+
+int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs, const size_t* in_lens,
+                   float* const* ys, const size_t* out_caps, int* status) {
+    if (!c) return SMX_ERR_ARG;
+    if (!keys || !xs || !in_lens || !ys || !out_caps || !status) return fail(c, SMX_ERR_ARG, "gemv_batch: null argument");
+    SMX_HIP(c, hipSetDevice(c->device));
+    // Pass 1: validate and size one scratch region per item so the whole batch is one device job.
+    std::vector<const Weight*> ws(n, nullptr);
+    size_t xbytes = 0, ybytes = 0, qbytes = 0, dbytes = 0;
+    for (size_t i = 0; i < n; i++) {
+        status[i] = SMX_NOT_RESIDENT;
+        if (!keys[i] || !xs[i] || !ys[i]) {
+            status[i] = fail(c, SMX_ERR_ARG, "gemv_batch: item %zu has a null pointer", i);
+            continue;
+        }
+        const Weight* w = find_weight(c, keys[i]);
+        if (!w) continue;
+        if (in_lens[i] != w->K) {
+            status[i] = fail(c, SMX_ERR_ARG, "gemv_batch: item %zu activation length %zu, in_dim %zu", i, in_lens[i], w->K);
+            continue;
+        }
+        if (out_caps[i] < w->N) {
+            status[i] = fail(c, SMX_ERR_ARG, "gemv_batch: item %zu output capacity %zu < %zu", i, out_caps[i], w->N);
+            continue;
+        }
+        ws[i] = w;
+        xbytes += (w->K * 4 + 255) & ~size_t(255);
+        ybytes += (w->N * 4 + 255) & ~size_t(255);
+        qbytes += (w->K + 255) & ~size_t(255);
+        dbytes += ((w->K / 32) * 4 + 255) & ~size_t(255);
+    }
+    int rc;
+    if ((rc = ensure(c, c->xf32, xbytes)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, ybytes)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xq, qbytes)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xd, dbytes)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xs, dbytes)) != SMX_OK) return rc;
+    size_t xo = 0, yo = 0, qo = 0, dofs = 0;
+    std::vector<size_t> yoff(n, 0);
+    for (size_t i = 0; i < n; i++) {
+        const Weight* w = ws[i];
+        if (!w) continue;
+        float* xdv = (float*)(c->xf32.p + xo);
+        int8_t* q = (int8_t*)(c->xq.p + qo);
+        float* d = (float*)(c->xd.p + dofs);
+        int32_t* s = (int32_t*)(c->xs.p + dofs);
+        float* yd = (float*)(c->yf32.p + yo);
+        yoff[i] = yo;
+        SMX_HIP(c, hipMemcpyAsync(xdv, xs[i], w->K * 4, hipMemcpyHostToDevice, c->stream));
+        rc = launch_actquant(c, xdv, 1, w->K, q, d, s);
+        if (rc == SMX_OK) rc = launch_gemv(c, *w, q, d, s, 1, yd, nullptr);
+        status[i] = rc;
+        xo += (w->K * 4 + 255) & ~size_t(255);
+        yo += (w->N * 4 + 255) & ~size_t(255);
+        qo += (w->K + 255) & ~size_t(255);
+        dofs += ((w->K / 32) * 4 + 255) & ~size_t(255);
+    }
+    for (size_t i = 0; i < n; i++)
+        if (ws[i] && status[i] == SMX_OK)
+            SMX_HIP(c, hipMemcpyAsync(ys[i], c->yf32.p + yoff[i], ws[i]->N * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));  // the batch's single sync (decode.rs:3247)
+    return SMX_OK;
+}
+
+int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, uint32_t* out) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !xs || !out) return fail(c, SMX_ERR_ARG, "lm_head_argmax_rows: null argument");
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (in_dim != w->K) return fail(c, SMX_ERR_ARG, "lm_head_argmax_rows: activation length %zu, in_dim %zu", in_dim, w->K);
+    if (m == 0) return fail(c, SMX_ERR_ARG, "lm_head_argmax_rows: zero rows");
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, m * w->K * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->tab, m * 4)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
+    if (w->type == kQ6_K && m > 1) {
+        // Q6_K heads run one activation row per launch
+        rc = ensure_act(c, m, w->K);
+        if (rc != SMX_OK) return rc;
+        rc = launch_actquant(c, (const float*)c->xf32.p, m, w->K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+        for (size_t t = 0; t < m && rc == SMX_OK; t++)
+            rc = launch_gemv(c, *w, (const int8_t*)c->xq.p + t * w->K, (const float*)c->xd.p + t * (w->K / 32),
+                             (const int32_t*)c->xs.p + t * (w->K / 32), 1, (float*)c->yf32.p + t * w->N, nullptr);
+    } else {
+        rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr);
+    }
+    if (rc != SMX_OK) return rc;
+    {
+        ProfScope ps(c, "argmax_rows");
+        hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)m), dim3(256), 0, c->stream, (const float*)c->yf32.p,
+                           w->N, (unsigned*)c->tab.p);
+        SMX_HIP(c, hipGetLastError());
+    }
+    SMX_HIP(c, hipMemcpyAsync(out, c->tab.p, m * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+int smx_gemv_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, float* y_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !xs_dev || !y_dev) return fail(c, SMX_ERR_ARG, "gemv_dev: null argument");
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (m == 0 || m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv_dev: %zu rows (1..%d)", m, SMX_GEMV_MAX_M);
+    return run_matmul_dev(c, *w, xs_dev, m, y_dev, false, nullptr);
+}
+
+int smx_gemm_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, float* y_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !xs_dev || !y_dev) return fail(c, SMX_ERR_ARG, "gemm_dev: null argument");
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (m == 0) return fail(c, SMX_ERR_ARG, "gemm_dev: zero rows");
+    return run_matmul_dev(c, *w, xs_dev, m, y_dev, true, nullptr);
+}
+
+int smx_quantize(smx_ctx* c, const float* x, size_t m, size_t k, int8_t* xq, float* xd, int16_t* xs16) {
+    if (!c) return SMX_ERR_ARG;
+    if (!x || !xq || !xd) return fail(c, SMX_ERR_ARG, "quantize: null argument");
+    if (m == 0 || k == 0 || k % 32 != 0) return fail(c, SMX_ERR_ARG, "quantize: bad shape %zu x %zu", m, k);
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, m * k * 4)) != SMX_OK) return rc;
+    if ((rc = ensure_act(c, m, k)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, x, m * k * 4, hipMemcpyHostToDevice, c->stream));
+    rc = launch_actquant(c, (const float*)c->xf32.p, m, k, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+    if (rc != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(xq, c->xq.p, m * k, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(xd, c->xd.p, m * (k / 32) * 4, hipMemcpyDeviceToHost, c->stream));
+    // the packed dword (lo16 | hi16 << 16) is two consecutive little-endian i16: xs16[m][k/16]
+    if (xs16) SMX_HIP(c, hipMemcpyAsync(xs16, c->xs.p, m * (k / 32) * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+static int block_dots(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, int32_t* out,
+                      size_t out_cap, bool gemm, const char* who) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !xs || !out) return fail(c, SMX_ERR_ARG, "%s: null argument", who);
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (in_dim != w->K) return fail(c, SMX_ERR_ARG, "%s: activation length %zu, in_dim %zu", who, in_dim, w->K);
+    const size_t per = w->type == kQ6_K ? w->K / 16 : w->K / 32;
+    const size_t need = m * w->N * per;
+    if (out_cap < need) return fail(c, SMX_ERR_ARG, "%s: output capacity %zu < %zu", who, out_cap, need);
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, m * w->K * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->work, need * 4)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
+    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, gemm, (int32_t*)c->work.p);
+    if (rc != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(out, c->work.p, need * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+int smx_gemv_block_dots(smx_ctx* c, const char* key, const float* x, size_t in_len, int32_t* out, size_t out_cap) {
+    return block_dots(c, key, x, 1, in_len, out, out_cap, false, "gemv_block_dots");
+}
+
+int smx_gemm_block_dots(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, int32_t* out,
+                        size_t out_cap) {
+    return block_dots(c, key, xs, m, in_dim, out, out_cap, true, "gemm_block_dots");
+}
+
+}  // extern "C"

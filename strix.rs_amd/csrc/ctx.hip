@@ -1,0 +1,399 @@
+// Context, weight residency (upload + repack to planar HBM layout), scratch and profiling.
+#include <cstring>
+#include <memory>
+
+#include "smx_internal.h"
+
+namespace smx {
+
+static thread_local std::string g_create_err;
+
+int fail(smx_ctx* c, int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (c) c->err = buf; else g_create_err = buf;
+    return code;
+}
+
+int hip_fail(smx_ctx* c, hipError_t e, const char* what) {
+    (void)hipGetLastError();  // clear the sticky error so the next call reports its own
+    return fail(c, SMX_ERR_HIP, "HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+}
+
+int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
+    if (bytes <= b.cap) return SMX_OK;
+    if (b.p) {
+        SMX_HIP(c, hipStreamSynchronize(c->stream));
+        SMX_HIP(c, hipFree(b.p));
+        b.p = nullptr;
+        b.cap = 0;
+    }
+    size_t cap = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    hipError_t e = hipMalloc((void**)&b.p, cap);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        b.p = nullptr;
+        return fail(c, SMX_ERR_NOMEM, "device allocation of %zu bytes failed: %s", cap, hipGetErrorString(e));
+    }
+    b.cap = cap;
+    return SMX_OK;
+}
+
+ProfScope::ProfScope(smx_ctx* c_, const char* name) : c(c_) {
+    if (!c->prof_on) return;
+    hipEvent_t e0, e1;
+    if (!c->ev_pool.empty()) {
+        e0 = c->ev_pool.back().first;
+        e1 = c->ev_pool.back().second;
+        c->ev_pool.pop_back();
+    } else {
+        if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return;
+    }
+    c->prof.push_back(ProfRec{name, e0, e1});
+    idx = (int)c->prof.size() - 1;
+    (void)hipEventRecord(e0, c->stream);
+}
+
+ProfScope::~ProfScope() {
+    if (idx >= 0) (void)hipEventRecord(c->prof[idx].e1, c->stream);
+}
+
+static size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
+
+static void free_weight(Weight& w) {
+    if (w.base) (void)hipFree(w.base);
+    w.base = nullptr;
+}
+
+// Host-side repack of raw GGUF blocks into the planar layout (the reference
+// repacks on the host too: decode.rs:2500-2509, 2639-2664, 2693-2700), then one
+// copy to a fresh device allocation.
+static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nbytes, size_t K, size_t N,
+                        Weight* out) {
+    const size_t be = type == kQ6_K ? 256 : 32;
+    const size_t bb = type == kQ4_0 ? 18 : (type == kQ8_0 ? 34 : 210);
+    if (!bytes) return fail(c, SMX_ERR_ARG, "upload: null bytes");
+    if (K == 0 || N == 0 || K % be != 0)
+        return fail(c, SMX_ERR_ARG, "upload: in_dim %zu is not a positive multiple of %zu", K, be);
+    const size_t nblk = K / be, total = nblk * N;
+    if (nbytes != total * bb)
+        return fail(c, SMX_ERR_ARG, "upload: got %zu bytes, [%zu x %zu] needs %zu", nbytes, N, K, total * bb);
+    Weight w;
+    w.type = type;
+    w.K = K;
+    w.N = N;
+    w.nblk = nblk;
+    size_t off_scales = 0, off_quants = 0, off_qh = 0, off_sc = 0;
+    if (type == kQ4_0) {
+        off_quants = align256(total * 2);
+        w.bytes = off_quants + total * 16;
+    } else if (type == kQ8_0) {
+        off_quants = align256(total * 2);
+        w.bytes = off_quants + total * 32;
+    } else {
+        off_quants = 0;  // ql
+        off_qh = align256(total * 128);
+        off_sc = off_qh + align256(total * 64);
+        off_scales = off_sc + align256(total * 16);
+        w.bytes = off_scales + total * 2;
+    }
+    std::unique_ptr<uint8_t[]> host(new (std::nothrow) uint8_t[w.bytes]);
+    if (!host) return fail(c, SMX_ERR_NOMEM, "upload: host staging of %zu bytes failed", w.bytes);
+    uint8_t* h = host.get();
+    if (type == kQ4_0 || type == kQ8_0) {
+        const size_t qb = bb - 2;
+        for (size_t b = 0; b < total; b++) {
+            const uint8_t* blk = bytes + b * bb;
+            h[off_scales + b * 2] = blk[0];
+            h[off_scales + b * 2 + 1] = blk[1];
+            memcpy(h + off_quants + b * qb, blk + 2, qb);
+        }
+        if (off_quants > total * 2) memset(h + total * 2, 0, off_quants - total * 2);
+    } else {
+        memset(h, 0, w.bytes);
+        for (size_t b = 0; b < total; b++) {
+            const uint8_t* blk = bytes + b * 210;
+            memcpy(h + off_quants + b * 128, blk, 128);
+            memcpy(h + off_qh + b * 64, blk + 128, 64);
+            memcpy(h + off_sc + b * 16, blk + 192, 16);
+            h[off_scales + b * 2] = blk[208];
+            h[off_scales + b * 2 + 1] = blk[209];
+        }
+    }
+    hipError_t e = hipMalloc((void**)&w.base, w.bytes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(c, SMX_ERR_NOMEM, "upload: device allocation of %zu bytes failed: %s", w.bytes,
+                    hipGetErrorString(e));
+    }
+    e = hipMemcpy(w.base, h, w.bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(w.base);
+        return hip_fail(c, e, "hipMemcpy(weight)");
+    }
+    w.scales = (const uint16_t*)(w.base + off_scales);
+    w.quants = w.base + off_quants;
+    w.qh = type == kQ6_K ? w.base + off_qh : nullptr;
+    w.sc = type == kQ6_K ? (const int8_t*)(w.base + off_sc) : nullptr;
+    *out = w;
+    return SMX_OK;
+}
+
+static int upload(smx_ctx* c, QType type, const char* key, const void* bytes, size_t nbytes, size_t K,
+                  size_t N) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key) return fail(c, SMX_ERR_ARG, "upload: null key");
+    SMX_HIP(c, hipSetDevice(c->device));
+    Weight w;
+    int rc = build_weight(c, type, (const uint8_t*)bytes, nbytes, K, N, &w);
+    if (rc != SMX_OK) return rc;
+    auto it = c->weights.find(key);
+    if (it != c->weights.end()) {
+        (void)hipStreamSynchronize(c->stream);
+        free_weight(it->second);
+        it->second = w;
+    } else {
+        c->weights.emplace(key, w);
+    }
+    return SMX_OK;
+}
+
+}  // namespace smx
+
+using namespace smx;
+
+extern "C" {
+
+int smx_create(int device, smx_ctx** out) {
+    if (!out) return fail(nullptr, SMX_ERR_ARG, "smx_create: null out pointer");
+    *out = nullptr;
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev <= 0) {
+        (void)hipGetLastError();
+        return fail(nullptr, SMX_ERR_HIP, "smx_create: no HIP device (%s)", hipGetErrorString(e));
+    }
+    if (device < 0 || device >= ndev) return fail(nullptr, SMX_ERR_ARG, "smx_create: device %d of %d", device, ndev);
+    e = hipSetDevice(device);
+    if (e != hipSuccess) return hip_fail(nullptr, e, "hipSetDevice");
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, device);
+    if (e != hipSuccess) return hip_fail(nullptr, e, "hipGetDeviceProperties");
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(nullptr, SMX_ERR_ARG, "smx_create: device %d is %s; this library is built for gfx950 only",
+                    device, prop.gcnArchName);
+    smx_ctx* c = new (std::nothrow) smx_ctx();
+    if (!c) return fail(nullptr, SMX_ERR_NOMEM, "smx_create: out of host memory");
+    c->device = device;
+    c->num_cu = prop.multiProcessorCount;
+    c->name = std::string(prop.name) + " (" + prop.gcnArchName + ", strix-mi355)";
+    e = hipStreamCreate(&c->stream);  // default priority
+    if (e != hipSuccess) {
+        delete c;
+        return hip_fail(nullptr, e, "hipStreamCreate");
+    }
+    if (hipEventCreate(&c->t0) != hipSuccess || hipEventCreate(&c->t1) != hipSuccess) {
+        (void)hipStreamDestroy(c->stream);
+        delete c;
+        return fail(nullptr, SMX_ERR_HIP, "smx_create: hipEventCreate failed");
+    }
+    *out = c;
+    return SMX_OK;
+}
+
+void smx_destroy(smx_ctx* c) {
+    if (!c) return;
+    (void)hipSetDevice(c->device);
+    (void)hipStreamSynchronize(c->stream);
+    for (auto& kv : c->weights) free_weight(kv.second);
+    for (auto& kv : c->moe) {
+        free_weight(kv.second.gate);
+        free_weight(kv.second.up);
+        free_weight(kv.second.down);
+    }
+    for (DevBuf* b : {&c->xf32, &c->xq, &c->xd, &c->xs, &c->yf32, &c->work, &c->work2, &c->tab})
+        if (b->p) (void)hipFree(b->p);
+    for (auto& r : c->prof) {
+        (void)hipEventDestroy(r.e0);
+        (void)hipEventDestroy(r.e1);
+    }
+    for (auto& p : c->ev_pool) {
+        (void)hipEventDestroy(p.first);
+        (void)hipEventDestroy(p.second);
+    }
+    (void)hipEventDestroy(c->t0);
+    (void)hipEventDestroy(c->t1);
+    (void)hipStreamDestroy(c->stream);
+    delete c;
+}
+
+const char* smx_last_error(const smx_ctx* c) { return c ? c->err.c_str() : g_create_err.c_str(); }
+const char* smx_name(const smx_ctx* c) { return c ? c->name.c_str() : ""; }
+size_t smx_resident_count(const smx_ctx* c) { return c ? c->weights.size() + c->moe.size() : 0; }
+
+size_t smx_resident_bytes(const smx_ctx* c) {
+    if (!c) return 0;
+    size_t n = 0;
+    for (auto& kv : c->weights) n += kv.second.bytes;
+    for (auto& kv : c->moe) n += kv.second.gate.bytes + kv.second.up.bytes + kv.second.down.bytes;
+    return n;
+}
+
+int smx_upload_q4_0(smx_ctx* c, const char* key, const void* bytes, size_t nbytes, size_t in_dim, size_t out_dim) {
+    return upload(c, kQ4_0, key, bytes, nbytes, in_dim, out_dim);
+}
+int smx_upload_q8_0(smx_ctx* c, const char* key, const void* bytes, size_t nbytes, size_t in_dim, size_t out_dim) {
+    return upload(c, kQ8_0, key, bytes, nbytes, in_dim, out_dim);
+}
+int smx_upload_q6_k(smx_ctx* c, const char* key, const void* bytes, size_t nbytes, size_t in_dim, size_t out_dim) {
+    return upload(c, kQ6_K, key, bytes, nbytes, in_dim, out_dim);
+}
+
+int smx_upload_moe_q8(smx_ctx* c, size_t layer, const void* gate, size_t gate_n, const void* up, size_t up_n,
+                      const void* down, size_t down_n, size_t hidden, size_t eff, size_t ne) {
+    if (!c) return SMX_ERR_ARG;
+    if (!gate || !up || !down) return fail(c, SMX_ERR_ARG, "upload_moe_q8: null tensor");
+    if (hidden == 0 || eff == 0 || ne == 0 || hidden % 32 != 0 || eff % 32 != 0)
+        return fail(c, SMX_ERR_ARG, "upload_moe_q8: hidden %zu / eff %zu must be positive multiples of 32", hidden, eff);
+    const size_t gate_eb = (hidden / 32) * 34 * eff, down_eb = (eff / 32) * 34 * hidden;  // decode.rs:2730-2731
+    if (gate_n != gate_eb * ne || up_n != gate_eb * ne || down_n != down_eb * ne)
+        return fail(c, SMX_ERR_ARG, "upload_moe_q8: byte lengths (%zu, %zu, %zu) do not match %zu experts of %zu/%zu",
+                    gate_n, up_n, down_n, ne, gate_eb, down_eb);
+    SMX_HIP(c, hipSetDevice(c->device));
+    MoeLayer L;
+    L.hidden = hidden;
+    L.eff = eff;
+    L.ne = ne;
+    int rc = build_weight(c, kQ8_0, (const uint8_t*)gate, gate_n, hidden, ne * eff, &L.gate);
+    if (rc != SMX_OK) return rc;
+    rc = build_weight(c, kQ8_0, (const uint8_t*)up, up_n, hidden, ne * eff, &L.up);
+    if (rc != SMX_OK) {
+        free_weight(L.gate);
+        return rc;
+    }
+    rc = build_weight(c, kQ8_0, (const uint8_t*)down, down_n, eff, ne * hidden, &L.down);
+    if (rc != SMX_OK) {
+        free_weight(L.gate);
+        free_weight(L.up);
+        return rc;
+    }
+    auto it = c->moe.find(layer);
+    if (it != c->moe.end()) {
+        (void)hipStreamSynchronize(c->stream);
+        free_weight(it->second.gate);
+        free_weight(it->second.up);
+        free_weight(it->second.down);
+        it->second = L;
+    } else {
+        c->moe.emplace(layer, L);
+    }
+    return SMX_OK;
+}
+
+int smx_evict(smx_ctx* c, const char* key) {
+    if (!c || !key) return SMX_ERR_ARG;
+    auto it = c->weights.find(key);
+    if (it == c->weights.end()) return SMX_NOT_RESIDENT;
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    free_weight(it->second);
+    c->weights.erase(it);
+    return SMX_OK;
+}
+
+int smx_dev_alloc(smx_ctx* c, size_t nbytes, void** dptr) {
+    if (!c || !dptr) return SMX_ERR_ARG;
+    SMX_HIP(c, hipSetDevice(c->device));
+    hipError_t e = hipMalloc(dptr, nbytes ? nbytes : 1);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(c, SMX_ERR_NOMEM, "smx_dev_alloc: %zu bytes: %s", nbytes, hipGetErrorString(e));
+    }
+    return SMX_OK;
+}
+
+int smx_dev_free(smx_ctx* c, void* dptr) {
+    if (!c) return SMX_ERR_ARG;
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    SMX_HIP(c, hipFree(dptr));
+    return SMX_OK;
+}
+
+int smx_h2d(smx_ctx* c, void* dst, const void* src, size_t n) {
+    if (!c || !dst || !src) return SMX_ERR_ARG;
+    SMX_HIP(c, hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+int smx_d2h(smx_ctx* c, void* dst, const void* src, size_t n) {
+    if (!c || !dst || !src) return SMX_ERR_ARG;
+    SMX_HIP(c, hipMemcpyAsync(dst, src, n, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+int smx_sync(smx_ctx* c) {
+    if (!c) return SMX_ERR_ARG;
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+int smx_prof_enable(smx_ctx* c, int on) {
+    if (!c) return SMX_ERR_ARG;
+    c->prof_on = on != 0;
+    return SMX_OK;
+}
+
+int smx_prof_reset(smx_ctx* c) {
+    if (!c) return SMX_ERR_ARG;
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    for (auto& r : c->prof) c->ev_pool.emplace_back(r.e0, r.e1);
+    c->prof.clear();
+    return SMX_OK;
+}
+
+int smx_prof_read(smx_ctx* c, const char* prefix, double* total_ms, size_t* launches) {
+    if (!c || !prefix || !total_ms || !launches) return SMX_ERR_ARG;
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    double tot = 0;
+    size_t n = 0;
+    const size_t pl = strlen(prefix);
+    for (auto& r : c->prof) {
+        if (r.name.compare(0, pl, prefix) != 0) continue;
+        float ms = 0;
+        SMX_HIP(c, hipEventElapsedTime(&ms, r.e0, r.e1));
+        tot += ms;
+        n++;
+    }
+    *total_ms = tot;
+    *launches = n;
+    return SMX_OK;
+}
+
+const char* smx_prof_names(smx_ctx* c) {
+    if (!c) return "";
+    c->prof_names.clear();
+    for (auto& r : c->prof)
+        if (("," + c->prof_names + ",").find("," + r.name + ",") == std::string::npos)
+            c->prof_names += (c->prof_names.empty() ? "" : ",") + r.name;
+    return c->prof_names.c_str();
+}
+
+int smx_timer_begin(smx_ctx* c) {
+    if (!c) return SMX_ERR_ARG;
+    SMX_HIP(c, hipEventRecord(c->t0, c->stream));
+    return SMX_OK;
+}
+
+int smx_timer_end(smx_ctx* c, float* ms) {
+    if (!c || !ms) return SMX_ERR_ARG;
+    SMX_HIP(c, hipEventRecord(c->t1, c->stream));
+    SMX_HIP(c, hipEventSynchronize(c->t1));
+    SMX_HIP(c, hipEventElapsedTime(ms, c->t0, c->t1));
+    return SMX_OK;
+}
+
+}  // extern "C"

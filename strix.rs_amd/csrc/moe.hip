@@ -1,0 +1,416 @@
+// Mixture-of-experts FFN on resident Q8_0 experts: decode (one token, k routed experts, grouped
+// GEMVs) and prefill (m tokens grouped by expert, one table-driven MFMA GEMM launch per stage).
+//
+// Stands in for crates/strix-backend-rocm/src/decode.rs:1923-2128 (moe_launches: q8i_moe_gu ->
+// silu_quant -> q8i_moe_down -> moe_wsum, kernels.rs:942-996, 879-892, 1875-1882) and
+// decode.rs:1608-1739 (moe_layer_dev_inner: xquant8_rows -> gather_xq8 -> per-expert GEMMs ->
+// silu_quant_rows -> per-expert GEMMs -> scatter_add_w, kernels.rs:1162-1198).
+// Differences by design: the gather is an index indirection inside the GEMM's loader, all experts
+// of a stage share one launch (tile table) instead of one launch per expert, and the weighted
+// combine walks each token's slots in ascending slot order instead of fp32 atomics, so results do
+// not depend on scheduling.
+#include <algorithm>
+
+#include "gemv_body.h"
+#include "smx_internal.h"
+
+namespace smx {
+
+// exp() as a fixed sequence of IEEE fp32 operations (no contraction), so that the quantised
+// silu(g)*u is reproducible bit for bit on any conforming implementation.
+__device__ __forceinline__ float det_expf(float x) {
+#pragma clang fp contract(off)
+    x = x > 88.0f ? 88.0f : x;
+    x = x < -87.0f ? -87.0f : x;
+    const float n = rintf(x * 1.44269504088896341f);
+    float r = x - n * 0.693359375f;
+    r = r - n * -2.12194440e-4f;
+    float p = 1.9875691500e-4f;
+    p = p * r + 1.3981999507e-3f;
+    p = p * r + 8.3334519073e-3f;
+    p = p * r + 4.1665795894e-2f;
+    p = p * r + 1.6666665459e-1f;
+    p = p * r + 5.0000001201e-1f;
+    const float r2 = r * r;
+    p = p * r2;
+    p = p + r;
+    p = p + 1.0f;
+    return ldexpf(p, (int)n);
+}
+
+// silu(x) = x / (1 + exp(-x)), crates/strix-backend-cpu/src/ops.rs:73-76
+__device__ __forceinline__ float det_silu(float x) {
+#pragma clang fp contract(off)
+    return x / (1.0f + det_expf(-x));
+}
+
+// a = silu(g)*u, then the activation quantiser (kernels.rs:879-892, 1174-1187).  g and u are rows
+// of `eff` floats at strides ldg; 8 lanes per 32-block.
+__global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                             size_t ldg, int eff, int* __restrict__ xq4,
+                                                             float* __restrict__ xd, size_t nblocks) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t blk = gid >> 3;
+    const bool live = blk < nblocks;
+    float4 gv = make_float4(0.f, 0.f, 0.f, 0.f), uv = gv;
+    if (live) {
+        const int bpr = eff / 32;
+        const size_t row = blk / bpr, e0 = (blk % bpr) * 32 + (gid & 7) * 4;
+        gv = *(const float4*)(g + row * ldg + e0);
+        uv = *(const float4*)(u + row * ldg + e0);
+    }
+    float4 v;
+    {
+#pragma clang fp contract(off)
+        v.x = det_silu(gv.x) * uv.x;
+        v.y = det_silu(gv.y) * uv.y;
+        v.z = det_silu(gv.z) * uv.z;
+        v.w = det_silu(gv.w) * uv.w;
+    }
+    float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    a = fmaxf(a, __shfl_xor(a, 1));
+    a = fmaxf(a, __shfl_xor(a, 2));
+    a = fmaxf(a, __shfl_xor(a, 4));
+    const float d = a / 127.f;
+    const float inv = d > 0.f ? 1.f / d : 0.f;
+    const int q0 = max(-127, min(127, (int)rintf(v.x * inv)));
+    const int q1 = max(-127, min(127, (int)rintf(v.y * inv)));
+    const int q2 = max(-127, min(127, (int)rintf(v.z * inv)));
+    const int q3 = max(-127, min(127, (int)rintf(v.w * inv)));
+    if (live) {
+        xq4[gid] = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+        if ((gid & 7) == 0) xd[blk] = d;
+    }
+}
+
+// Decode GEMV over the routed experts of stacked planar Q8_0 tensors.
+//   grid = (row groups, k, ntens);  tensor z in {0,1} (gate, up) or {0} (down).
+//   expert e's rows are rows [e*rows, (e+1)*rows) of the stacked tensor.
+//   x: shared by all experts (per_k_x = 0) or one quantised row per routed expert (1).
+// Routed expert ids and weights travel as kernel arguments (no table upload on the decode path).
+struct MoeRoute {
+    int ids[64];
+    float w[64];
+};
+
+template <int RPW>
+__global__ __launch_bounds__(1024) void moe_gemv_q8_kernel(const uint16_t* __restrict__ s0,
+                                                           const uint4* __restrict__ q0,
+                                                           const uint16_t* __restrict__ s1,
+                                                           const uint4* __restrict__ q1,
+                                                           const MoeRoute route, const int8_t* __restrict__ xq,
+                                                           const float* __restrict__ xd, float* __restrict__ y0,
+                                                           float* __restrict__ y1, int nb, int rows, int per_k_x) {
+    const int kk = blockIdx.y;
+    const size_t ebase = (size_t)route.ids[kk] * rows * nb;  // in blocks
+    const uint16_t* sc = (blockIdx.z ? s1 : s0) + ebase;
+    const uint4* qu = (blockIdx.z ? q1 : q0) + ebase * 2;
+    float* y = (blockIdx.z ? y1 : y0) + (size_t)kk * rows;
+    const int8_t* xqk = per_k_x ? xq + (size_t)kk * nb * 32 : xq;
+    const float* xdk = per_k_x ? xd + (size_t)kk * nb : xd;
+    const int row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW;
+    gemv_q8_0_body<1, RPW, false>(sc, qu, xqk, xdk, y, nb, rows, 1, nullptr, row0);
+}
+
+// out[o] = sum_k wexp[k]*dy[k][o], k ascending (kernels.rs:1875-1882)
+__global__ __launch_bounds__(256) void moe_wsum_kernel(const float* __restrict__ dy, const MoeRoute route,
+                                                       float* __restrict__ out, int n, int k) {
+    const int o = blockIdx.x * 256 + threadIdx.x;
+    if (o >= n) return;
+    float s = 0.f;
+    for (int e = 0; e < k; e++) s += route.w[e] * dy[(size_t)e * n + o];
+    out[o] = s;
+}
+
+// y[t][i] = sum over the token's slots (ascending slot index) of wslot[s]*dy[s][i]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ dy, const int* __restrict__ tok_ptr,
+                                                          const int* __restrict__ tok_slots,
+                                                          const float* __restrict__ wslot, float* __restrict__ y,
+                                                          int hidden) {
+    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= hidden) return;
+    float s = 0.f;
+    for (int j = tok_ptr[t]; j < tok_ptr[t + 1]; j++) {
+        const int sl = tok_slots[j];
+        s += wslot[sl] * dy[(size_t)sl * hidden + i];
+    }
+    y[(size_t)t * hidden + i] = s;
+}
+
+static int moe_gemv(smx_ctx* c, const Weight& a, const Weight* b, const MoeRoute& route, int k, const int8_t* xq,
+                    const float* xd, float* y0, float* y1, int rows, int per_k_x, const char* name) {
+    const int nb = (int)a.nblk;
+    const size_t lds = ((size_t)nb * 36 + 15) & ~size_t(15);
+    if (lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "moe: activation of %d blocks does not fit LDS", nb);
+    const int nw = 4, rpw = 2;
+    const unsigned gx = (unsigned)((rows + nw * rpw - 1) / (nw * rpw));
+    ProfScope ps(c, name);
+    auto kern = moe_gemv_q8_kernel<2>;
+    if (lds > 48 * 1024)
+        SMX_HIP(c, hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(gx, (unsigned)k, b ? 2u : 1u), dim3(nw * 64), lds, c->stream, a.scales,
+                       (const uint4*)a.quants, b ? b->scales : a.scales, (const uint4*)(b ? b->quants : a.quants), route,
+                       xq, xd, y0, y1, nb, rows, per_k_x);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
+static int silu_mul_quant(smx_ctx* c, const float* g, const float* u, size_t ldg, size_t rows, size_t eff, int8_t* xq,
+                          float* xd) {
+    const size_t nblocks = rows * (eff / 32);
+    ProfScope ps(c, "silu_mul_quant");
+    hipLaunchKernelGGL(silu_mul_quant_kernel, dim3((unsigned)((nblocks * 8 + 255) / 256)), dim3(256), 0, c->stream, g, u,
+                       ldg, (int)eff, (int*)xq, xd, nblocks);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
+// Scratch carve-up helper: 256-byte aligned bump allocation inside one DevBuf.
+struct Carver {
+    size_t off = 0;
+    size_t take(size_t bytes) {
+        const size_t o = off;
+        off += (bytes + 255) & ~size_t(255);
+        return o;
+    }
+};
+
+// One token through k routed experts; x_dev fp32 [hidden] on the device, y_dev fp32 [hidden].
+// Intermediates live in c->work: g[k][eff], u[k][eff], aq[k][eff], ad[k][eff/32], dy[k][hidden].
+struct MoeScratch {
+    float *g, *u, *dy;
+    int8_t* aq;
+    float* ad;
+};
+
+static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, const float* wexp, size_t k,
+                           const float* x_dev, float* y_dev, MoeScratch* out_scratch) {
+    if (k == 0 || k > 64) return fail(c, SMX_ERR_LIMIT, "moe_ffn: %zu routed experts (1..64 supported)", k);
+    for (size_t i = 0; i < k; i++)
+        if (ids[i] < 0 || (size_t)ids[i] >= L.ne)
+            return fail(c, SMX_ERR_ARG, "moe_ffn: expert id %d outside 0..%zu", ids[i], L.ne - 1);
+    const size_t hidden = L.hidden, eff = L.eff;
+    int rc;
+    if ((rc = ensure(c, c->xq, hidden)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xd, (hidden / 32) * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xs, (hidden / 32) * 4)) != SMX_OK) return rc;
+    Carver cv;
+    const size_t o_g = cv.take(k * eff * 4), o_u = cv.take(k * eff * 4), o_aq = cv.take(k * eff),
+                 o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(k * hidden * 4);
+    if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
+    MoeRoute route = {};
+    for (size_t i = 0; i < k; i++) {
+        route.ids[i] = ids[i];
+        route.w[i] = wexp[i];
+    }
+    MoeScratch s;
+    s.g = (float*)(c->work.p + o_g);
+    s.u = (float*)(c->work.p + o_u);
+    s.aq = (int8_t*)(c->work.p + o_aq);
+    s.ad = (float*)(c->work.p + o_ad);
+    s.dy = (float*)(c->work.p + o_dy);
+    rc = launch_actquant(c, x_dev, 1, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+    if (rc != SMX_OK) return rc;
+    rc = moe_gemv(c, L.gate, &L.up, route, (int)k, (const int8_t*)c->xq.p, (const float*)c->xd.p, s.g, s.u, (int)eff, 0,
+                  "moe_gemv_gate_up");
+    if (rc != SMX_OK) return rc;
+    rc = silu_mul_quant(c, s.g, s.u, eff, k, eff, s.aq, s.ad);
+    if (rc != SMX_OK) return rc;
+    rc = moe_gemv(c, L.down, nullptr, route, (int)k, s.aq, s.ad, s.dy, s.dy, (int)hidden, 1, "moe_gemv_down");
+    if (rc != SMX_OK) return rc;
+    {
+        ProfScope ps(c, "moe_wsum");
+        hipLaunchKernelGGL(moe_wsum_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, c->stream, s.dy, route,
+                           y_dev, (int)hidden, (int)k);
+        SMX_HIP(c, hipGetLastError());
+    }
+    if (out_scratch) *out_scratch = s;
+    return SMX_OK;
+}
+
+static int moe_ffn_host(smx_ctx* c, size_t layer, const int32_t* ids, const float* wexp, size_t k, const float* x,
+                        size_t x_len, float sgate, float* y, size_t y_cap, float* gu, int8_t* aq, float* ad) {
+    if (!c) return SMX_ERR_ARG;
+    if (!ids || !wexp || !x || !y) return fail(c, SMX_ERR_ARG, "moe_ffn: null argument");
+    auto it = c->moe.find(layer);
+    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+    const MoeLayer& L = it->second;
+    if (x_len != L.hidden) return fail(c, SMX_ERR_ARG, "moe_ffn: activation length %zu, hidden %zu", x_len, L.hidden);
+    if (y_cap < L.hidden) return fail(c, SMX_ERR_ARG, "moe_ffn: output capacity %zu < %zu", y_cap, L.hidden);
+    if (sgate != 0.0f)
+        return fail(c, SMX_ERR_ARG, "moe_ffn: shared-expert gate %g: the shared expert is outside this path", (double)sgate);
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, L.hidden * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, L.hidden * 4)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, x, L.hidden * 4, hipMemcpyHostToDevice, c->stream));
+    MoeScratch s;
+    rc = moe_ffn_enqueue(c, L, ids, wexp, k, (const float*)c->xf32.p, (float*)c->yf32.p, &s);
+    if (rc != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, L.hidden * 4, hipMemcpyDeviceToHost, c->stream));
+    if (gu) {
+        for (size_t kk = 0; kk < k; kk++) {
+            SMX_HIP(c, hipMemcpyAsync(gu + (kk * 2) * L.eff, s.g + kk * L.eff, L.eff * 4, hipMemcpyDeviceToHost, c->stream));
+            SMX_HIP(c, hipMemcpyAsync(gu + (kk * 2 + 1) * L.eff, s.u + kk * L.eff, L.eff * 4, hipMemcpyDeviceToHost, c->stream));
+        }
+    }
+    if (aq) SMX_HIP(c, hipMemcpyAsync(aq, s.aq, k * L.eff, hipMemcpyDeviceToHost, c->stream));
+    if (ad) SMX_HIP(c, hipMemcpyAsync(ad, s.ad, k * (L.eff / 32) * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+// Tile table of one grouped GEMM stage: for every plan entry, ceil(cnt/128) x ceil(rows/128) tiles.
+static void build_tiles(const size_t* plan, size_t nplan, size_t rows_per_expert, std::vector<GemmTile>* tiles) {
+    tiles->clear();
+    for (size_t i = 0; i < nplan; i++) {
+        const int e = (int)plan[i * 3], off = (int)plan[i * 3 + 1], cnt = (int)plan[i * 3 + 2];
+        for (int tn = 0; tn * 128 < (int)rows_per_expert; tn++)      // tiles of one weight strip are adjacent
+            for (int tm = 0; tm * 128 < cnt; tm++) {
+                GemmTile t;
+                t.tok0 = off + tm * 128;
+                t.tok_end = off + cnt;
+                t.row0 = e * (int)rows_per_expert + tn * 128;
+                t.row_end = (e + 1) * (int)rows_per_expert;
+                t.col0 = tn * 128;
+                tiles->push_back(t);
+            }
+    }
+}
+
+}  // namespace smx
+
+using namespace smx;
+
+extern "C" {
+
+int smx_moe_ffn(smx_ctx* c, size_t layer, const int32_t* ids, const float* wexp, size_t k, const float* x, size_t x_len,
+                float sgate, float* y, size_t y_cap) {
+    return moe_ffn_host(c, layer, ids, wexp, k, x, x_len, sgate, y, y_cap, nullptr, nullptr, nullptr);
+}
+
+int smx_moe_ffn_stages(smx_ctx* c, size_t layer, const int32_t* ids, const float* wexp, size_t k, const float* x,
+                       size_t x_len, float* y, float* gu, int8_t* aq, float* ad) {
+    return moe_ffn_host(c, layer, ids, wexp, k, x, x_len, 0.0f, y, x_len, gu, aq, ad);
+}
+
+int smx_moe_ffn_dev(smx_ctx* c, size_t layer, const int32_t* ids, const float* wexp, size_t k, const float* x_dev,
+                    float* y_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!ids || !wexp || !x_dev || !y_dev) return fail(c, SMX_ERR_ARG, "moe_ffn_dev: null argument");
+    auto it = c->moe.find(layer);
+    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+    return moe_ffn_enqueue(c, it->second, ids, wexp, k, x_dev, y_dev, nullptr);
+}
+
+int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
+                  const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap) {
+    if (!c) return SMX_ERR_ARG;
+    if (!xs || !plan || !slot_tok || !wslot || !y) return fail(c, SMX_ERR_ARG, "moe_layer: null argument");
+    auto it = c->moe.find(layer);
+    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+    const MoeLayer& L = it->second;
+    const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
+    if (m == 0 || slots == 0) return fail(c, SMX_ERR_ARG, "moe_layer: m %zu, slots %zu", m, slots);  // decode.rs:1622
+    if (y_cap < m * hidden) return fail(c, SMX_ERR_ARG, "moe_layer: output capacity %zu < %zu", y_cap, m * hidden);
+    if (slots > (size_t(1) << 24) || m > 65535) return fail(c, SMX_ERR_LIMIT, "moe_layer: m %zu / slots %zu exceed the launch limits", m, slots);
+    // the plan must tile [0, slots) with in-range experts; every slot's token must exist
+    size_t covered = 0;
+    for (size_t i = 0; i < nplan; i++) {
+        const size_t e = plan[i * 3], off = plan[i * 3 + 1], cnt = plan[i * 3 + 2];
+        if (e >= L.ne || cnt == 0 || off != covered || off + cnt > slots)
+            return fail(c, SMX_ERR_ARG, "moe_layer: plan entry %zu (expert %zu, off %zu, count %zu) is inconsistent", i, e, off, cnt);
+        covered += cnt;
+    }
+    if (covered != slots) return fail(c, SMX_ERR_ARG, "moe_layer: plan covers %zu of %zu slots", covered, slots);
+    std::vector<int> tok_ptr(m + 1, 0), tok_slots(slots);
+    for (size_t s = 0; s < slots; s++) {
+        if (slot_tok[s] < 0 || (size_t)slot_tok[s] >= m)
+            return fail(c, SMX_ERR_ARG, "moe_layer: slot %zu names token %d of %zu", s, slot_tok[s], m);
+        tok_ptr[slot_tok[s] + 1]++;
+    }
+    for (size_t t = 0; t < m; t++) tok_ptr[t + 1] += tok_ptr[t];
+    {
+        std::vector<int> fill(tok_ptr.begin(), tok_ptr.end() - 1);
+        for (size_t s = 0; s < slots; s++) tok_slots[fill[slot_tok[s]]++] = (int)s;  // ascending slot order per token
+    }
+    std::vector<GemmTile> tiles_gu, tiles_dn;
+    build_tiles(plan, nplan, eff, &tiles_gu);
+    build_tiles(plan, nplan, hidden, &tiles_dn);
+
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, m * hidden * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, m * hidden * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xq, m * hidden)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xd, m * nb * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->xs, m * nb * 4)) != SMX_OK) return rc;
+    Carver cv;
+    const size_t o_g = cv.take(slots * eff * 4), o_u = cv.take(slots * eff * 4), o_aq = cv.take(slots * eff),
+                 o_ad = cv.take(slots * enb * 4), o_dy = cv.take(slots * hidden * 4);
+    if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
+    Carver ct;
+    const size_t o_st = ct.take(slots * 4), o_ws = ct.take(slots * 4), o_tp = ct.take((m + 1) * 4), o_ts = ct.take(slots * 4),
+                 o_t1 = ct.take(tiles_gu.size() * sizeof(GemmTile)), o_t2 = ct.take(tiles_dn.size() * sizeof(GemmTile));
+    if ((rc = ensure(c, c->tab, ct.off)) != SMX_OK) return rc;
+    float* g = (float*)(c->work.p + o_g);
+    float* u = (float*)(c->work.p + o_u);
+    int8_t* aq = (int8_t*)(c->work.p + o_aq);
+    float* ad = (float*)(c->work.p + o_ad);
+    float* dy = (float*)(c->work.p + o_dy);
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_st, slot_tok, slots * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ws, wslot, slots * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_tp, tok_ptr.data(), (m + 1) * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ts, tok_slots.data(), slots * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t1, tiles_gu.data(), tiles_gu.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t2, tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
+    // the host vectors above are pageable: the copies have completed when hipMemcpyAsync returns
+    rc = launch_actquant(c, (const float*)c->xf32.p, m, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+    if (rc != SMX_OK) return rc;
+    {
+        GemmArgs p = {};
+        p.op[0] = {L.gate.scales, L.gate.quants, g};
+        p.op[1] = {L.up.scales, L.up.quants, u};
+        p.xq = (const int8_t*)c->xq.p;
+        p.xd = (const float*)c->xd.p;
+        p.a_rowmap = (const int*)(c->tab.p + o_st);  // slot -> token: the gather of kernels.rs:1162-1171
+        p.tiles = (const GemmTile*)(c->tab.p + o_t1);
+        p.M = (int)slots;
+        p.N = (int)eff;
+        p.nb = (int)nb;
+        p.ldo = (int)eff;
+        p.stages_per_slice = (int)((nb + 3) / 4);
+        rc = launch_gemm_grouped(c, p, (int)tiles_gu.size(), 2, "moe_gemm_gate_up");
+        if (rc != SMX_OK) return rc;
+    }
+    rc = silu_mul_quant(c, g, u, eff, slots, eff, aq, ad);
+    if (rc != SMX_OK) return rc;
+    {
+        GemmArgs p = {};
+        p.op[0] = {L.down.scales, L.down.quants, dy};
+        p.op[1] = p.op[0];
+        p.xq = aq;
+        p.xd = ad;
+        p.tiles = (const GemmTile*)(c->tab.p + o_t2);
+        p.M = (int)slots;
+        p.N = (int)hidden;
+        p.nb = (int)enb;
+        p.ldo = (int)hidden;
+        p.stages_per_slice = (int)((enb + 3) / 4);
+        rc = launch_gemm_grouped(c, p, (int)tiles_dn.size(), 1, "moe_gemm_down");
+        if (rc != SMX_OK) return rc;
+    }
+    {
+        ProfScope ps(c, "moe_combine");
+        hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((hidden + 255) / 256), (unsigned)m), dim3(256), 0, c->stream,
+                           dy, (const int*)(c->tab.p + o_tp), (const int*)(c->tab.p + o_ts),
+                           (const float*)(c->tab.p + o_ws), (float*)c->yf32.p, (int)hidden);
+        SMX_HIP(c, hipGetLastError());
+    }
+    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, m * hidden * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,139 @@
+// Internal declarations shared by the library's translation units.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/strix_mi355.h"
+
+namespace smx {
+
+enum QType { kQ4_0 = 2, kQ8_0 = 8, kQ6_K = 14 };
+
+// A resident weight: one device allocation, planes at 256-byte aligned offsets,
+// at on-disk density (no f32 scale expansion).
+//   Q4_0: scales f16[N*nb]            | quants  16 B/block [N*nb]   (nibble bytes as stored)
+//   Q8_0: scales f16[N*nb]            | quants  i8[N*nb*32]
+//   Q6_K: ql 128 B/sb | qh 64 B/sb | sc i8 16/sb | d f16 /sb       (sb = 256-wide superblock)
+struct Weight {
+    QType type;
+    size_t K = 0, N = 0;   // in_dim, out_dim
+    size_t nblk = 0;       // blocks (Q4_0/Q8_0) or superblocks (Q6_K) per row
+    char* base = nullptr;  // device allocation
+    size_t bytes = 0;
+    // plane pointers into base
+    const uint16_t* scales = nullptr;  // Q4_0/Q8_0 f16 block scales; Q6_K: per-superblock d
+    const void* quants = nullptr;      // Q4_0/Q8_0 quants; Q6_K: ql
+    const void* qh = nullptr;          // Q6_K
+    const int8_t* sc = nullptr;        // Q6_K sub-scales
+};
+
+// A resident MoE layer (Q8_0 experts): three planar Q8_0 tensors whose rows are
+// the experts' rows back to back (expert e, row r -> row e*rows + r).
+struct MoeLayer {
+    size_t hidden = 0, eff = 0, ne = 0;
+    Weight gate, up, down;  // gate/up: N = ne*eff, K = hidden; down: N = ne*hidden, K = eff
+};
+
+struct DevBuf {
+    char* p = nullptr;
+    size_t cap = 0;
+};
+
+struct ProfRec {
+    std::string name;
+    hipEvent_t e0, e1;
+};
+
+}  // namespace smx
+
+struct smx_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string name;
+    std::string err;
+    std::unordered_map<std::string, smx::Weight> weights;
+    std::unordered_map<size_t, smx::MoeLayer> moe;
+    int num_cu = 256;
+
+    // scratch, grown on demand (never shrinks)
+    smx::DevBuf xf32;   // staged fp32 activations
+    smx::DevBuf xq;     // int8 activations
+    smx::DevBuf xd;     // f32 block scales
+    smx::DevBuf xs;     // packed i16 pairs: sums of each 16-element half block
+    smx::DevBuf yf32;   // staged outputs
+    smx::DevBuf work;   // split-K partials, MoE intermediates, dumps
+    smx::DevBuf work2;
+    smx::DevBuf tab;    // small tables (ids, weights, tile tables)
+
+    // profiling
+    bool prof_on = false;
+    std::vector<smx::ProfRec> prof;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> ev_pool;
+    std::string prof_names;
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+};
+
+namespace smx {
+
+int fail(smx_ctx* c, int code, const char* fmt, ...);
+int hip_fail(smx_ctx* c, hipError_t e, const char* what);
+#define SMX_HIP(c, call)                                                   \
+    do {                                                                   \
+        hipError_t e_ = (call);                                            \
+        if (e_ != hipSuccess) return ::smx::hip_fail((c), e_, #call);      \
+    } while (0)
+
+int ensure(smx_ctx* c, DevBuf& b, size_t bytes);
+
+// Brackets one kernel launch with an event pair when profiling is on.
+struct ProfScope {
+    smx_ctx* c;
+    int idx = -1;
+    ProfScope(smx_ctx* c, const char* name);
+    ~ProfScope();
+};
+
+// One weight/output pair of a GEMM launch.
+struct GemmOperand {
+    const uint16_t* wscales;  // f16 [rows][nb]
+    const void* wquants;      // Q8_0: i8 [rows][K];  Q4_0: 16 B [rows][nb]
+    float* out;               // [M][ldo] (split-K: Z such planes)
+};
+// One 128 x 128 output tile of a grouped GEMM.
+struct GemmTile {
+    int tok0, tok_end;  // activation rows [tok0, tok_end) (through a_rowmap if set)
+    int row0, row_end;  // weight rows, limit = end of this expert's rows
+    int col0;           // output column of row0
+};
+struct GemmArgs {
+    GemmOperand op[2];
+    const int8_t* xq;       // [*][K]
+    const float* xd;        // [*][nb]
+    const int* a_rowmap;    // optional: activation row index per logical row (MoE gather)
+    const GemmTile* tiles;  // optional tile table; dense tiling when null
+    int* dump;              // optional [M][N][nb]
+    int M, N, nb, ldo;
+    int tiles_m, tiles_n;
+    int stages_per_slice;   // stages (of 4 blocks) each grid.z slice covers
+    int xcd_remap;
+};
+
+// ---- launchers (all enqueue on c->stream; return SMX_OK or an error) ----
+// Activation quantiser: x[m][K] f32 -> xq[m][K], xd[m][K/32], xs[m][K/32] (two i16 sums per block).
+int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, float* xd, int32_t* xs);
+// GEMV: y[m][N], m <= SMX_GEMV_MAX_M (Q6_K: m == 1).  dump (optional): per-block i32 dots of row 0.
+int launch_gemv(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, const int32_t* xs,
+                size_t m, float* y, int32_t* dump);
+// GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
+int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
+                int32_t* dump);
+
+int launch_gemm_grouped(smx_ctx* c, const GemmArgs& args, int ntiles, int nops, const char* name);
+
+}  // namespace smx

@@ -1,0 +1,317 @@
+"""Pins the CPU oracle before anything is compared with it.
+
+* block layout + dequant: the reference's own literal-value tests
+  (crates/strix-models/src/ggml_quant.rs:443-469, 497-514, 562-565);
+* f32 matmul: the reference's seeded device-test data
+  (crates/strix-backend-rocm/src/lib.rs:135-180) against an independent float64 computation;
+* integer path (no reference test exists for it): brute-force int64 dots over integers recovered
+  through the pinned dequantiser, algebraic identities, quantiser invariants.
+"""
+import numpy as np
+import pytest
+
+Q4_0, Q8_0, Q6_K = 2, 8, 14
+
+
+def f16_bytes(orc, v):
+    h = orc.f32_to_f16(v)
+    return [h & 0xff, h >> 8]
+
+
+# ---------------------------------------------------------------- half precision
+
+def test_f16_exact_against_numpy(orc):
+    hs = np.arange(0, 65536, dtype=np.uint16)
+    ref = hs.view(np.float16).astype(np.float32)
+    got = np.array([orc.f16_to_f32(int(h)) for h in hs], np.float32)
+    ok = ~np.isnan(ref)
+    assert np.array_equal(got[ok].view(np.uint32), ref[ok].view(np.uint32))
+    # subnormal case the reference's device decode handles by hand (kernels.rs:9-15)
+    assert orc.f16_to_f32(0x0001) == 2.0 ** -24
+    rng = np.random.default_rng(0)
+    fs = np.concatenate([rng.standard_normal(2000).astype(np.float32) * 10.0 ** rng.integers(-8, 5, 2000),
+                         np.array([0.0, -0.0, 65504.0, 65520.0, 1e-8, 6e-8, 6.1e-5], np.float32)]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = fs.astype(np.float16).view(np.uint16)
+    got = np.array([orc.f32_to_f16(float(f)) for f in fs], np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- reference literal vectors
+
+def test_q8_0_scales_each_int(orc):          # ggml_quant.rs:443-453
+    qs = np.arange(32, dtype=np.int32) - 4
+    raw = np.array(f16_bytes(orc, 0.5) + [int(q) & 0xff for q in qs], np.uint8)
+    y = orc.dequantize(Q8_0, raw, 32)
+    assert np.abs(y - 0.5 * (np.arange(32) - 4.0)).max() < 1e-3
+
+
+def test_q4_0_nibble_layout_and_bias(orc):   # ggml_quant.rs:456-469
+    qs = [0] * 16
+    qs[0], qs[1] = 0x80, 0xF1
+    raw = np.array(f16_bytes(orc, 2.0) + qs, np.uint8)
+    y = orc.dequantize(Q4_0, raw, 32)
+    assert (y[0], y[16], y[1], y[17]) == (-16.0, 0.0, -14.0, 14.0)
+
+
+def test_q6_k_decodes_known_values(orc):     # ggml_quant.rs:497-514
+    blk = np.zeros(210, np.uint8)
+    blk[0] = 0x05
+    blk[128] = 0x01
+    blk[192:208] = 1
+    blk[208:210] = f16_bytes(orc, 1.0)
+    y = orc.dequantize(Q6_K, blk, 256)
+    assert y[0] == -11.0 and y[1] == -32.0 and y[32] == -32.0 and y.size == 256
+
+
+def test_rejects_bad_sizes(orc):             # ggml_quant.rs:562-565
+    with pytest.raises(ValueError):
+        orc.dequantize(Q8_0, np.zeros(34, np.uint8), 16)
+    with pytest.raises(ValueError):
+        orc.dequantize(Q4_0, np.zeros(4, np.uint8), 32)
+
+
+def test_golden_literal_fixture(orc, golden):
+    g = golden("literal_blocks.npz")
+    for name, ty in (("q8_0", Q8_0), ("q4_0", Q4_0), ("q6_k", Q6_K)):
+        y = orc.dequantize(ty, g[name + "_raw"], g[name + "_out"].size)
+        assert np.array_equal(y, g[name + "_out"])
+
+
+# ---------------------------------------------------------------- independent decoders (numpy)
+
+def np_q4_ints(raw, N, K):
+    b = raw.reshape(N, K // 32, 18)
+    d = b[:, :, :2].copy().view(np.float16).astype(np.float64)[:, :, 0]
+    qs = b[:, :, 2:].astype(np.int64)
+    q = np.concatenate([qs & 15, qs >> 4], axis=2) - 8          # elems 0..15 low nibbles, 16..31 high
+    return d, q
+
+
+def np_q8_ints(raw, N, K):
+    b = raw.reshape(N, K // 32, 34)
+    d = b[:, :, :2].copy().view(np.float16).astype(np.float64)[:, :, 0]
+    q = b[:, :, 2:].copy().view(np.int8).astype(np.int64)
+    return d, q
+
+
+@pytest.mark.parametrize("ty", [Q4_0, Q8_0])
+def test_dequant_matches_independent_numpy(orc, synth, ty):
+    N, K = 5, 160
+    raw = synth.make_weight(ty, N, K, seed=3)
+    d, q = (np_q4_ints if ty == Q4_0 else np_q8_ints)(raw, N, K)
+    want = (d[:, :, None].astype(np.float32) * q.astype(np.float32)).reshape(N, K)
+    assert np.array_equal(orc.dequantize(ty, raw, N * K).reshape(N, K), want)
+
+
+def test_f32_oracle_on_reference_seeded_data(orc):
+    """lib.rs:135-153: LCG 0xA5A5_1234, scales 0.03+(r%32)*0.003 as f16, x = 0.5 sin(0.017 i);
+    (rows cut from 3840 to 64 to keep the float64 check quick; same generator stream)."""
+    in_dim, out_dim = 15360, 64
+    nblk = in_dim // 32
+    total = nblk * out_dim
+    draws, _ = orc.lcg(0xA5A51234, total * 5)
+    draws = draws.reshape(total, 5)
+    sc = (np.float32(0.03) + (draws[:, 0] % 32).astype(np.float32) * np.float32(0.003)).astype(np.float32)
+    # the reference truncates toward zero in its test helper; both conversions of these values
+    # agree with numpy's to within one f16 ulp, and the test's claim is on the decoded value
+    sch = sc.astype(np.float16)
+    raw = np.empty((total, 18), np.uint8)
+    raw[:, :2] = sch.view(np.uint8).reshape(total, 2)
+    raw[:, 2:] = draws[:, 1:].astype("<u4").view(np.uint8).reshape(total, 16)
+    x = (np.sin(np.arange(in_dim, dtype=np.float32) * np.float32(0.017)) * np.float32(0.5)).astype(np.float32)
+    d, q = np_q4_ints(raw.reshape(-1), out_dim, in_dim)
+    want = (d[:, :, None] * q).reshape(out_dim, in_dim) @ x.astype(np.float64)
+    for order in (0, 1):
+        y = orc.matmul_f32(Q4_0, raw.reshape(-1), in_dim, out_dim, x, order)[0]
+        rel = np.abs(y - want).max() / np.abs(want).max()
+        assert rel < 1e-3          # the reference's own bar (lib.rs:231)
+        assert rel < 2e-5          # and what fp32 accumulation over 15360 terms actually gives
+
+
+def test_two_reference_summation_orders_differ_only_by_rounding(orc, synth):
+    raw = synth.make_weight(Q8_0, 8, 2560, seed=1)
+    x = synth.make_acts(1, 2560, seed=2)
+    a = orc.matmul_f32(Q8_0, raw, 2560, 8, x, 0)
+    b = orc.matmul_f32(Q8_0, raw, 2560, 8, x, 1)
+    assert np.abs(a - b).max() / np.abs(a).max() < 1e-5
+
+
+# ---------------------------------------------------------------- quantiser
+
+def test_actquant_invariants_and_brute_force(orc, synth):
+    K = 256
+    x = synth.make_acts(4, K, seed=11)
+    x[0, :32] = 0.0
+    x[1, 32:64] = np.float32(3.5)                     # constant block: every q = 127
+    xq, xd, xs = orc.actquant(x, K)
+    xb, qb = x.reshape(4, K // 32, 32), xq.reshape(4, K // 32, 32).astype(np.int32)
+    amax = np.abs(xb).max(axis=2)
+    assert np.array_equal(xd, (amax / np.float32(127.0)).astype(np.float32))
+    assert np.all(np.abs(qb).max(axis=2)[amax > 0] == 127)
+    assert np.all(qb[0, 0] == 0) and xd[0, 0] == 0.0
+    assert np.all(qb[1, 1] == 127)
+    assert np.all(np.abs(xb - qb * xd[:, :, None]) <= xd[:, :, None] * 0.5000001 + 1e-12)
+    assert np.array_equal(xs.reshape(4, K // 32, 2).astype(np.int32),
+                          np.stack([qb[:, :, :16].sum(2), qb[:, :, 16:].sum(2)], axis=2))
+    # elementwise definition, rint = ties to even (kernels.rs:86-88)
+    inv = np.where(xd > 0, np.float32(1.0) / np.where(xd > 0, xd, 1), 0).astype(np.float32)
+    want = np.clip(np.rint((xb * inv[:, :, None]).astype(np.float32)), -127, 127).astype(np.int8)
+    assert np.array_equal(xq.reshape(4, K // 32, 32), want)
+    # a value that lands exactly on .5 rounds to even, not away (unlike ggml_quant.rs:203)
+    x2 = np.zeros((1, 32), np.float32)
+    x2[0, 0], x2[0, 1] = 127.0, 2.5
+    assert orc.actquant(x2, 32)[0][0, 1] == 2
+
+
+# ---------------------------------------------------------------- integer block dots
+
+@pytest.mark.parametrize("ty", [Q4_0, Q8_0])
+def test_block_dots_brute_force(orc, synth, ty):
+    N, K = 6, 192
+    raw = synth.make_weight(ty, N, K, seed=21)
+    x = synth.make_acts(1, K, seed=22)
+    xq, xd, xs = orc.actquant(x, K)
+    _, q = (np_q4_ints if ty == Q4_0 else np_q8_ints)(raw, N, K)
+    xi = xq[0].astype(np.int64).reshape(K // 32, 32)
+    want = np.einsum("nbk,bk->nb", q, xi)
+    got = orc.block_dots(ty, raw, K, N, xq[0])
+    assert np.array_equal(got.astype(np.int64), want)
+    if ty == Q4_0:   # sum((q-8)x) = sum(qx) - 8 sum(x)  (kernels.rs:250)
+        s32 = xs[0].astype(np.int64).reshape(-1, 2).sum(1)
+        assert np.array_equal(want, np.einsum("nbk,bk->nb", q + 8, xi) - 8 * s32[None, :])
+
+
+def test_block_dots_extremes(orc):
+    # all-max magnitudes: |isum| = 32*127*127 for Q8_0, 32*8*127 for Q4_0 (q=0 -> -8)
+    K = 32
+    x = np.full((1, K), 5.0, np.float32)
+    xq, _, _ = orc.actquant(x, K)
+    assert np.all(xq == 127)
+    raw8 = np.array([0, 0x3c] + [0x81] * 32, np.uint8)     # d = 1.0, q = -127
+    assert orc.block_dots(Q8_0, raw8, K, 1, xq[0])[0, 0] == -32 * 127 * 127
+    raw4 = np.array([0, 0x3c] + [0x00] * 16, np.uint8)
+    assert orc.block_dots(Q4_0, raw4, K, 1, xq[0])[0, 0] == -8 * 32 * 127
+
+
+def test_q6k_block_dots_via_pinned_dequant(orc, synth):
+    """With d = 1 and every sub-scale 1 the (reference-pinned) dequantiser returns q-32 itself."""
+    N, K = 3, 512
+    raw = synth.make_q6_k(N, K, seed=31).reshape(-1, 210).copy()
+    raw[:, 192:208] = 1
+    raw[:, 208:210] = [0x00, 0x3c]
+    raw = raw.reshape(-1)
+    qi = orc.dequantize(Q6_K, raw, N * K).reshape(N, K).astype(np.int64)
+    assert qi.min() >= -32 and qi.max() <= 31
+    x = synth.make_acts(1, K, seed=32)
+    xq, _, _ = orc.actquant(x, K)
+    want = (qi * xq[0].astype(np.int64)[None, :]).reshape(N, K // 16, 16).sum(2)
+    assert np.array_equal(orc.block_dots(Q6_K, raw, K, N, xq[0]).astype(np.int64), want)
+
+
+# ---------------------------------------------------------------- fp32 combine
+
+@pytest.mark.parametrize("ty,K", [(Q4_0, 2560), (Q8_0, 2560), (Q6_K, 2560 + 256 * 2)])
+def test_q8_matmul_against_float64(orc, synth, ty, K):
+    """Exact value of the quantised product: sum over elements of w_dequant * (xq * xd), in float64."""
+    N, m = 12, 3
+    raw = synth.make_weight(ty, N, K, seed=41)
+    x = synth.make_acts(m, K, seed=42)
+    xq, xd, _ = orc.actquant(x, K)
+    wd = orc.dequantize(ty, raw, N * K).reshape(N, K).astype(np.float64)
+    xdeq = xq.astype(np.float64) * np.repeat(xd.astype(np.float64), 32, axis=1)
+    want = xdeq @ wd.T
+    got = orc.matmul_q8(ty, raw, K, N, xq, xd)
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-6
+    # and it sits within activation-rounding distance of the f32 oracle
+    f32 = orc.matmul_f32(ty, raw, K, N, x, 1)
+    assert np.abs(got - f32).max() / np.abs(f32).max() < 3e-2
+
+
+def test_q8_matmul_block_order_is_sequential(orc, synth):
+    """acc += (dw*dx)*float(isum), b ascending: replay in numpy float32."""
+    N, K = 4, 320
+    raw = synth.make_weight(Q8_0, N, K, seed=51)
+    x = synth.make_acts(1, K, seed=52)
+    xq, xd, _ = orc.actquant(x, K)
+    d, _ = np_q8_ints(raw, N, K)
+    isum = orc.block_dots(Q8_0, raw, K, N, xq[0])
+    acc = np.zeros(N, np.float32)
+    for b in range(K // 32):
+        acc = (acc + (d[:, b].astype(np.float32) * xd[0, b]) * isum[:, b].astype(np.float32)).astype(np.float32)
+    assert np.array_equal(orc.matmul_q8(Q8_0, raw, K, N, xq, xd)[0], acc)
+
+
+def test_gemm_rows_equal_gemv(orc, synth):
+    # mellum.rs:239-243: a batch row is bit-identical to the single-token result
+    raw = synth.make_weight(Q4_0, 10, 256, seed=61)
+    xs = synth.make_acts(4, 256, seed=62)
+    full = orc.matmul_q8_from_f32(Q4_0, raw, 256, 10, xs)
+    for t in range(4):
+        assert np.array_equal(full[t], orc.matmul_q8_from_f32(Q4_0, raw, 256, 10, xs[t])[0])
+
+
+# ---------------------------------------------------------------- GGUF-side quantisers
+
+def test_cpu_quantisers_roundtrip(orc, synth):
+    x = synth.make_acts(1, 256, seed=71)[0]
+    r8 = orc.quantize_q8_0(x)
+    y8 = orc.dequantize(Q8_0, r8, 256)
+    assert np.abs(y8 - x).max() <= np.abs(x).max() / 127 * 0.51 + 1e-3
+    r4 = orc.quantize_q4_0(x)
+    y4 = orc.dequantize(Q4_0, r4, 256)
+    assert np.abs(y4 - x).max() <= np.abs(x).max() / 8 * 1.01
+    # ggml_quant.rs:203 rounds ties away from zero
+    t = np.zeros(32, np.float32)
+    t[0], t[1] = 127.0, 2.5
+    assert orc.quantize_q8_0(t).view(np.int8)[2 + 1] == 3
+
+
+# ---------------------------------------------------------------- MoE
+
+def test_expf_and_silu_accuracy(orc):
+    xs = np.linspace(-30, 30, 4001, dtype=np.float32)
+    got = np.array([orc.expf(float(v)) for v in xs], np.float64)
+    want = np.exp(xs.astype(np.float64))
+    assert np.abs(got / want - 1).max() < 3e-7
+    assert orc.silu(0.0) == 0.0
+    g = np.array([orc.silu(float(v)) for v in xs], np.float64)
+    assert np.abs(g - xs / (1 + np.exp(-xs.astype(np.float64)))).max() < 3e-6
+
+
+def test_route_topk_ties_lowest_index(orc):
+    ids, w = orc.route_topk(np.array([0.5, 2.0, 2.0, -1.0, 2.0], np.float32), 2)
+    assert list(ids) == [1, 2] and abs(w.sum() - 1) < 1e-6 and abs(w[0] - 0.5) < 1e-6
+    logits = np.random.default_rng(3).standard_normal(64).astype(np.float32)
+    ids, w = orc.route_topk(logits, 8)
+    assert list(ids) == list(np.argsort(-logits, kind="stable")[:8])
+    p = np.exp(logits - logits.max())
+    p /= p.sum()
+    assert np.allclose(w, p[ids] / p[ids].sum(), rtol=1e-5)
+
+
+def test_moe_ffn_equals_sum_of_dense_experts(orc, synth):
+    """mellum.rs:1623-1669: y = sum_k w_k * down_k(silu(gate_k x) * up_k x), routed order."""
+    ne, hidden, eff, k = 6, 128, 64, 3
+    gate, up, down = synth.make_moe_q8(ne, hidden, eff, seed=81)
+    ids, w = synth.zipf_routing(1, ne, k, seed=82)
+    x = synth.make_acts(1, hidden, seed=83)[0]
+    y, gu, aq, ad = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[0], w[0], x)
+    geb, deb = (hidden // 32) * 34 * eff, (eff // 32) * 34 * hidden
+    acc = np.zeros(hidden, np.float32)
+    for kk, e in enumerate(ids[0]):
+        g = orc.matmul_q8_from_f32(Q8_0, gate[e * geb:(e + 1) * geb], hidden, eff, x)[0]
+        u = orc.matmul_q8_from_f32(Q8_0, up[e * geb:(e + 1) * geb], hidden, eff, x)[0]
+        assert np.array_equal(gu[kk, 0], g) and np.array_equal(gu[kk, 1], u)
+        a = np.array([orc.silu(float(a_)) for a_ in g], np.float32) * u
+        dy = orc.matmul_q8_from_f32(Q8_0, down[e * deb:(e + 1) * deb], eff, hidden, a)[0]
+        acc = (acc + w[0][kk] * dy).astype(np.float32)
+    assert np.array_equal(y, acc)
+    # against the f32 path end to end: only quantisation noise
+    accf = np.zeros(hidden, np.float64)
+    for kk, e in enumerate(ids[0]):
+        g = orc.matmul_f32(Q8_0, gate[e * geb:(e + 1) * geb], hidden, eff, x, 1)[0].astype(np.float64)
+        u = orc.matmul_f32(Q8_0, up[e * geb:(e + 1) * geb], hidden, eff, x, 1)[0].astype(np.float64)
+        a = (g / (1 + np.exp(-g)) * u).astype(np.float32)
+        accf += w[0][kk] * orc.matmul_f32(Q8_0, down[e * deb:(e + 1) * deb], eff, hidden, a, 1)[0]
+    assert np.abs(y - accf).max() / np.abs(accf).max() < 5e-2
