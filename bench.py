@@ -1,0 +1,314 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-matmul hot path on one MI355X.
+
+Headline workload (`value`): the Q4_0 decode GEMV, weight 9728 x 2560, one token, cache-cold:
+every step quantises the activation and runs the GEMV against the next of >= 1 GB of distinct
+resident weight copies, so no weight byte is served from the 256 MB Infinity Cache.  One step =
+one pass of the path (activation quantiser + GEMV) over one synthetic activation.  Inputs are
+resident in HBM before the timed region starts.
+
+The same JSON line carries the other configurations of the metric (Q8_0 / Q6_K GEMV, the int8
+MFMA prefill GEMM in TOPS, MoE) under "workloads", the roofline of the dominant kernel and the
+CPU baseline (the oracle's restatement of the reference's CPU matmul, timed on this host).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only name,...] [--no-cpu]
+"""
+import argparse
+import importlib.util
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
+Q4_0, Q8_0, Q6_K = 2, 8, 14
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q6_K: 210}
+BLOCK_ELEMS = {Q4_0: 32, Q8_0: 32, Q6_K: 256}
+KERNEL = {Q4_0: "gemv_q4_0", Q8_0: "gemv_q8_0", Q6_K: "gemv_q6_k"}
+UPLOAD = {Q4_0: "upload_q4_0", Q8_0: "upload_q8_0", Q6_K: "upload_q6_k"}
+
+
+def _load(name, path, search=None):
+    spec = importlib.util.spec_from_file_location(name, path, submodule_search_locations=search)
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def gemv_bytes(ty, N, K, m=1):
+    """Algorithmic bytes of one GEMV: weight blocks at on-disk density + int8 activations and their
+    f32 scales (+ the packed sums Q4_0/Q6_K read) + fp32 outputs."""
+    w = N * (K // BLOCK_ELEMS[ty]) * BLOCK_BYTES[ty]
+    act = m * K * (1 + 4 / 32 + (4 / 32 if ty != Q8_0 else 0))
+    return int(w + act + m * N * 4), w
+
+
+class Bench:
+    def __init__(self, steps, warmup):
+        pkg_dir = os.path.join(ROOT, "strix.rs_amd")
+        self.pkg = _load("strix_rs_amd", os.path.join(pkg_dir, "__init__.py"), [pkg_dir])
+        self.synth = _load("strix_rs_amd_synth", os.path.join(pkg_dir, "synth.py"))
+        self.acc = self.pkg.Mi355WeightAccel(0)
+        self.steps, self.warmup = steps, warmup
+
+    def log(self, *a):
+        print(*a, file=sys.stderr, flush=True)
+
+    def _timed(self, fn, steps, warmup):
+        """W untimed + exactly K timed steps, bracketed by stream syncs; HIP events on the stream."""
+        acc = self.acc
+        for i in range(warmup):
+            fn(i)
+        acc.sync()
+        t0 = time.perf_counter()
+        acc.timer_begin()
+        for i in range(steps):
+            fn(warmup + i)
+        ms = acc.timer_end()
+        acc.sync()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        return ms, wall_ms
+
+    def _kernel_avg_us(self, fn, steps, warmup, prefix):
+        """Second, identical pass with an event pair around every matmul kernel launch."""
+        acc = self.acc
+        acc.prof_reset()
+        for i in range(warmup):
+            fn(i)
+        acc.sync()
+        acc.prof_enable(True)
+        for i in range(steps):
+            fn(warmup + i)
+        acc.sync()
+        acc.prof_enable(False)
+        ms, n = acc.prof_read(prefix)
+        acc.prof_reset()
+        return (ms / n * 1e3 if n else float("nan")), n
+
+    # ------------------------------------------------------------------ GEMV
+    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None):
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
+        algo, wbytes = gemv_bytes(ty, N, K, m)
+        ncopies = max(2, -(-min_total_bytes // wbytes))
+        self.log(f"[{name}] {ncopies} weight copies x {wbytes / 1e6:.1f} MB")
+        nsrc = min(ncopies, 3)
+        src = [sy.make_weight(ty, N, K, seed=1000 + i) for i in range(nsrc)]
+        keys = []
+        for i in range(ncopies):
+            key = f"{name}.w{i}"
+            assert getattr(acc, UPLOAD[ty])(key, src[i % nsrc], K, N)
+            keys.append(key)
+        del src
+        x = sy.make_acts(m, K, seed=7)
+        xd = acc.dev_alloc(x.nbytes)
+        yd = acc.dev_alloc(m * N * 4)
+        acc.h2d(xd, x)
+
+        def step(i):
+            acc.gemv_dev(keys[i % ncopies], xd, m, yd)
+
+        ms, wall_ms = self._timed(step, steps, warmup)
+        kus, nk = self._kernel_avg_us(step, steps, warmup, KERNEL[ty])
+        for k in keys:
+            acc.evict(k)
+        acc.dev_free(xd)
+        acc.dev_free(yd)
+        gbs = algo * steps / (ms * 1e-3) / 1e9
+        kgbs = algo / (kus * 1e-6) / 1e9
+        return {
+            "workload": name, "shape": {"N": N, "K": K, "M": m}, "weight_copies": ncopies,
+            "algorithmic_bytes": algo, "weight_bytes": wbytes, "steps": steps, "ms_per_step": ms / steps,
+            "wall_ms_per_step": wall_ms / steps, "GBps": gbs, "weight_only_GBps": wbytes * steps / (ms * 1e-3) / 1e9,
+            "frac_hbm_peak": gbs / HBM_PEAK_GBS,
+            "kernel": KERNEL[ty], "kernel_avg_us": kus, "kernel_launches": nk, "kernel_GBps": kgbs,
+            "kernel_frac_hbm_peak": kgbs / HBM_PEAK_GBS,
+        }
+
+    # ------------------------------------------------------------------ GEMM
+    def gemm(self, name, ty, M, N, K, steps=None, warmup=None):
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or max(5, self.steps // 20), warmup if warmup is not None else 2
+        raw = sy.make_weight(ty, N, K, seed=2000 + ty)
+        assert getattr(acc, UPLOAD[ty])(name, raw, K, N)
+        del raw
+        xs = sy.make_acts(M, K, seed=8)
+        xd = acc.dev_alloc(xs.nbytes)
+        yd = acc.dev_alloc(M * N * 4)
+        acc.h2d(xd, xs)
+
+        def step(i):
+            acc.gemm_dev(name, xd, M, yd)
+
+        ms, wall_ms = self._timed(step, steps, warmup)
+        kname = "gemm_i8_q4_0" if ty == Q4_0 else "gemm_i8_q8_0"
+        kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
+        names = acc.prof_names()
+        acc.evict(name)
+        acc.dev_free(xd)
+        acc.dev_free(yd)
+        ops = 2 * M * N * K
+        tops = ops * steps / (ms * 1e-3) / 1e12
+        ktops = ops / (kus * 1e-6) / 1e12
+        return {
+            "workload": name, "shape": {"M": M, "N": N, "K": K}, "ops": ops, "steps": steps,
+            "ms_per_step": ms / steps, "wall_ms_per_step": wall_ms / steps, "TOPS": tops,
+            "frac_int8_peak": tops / INT8_PEAK_TOPS, "kernel": kname, "kernel_avg_us": kus, "kernel_launches": nk,
+            "kernel_TOPS": ktops, "kernel_frac_int8_peak": ktops / INT8_PEAK_TOPS,
+            "split_k": "splitk_reduce" in names,
+        }
+
+    # ------------------------------------------------------------------ MoE
+    def moe(self, name, ne, hidden, eff, k, m, layers, steps=None, warmup=None):
+        """Decode (m == 1): rotate over `layers` resident layers (320 MB each) so expert reads are
+        cache-cold.  Prefill (m > 1): one layer, m tokens grouped by expert."""
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
+        gate, up, down = sy.make_moe_q8(ne, hidden, eff, seed=3000)
+        for l in range(layers):
+            assert acc.upload_moe_q8(l, gate, up, down, hidden, eff, ne)
+        del gate, up, down
+        out = {"workload": name, "shape": {"experts": ne, "hidden": hidden, "eff": eff, "top_k": k, "M": m}}
+        if m == 1:
+            ids, w = sy.zipf_routing(max(64, steps + warmup), ne, k, seed=5)
+            x = sy.make_acts(1, hidden, seed=9)
+            xd = acc.dev_alloc(x.nbytes)
+            yd = acc.dev_alloc(hidden * 4)
+            acc.h2d(xd, x)
+
+            def step(i):
+                acc.moe_ffn_dev(i % layers, ids[i % len(ids)], w[i % len(ids)], xd, yd)
+
+            ms, wall_ms = self._timed(step, steps, warmup)
+            kus, nk = self._kernel_avg_us(step, steps, warmup, "moe_gemv")
+            acc.dev_free(xd)
+            acc.dev_free(yd)
+            wbytes = k * 3 * eff * (hidden // 32) * 34
+            gbs = wbytes * steps / (ms * 1e-3) / 1e9
+            out.update({"expert_weight_bytes": wbytes, "layers_rotated": layers, "steps": steps,
+                        "ms_per_step": ms / steps, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
+                        "kernel": "moe_gemv_gate_up + moe_gemv_down", "kernel_avg_us_sum": kus * 2,
+                        "kernel_GBps": wbytes / (kus * 2 * 1e-6) / 1e9})
+        else:
+            steps = max(5, steps // 20)
+            ids, w = sy.zipf_routing(m, ne, k, seed=5)
+            plan, slot_tok, wslot = sy.group_by_expert(ids, w, ne)
+            xs = sy.make_acts(m, hidden, seed=9)
+            t0 = time.perf_counter()
+            for _ in range(2):
+                acc.moe_layer_q8_dev(0, xs, m, plan, slot_tok, wslot)
+            acc.prof_reset()
+            acc.prof_enable(True)
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                acc.moe_layer_q8_dev(0, xs, m, plan, slot_tok, wslot)
+            wall_ms = (time.perf_counter() - t0) * 1e3
+            acc.prof_enable(False)
+            g_ms, _ = acc.prof_read("moe_gemm")
+            all_ms = sum(acc.prof_read(p)[0] for p in ("actquant", "moe_gemm", "silu_mul_quant", "moe_combine"))
+            acc.prof_reset()
+            ops = 2 * slot_tok.size * 3 * eff * hidden
+            out.update({"slots": int(slot_tok.size), "ops": ops, "steps": steps,
+                        "device_ms_per_step": all_ms / steps, "host_call_ms_per_step": wall_ms / steps,
+                        "TOPS": ops * steps / (all_ms * 1e-3) / 1e12,
+                        "gemm_kernels_TOPS": ops * steps / (g_ms * 1e-3) / 1e12,
+                        "frac_int8_peak": ops * steps / (all_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS})
+        for l in range(layers):
+            pass  # layers stay resident until the context closes (they are re-uploaded per workload)
+        return out
+
+
+def cpu_baseline(seconds=12.0):
+    """The reference's CPU matmul (dequantise a row, f32 dot, rows split over the host's cores:
+    crates/strix-backend-cpu/src/mellum.rs:219-237) as restated by the oracle, on the headline shape."""
+    orc = _load("strix_oracle", os.path.join(ROOT, "oracle", "strix_oracle.py"))
+    synth = sys.modules["strix_rs_amd_synth"]
+    N, K = 9728, 2560
+    cores = min(os.cpu_count() or 1, 16)
+    raws = [synth.make_weight(Q4_0, N, K, seed=1000 + i) for i in range(4)]
+    x = synth.make_acts(1, K, seed=7)
+    orc.matmul_f32(Q4_0, raws[0], K, N, x, 1, cores)
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        orc.matmul_f32(Q4_0, raws[n % 4], K, N, x, 1, cores)
+        n += 1
+    dt = time.perf_counter() - t0
+    algo, _ = gemv_bytes(Q4_0, N, K, 1)
+    return {"value": algo * n / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{n} f32 GEMVs of the 9728x2560 Q4_0 weight over {dt:.1f} s, 4 rotating copies, "
+                      f"row-parallel dequantise+dot on {cores} threads", "ms_per_gemv": dt / n * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
+    ap.add_argument("--no-cpu", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X "
+                 "(--gpus must be 1); how it would shard over several is described in DESIGN.md")
+    only = set(filter(None, a.only.split(",")))
+    want = lambda n: not only or n in only
+    b = Bench(a.steps, a.warmup)
+    b.log("device:", b.acc.name())
+    GB = 1 << 30
+    work = {}
+    head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB))
+    work[head["workload"]] = head
+    b.log(json.dumps(head))
+    plans = [
+        ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
+        ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
+        ("q6_k_gemv_15360x3840", lambda: b.gemv("q6_k_gemv_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB))),
+        ("q6_k_lm_head_262144x3840", lambda: b.gemv("q6_k_lm_head_262144x3840", Q6_K, 262144, 3840, 1, int(1.6 * GB),
+                                                     steps=max(10, a.steps // 10), warmup=2)),
+        ("gemm_q8_0_ffn_up", lambda: b.gemm("gemm_q8_0_ffn_up", Q8_0, 2048, 15360, 3840)),
+        ("gemm_q4_0_ffn_up", lambda: b.gemm("gemm_q4_0_ffn_up", Q4_0, 2048, 15360, 3840)),
+        ("gemm_q8_0_ffn_down", lambda: b.gemm("gemm_q8_0_ffn_down", Q8_0, 2048, 3840, 15360)),
+        ("gemm_q4_0_ffn_down", lambda: b.gemm("gemm_q4_0_ffn_down", Q4_0, 2048, 3840, 15360)),
+        ("moe_decode", lambda: b.moe("moe_decode", 64, 2048, 768, 8, 1, layers=4)),
+        ("moe_prefill_m512", lambda: b.moe("moe_prefill_m512", 64, 2048, 768, 8, 512, layers=1)),
+    ]
+    for name, fn in plans:
+        if want(name):
+            r = fn()
+            work[name] = r
+            b.log(json.dumps(r))
+    gemms = [w for n, w in work.items() if n.startswith("gemm_")]
+    best_gemm = max(gemms, key=lambda w: w["TOPS"]) if gemms else None
+    line = {
+        "metric": "Q4_0 GEMV GB/s (% HBM peak); int8 prefill GEMM TOPS (% MFMA peak)",
+        "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": head["steps"], "warmup": a.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "Q4_0 decode GEMV, weight 9728x2560, 1 token, Q8 activations, cache-cold: "
+                               f"{head['weight_copies']} rotating resident weight copies "
+                               f"({head['weight_copies'] * head['weight_bytes'] / 1e9:.2f} GB); "
+                               "step = activation quantiser + GEMV", "frac_hbm_peak": head["frac_hbm_peak"]},
+        "roofline": {"bound": "hbm", "achieved": head["kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["kernel_frac_hbm_peak"], "traffic": None, "kernel": head["kernel"],
+                     "kernel_avg_us": head["kernel_avg_us"], "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
+                     "method": "HIP event pair around every GEMV launch on the launch stream, second identical pass"},
+        "gemm": None if not best_gemm else {
+            "workload": best_gemm["workload"], "value": best_gemm["TOPS"], "unit": "TOPS",
+            "frac_int8_mfma_peak": best_gemm["frac_int8_peak"],
+            "roofline": {"bound": "mfma", "achieved": best_gemm["kernel_TOPS"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": best_gemm["kernel_frac_int8_peak"], "traffic": None, "kernel": best_gemm["kernel"]}},
+        "workloads": work,
+    }
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline()
+    b.acc.close()
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -123,6 +123,22 @@ int smx_gemm_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, f
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                     const float* x_dev, float* y_dev);
 
+/* ---- HIP graph capture of a sequence of `_dev` calls: the role of the reference's captured decode
+ *      token (decode.rs:3053-3203), so a launch-bound chain of small GEMVs replays without per-launch
+ *      host cost.  Between begin and end only `_dev` entry points may be called, with shapes already
+ *      seen once outside capture (no scratch growth while capturing); per-kernel timing is off. ---- */
+typedef struct smx_graph smx_graph;
+int smx_graph_begin(smx_ctx* ctx);
+int smx_graph_end(smx_ctx* ctx, smx_graph** out);
+int smx_graph_launch(smx_ctx* ctx, smx_graph* g);   /* enqueue one replay on the context's stream */
+void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
+
+/* Launch-geometry overrides for measurement sweeps; value 0 restores the built-in choice.
+ * Knobs: "gemv_rpw" (rows per wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4),
+ * "gemv_lpr" (lanes per row: 16, 32, 64), "gemv_wpc" (persistent workgroups per CU), "gemm_splitk" (K slices).  Results do not
+ * depend on them beyond fp32 summation order. */
+int smx_tune(smx_ctx* ctx, const char* knob, int value);
+
 /* ---- per-kernel timing: the role of STRIX_PROF, decode.rs:25-69, 2190-2203,
  *      done with HIP events on the context's stream instead of host syncs ---- */
 int smx_prof_enable(smx_ctx* ctx, int on);   /* on: bracket each matmul kernel with an event pair */

@@ -30,7 +30,8 @@ EXPORTS = [
     "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev",
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
-    "smx_moe_ffn_stages",
+    "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
+    "smx_graph_destroy",
 ]
 
 
@@ -95,6 +96,12 @@ def load_library():
     L.smx_gemv_block_dots.argtypes = [vp, cp, vp, sz, vp, sz]
     L.smx_gemm_block_dots.argtypes = [vp, cp, vp, sz, sz, vp, sz]
     L.smx_moe_ffn_stages.argtypes = [vp, sz, vp, vp, sz, vp, sz, vp, vp, vp, vp]
+    L.smx_tune.argtypes = [vp, cp, i]
+    L.smx_graph_begin.argtypes = [vp]
+    L.smx_graph_end.argtypes = [vp, C.POINTER(vp)]
+    L.smx_graph_launch.argtypes = [vp, vp]
+    L.smx_graph_destroy.argtypes = [vp, vp]
+    L.smx_graph_destroy.restype = None
     _lib = L
     return L
 
@@ -296,6 +303,23 @@ class Mi355WeightAccel:
     def moe_ffn_dev(self, layer, ids, wexp, x_dev, y_dev):
         ids, wexp = _c(ids, np.int32), _c(wexp, np.float32)
         return self._check(self._L.smx_moe_ffn_dev(self._h, layer, _p(ids), _p(wexp), ids.size, x_dev, y_dev))
+
+    def graph_begin(self):
+        self._check(self._L.smx_graph_begin(self._h))
+
+    def graph_end(self):
+        g = C.c_void_p()
+        self._check(self._L.smx_graph_end(self._h, C.byref(g)))
+        return g
+
+    def graph_launch(self, g):
+        self._check(self._L.smx_graph_launch(self._h, g))
+
+    def graph_destroy(self, g):
+        self._L.smx_graph_destroy(self._h, g)
+
+    def tune(self, knob, value):
+        self._check(self._L.smx_tune(self._h, knob.encode(), int(value)))
 
     def prof_enable(self, on=True):
         self._check(self._L.smx_prof_enable(self._h, 1 if on else 0))

@@ -1,5 +1,6 @@
 // extern "C" entry points of the matmul path: host-pointer calls (copy in, run, copy out, sync)
 // and device-pointer calls (enqueue only).
+#include <algorithm>
 #include <cstring>
 
 #include "smx_internal.h"
@@ -61,15 +62,13 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restric
 // quantise m device rows and run the right matmul kernel into y_dev
 int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm,
                    int32_t* dump) {
+    if (m <= SMX_GEMV_MAX_M && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump);  // quantiser fused
+    if (w.type == kQ6_K)
+        return fail(c, SMX_ERR_LIMIT, "Q6_K weights are served by the GEMV path only (at most %d rows per call)", SMX_GEMV_MAX_M);
     int rc = ensure_act(c, m, w.K);
     if (rc != SMX_OK) return rc;
     rc = launch_actquant(c, xs_dev, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
     if (rc != SMX_OK) return rc;
-    const bool gemv_ok = m <= SMX_GEMV_MAX_M && (w.type != kQ6_K || m == 1);
-    if (gemv_ok && !force_gemm)
-        return launch_gemv(c, w, (const int8_t*)c->xq.p, (const float*)c->xd.p, (const int32_t*)c->xs.p, m, y_dev,
-                           dump);
-    if (w.type == kQ6_K) return fail(c, SMX_ERR_LIMIT, "Q6_K weights are served by the GEMV path only (one row per call)");
     return launch_gemm(c, w, (const int8_t*)c->xq.p, (const float*)c->xd.p, m, y_dev, dump);
 }
 
@@ -159,8 +158,8 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
         float* yd = (float*)(c->yf32.p + yo);
         yoff[i] = yo;
         SMX_HIP(c, hipMemcpyAsync(xdv, xs[i], w->K * 4, hipMemcpyHostToDevice, c->stream));
-        rc = launch_actquant(c, xdv, 1, w->K, q, d, s);
-        if (rc == SMX_OK) rc = launch_gemv(c, *w, q, d, s, 1, yd, nullptr);
+        (void)q; (void)d; (void)s;
+        rc = launch_gemv(c, *w, xdv, 1, yd, nullptr);
         status[i] = rc;
         xo += (w->K * 4 + 255) & ~size_t(255);
         yo += (w->N * 4 + 255) & ~size_t(255);
@@ -187,14 +186,13 @@ int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t
     if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->tab, m * 4)) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
-    if (w->type == kQ6_K && m > 1) {
-        // Q6_K heads run one activation row per launch
-        rc = ensure_act(c, m, w->K);
-        if (rc != SMX_OK) return rc;
-        rc = launch_actquant(c, (const float*)c->xf32.p, m, w->K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
-        for (size_t t = 0; t < m && rc == SMX_OK; t++)
-            rc = launch_gemv(c, *w, (const int8_t*)c->xq.p + t * w->K, (const float*)c->xd.p + t * (w->K / 32),
-                             (const int32_t*)c->xs.p + t * (w->K / 32), 1, (float*)c->yf32.p + t * w->N, nullptr);
+    if (w->type == kQ6_K && m > SMX_GEMV_MAX_M) {
+        // Q6_K has no GEMM on this path: heads with more rows go through in GEMV-sized groups
+        rc = SMX_OK;
+        for (size_t t = 0; t < m && rc == SMX_OK; t += SMX_GEMV_MAX_M) {
+            const size_t mm = std::min<size_t>(SMX_GEMV_MAX_M, m - t);
+            rc = launch_gemv(c, *w, (const float*)c->xf32.p + t * w->K, mm, (float*)c->yf32.p + t * w->N, nullptr);
+        }
     } else {
         rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr);
     }

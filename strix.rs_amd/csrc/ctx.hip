@@ -25,6 +25,8 @@ int hip_fail(smx_ctx* c, hipError_t e, const char* what) {
 
 int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
     if (bytes <= b.cap) return SMX_OK;
+    if (c->capturing)
+        return fail(c, SMX_ERR_ARG, "scratch would grow to %zu bytes during graph capture: run the call once outside capture first", bytes);
     if (b.p) {
         SMX_HIP(c, hipStreamSynchronize(c->stream));
         SMX_HIP(c, hipFree(b.p));
@@ -43,7 +45,7 @@ int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
 }
 
 ProfScope::ProfScope(smx_ctx* c_, const char* name) : c(c_) {
-    if (!c->prof_on) return;
+    if (!c->prof_on || c->capturing) return;
     hipEvent_t e0, e1;
     if (!c->ev_pool.empty()) {
         e0 = c->ev_pool.back().first;
@@ -338,6 +340,76 @@ int smx_d2h(smx_ctx* c, void* dst, const void* src, size_t n) {
 int smx_sync(smx_ctx* c) {
     if (!c) return SMX_ERR_ARG;
     SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+struct smx_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+int smx_graph_begin(smx_ctx* c) {
+    if (!c) return SMX_ERR_ARG;
+    if (c->capturing) return fail(c, SMX_ERR_ARG, "graph_begin: already capturing");
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    SMX_HIP(c, hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
+    c->capturing = true;
+    return SMX_OK;
+}
+
+int smx_graph_end(smx_ctx* c, smx_graph** out) {
+    if (!c || !out) return SMX_ERR_ARG;
+    if (!c->capturing) return fail(c, SMX_ERR_ARG, "graph_end: not capturing");
+    c->capturing = false;
+    smx_graph* g = new (std::nothrow) smx_graph();
+    if (!g) return fail(c, SMX_ERR_NOMEM, "graph_end: out of host memory");
+    hipError_t e = hipStreamEndCapture(c->stream, &g->graph);
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        if (g->graph) (void)hipGraphDestroy(g->graph);
+        delete g;
+        return hip_fail(c, e, "hipStreamEndCapture/hipGraphInstantiate");
+    }
+    *out = g;
+    return SMX_OK;
+}
+
+int smx_graph_launch(smx_ctx* c, smx_graph* g) {
+    if (!c || !g) return SMX_ERR_ARG;
+    SMX_HIP(c, hipGraphLaunch(g->exec, c->stream));
+    return SMX_OK;
+}
+
+void smx_graph_destroy(smx_ctx* c, smx_graph* g) {
+    if (!g) return;
+    if (c) (void)hipStreamSynchronize(c->stream);
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    delete g;
+}
+
+int smx_tune(smx_ctx* c, const char* knob, int value) {
+    if (!c || !knob) return SMX_ERR_ARG;
+    if (value < 0) return fail(c, SMX_ERR_ARG, "tune: negative value for %s", knob);
+    const std::string k = knob;
+    if (k == "gemv_rpw") {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return fail(c, SMX_ERR_ARG, "tune: gemv_rpw must be 0, 1, 2 or 4");
+        c->tune_gemv_rpw = value;
+    } else if (k == "gemv_ks") {
+        if (value != 0 && value != 1 && value != 2 && value != 4) return fail(c, SMX_ERR_ARG, "tune: gemv_ks must be 0, 1, 2 or 4");
+        c->tune_gemv_ks = value;
+    } else if (k == "gemv_lpr") {
+        if (value != 0 && value != 16 && value != 32 && value != 64) return fail(c, SMX_ERR_ARG, "tune: gemv_lpr must be 0, 16, 32 or 64");
+        c->tune_gemv_lpr = value;
+    } else if (k == "gemv_wpc") {
+        if (value > 32) return fail(c, SMX_ERR_ARG, "tune: gemv_wpc must be 0..32");
+        c->tune_gemv_wpc = value;
+    } else if (k == "gemm_splitk") {
+        if (value > 16) return fail(c, SMX_ERR_ARG, "tune: gemm_splitk must be 0..16");
+        c->tune_gemm_splitk = value;
+    } else {
+        return fail(c, SMX_ERR_ARG, "tune: unknown knob %s", knob);
+    }
     return SMX_OK;
 }
 

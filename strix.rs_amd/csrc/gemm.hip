@@ -67,65 +67,82 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
     const int s_begin = blockIdx.z * p.stages_per_slice;
     const int s_end = min(nstage_total, s_begin + p.stages_per_slice);
 
-    // ---- global -> register staging ----
+    // ---- global -> register staging: branch-free (clamped addresses, masks applied when the
+    //      registers are written to LDS) so the loads of stage s+1 stay in flight during stage s ----
     uint4 ra[4], rb[4];
-    float rscale[KB];
+    unsigned rsw;  // raw weight scales: two f16 (blocks 2*sh, 2*sh+1 of the stage) of row sr
+    uint2 rsx;     // raw activation scales: two f32 of token sr
     // A (and Q8_0 B): lane = [chunk_hi:2][row_lo:3][chunk_lo:1], 8 rows x 128 B per wave load
     const int g_chunk = ((lane >> 4) << 1) | (lane & 1);  // 16-byte chunk 0..7 within the 128-byte stage row
     const int g_rowlo = (lane >> 1) & 7;
     // Q4_0 B: lane = [bi:2][row_lo:4]
     const int q_bi = lane >> 4, q_rowlo = lane & 15;
+    const bool nb4 = (p.nb & 3) == 0;  // whole stages only, scale rows 8/16-byte aligned
+    // per-thread row bases (fixed for the whole K loop)
+    size_t a_off[4], b_off[4];
+#pragma unroll
+    for (int ps = 0; ps < 4; ps++) {
+        const int r = (ps * 4 + wave) * 8 + g_rowlo;
+        const int ti = min(tok0 + r, M_end - 1);
+        a_off[ps] = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * K;
+        if (!Q4) {
+            b_off[ps] = (size_t)min(row0 + r, N_end - 1) * K;
+        } else if (ps < 2) {
+            const int rq = (ps * 4 + wave) * 16 + q_rowlo;
+            b_off[ps] = (size_t)min(row0 + rq, N_end - 1) * p.nb;
+        }
+    }
+    // scales: thread (sr, sh) carries blocks 2*sh, 2*sh+1 of the stage for weight row sr and token sr
+    const int sr = tid & 127, sh = tid >> 7;
+    const bool w_valid = row0 + sr < N_end, x_valid = tok0 + sr < M_end;
+    const size_t scw_base = (size_t)min(row0 + sr, N_end - 1) * p.nb;
+    size_t scx_base;
+    {
+        const int ti = min(tok0 + sr, M_end - 1);
+        scx_base = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * p.nb;
+    }
 
     auto load_stage = [&](int s) {
         const int blk0 = s * KB;
+        const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);  // clamped: a K tail is zeroed at store time
 #pragma unroll
         for (int ps = 0; ps < 4; ps++) {
-            const int r = (ps * 4 + wave) * 8 + g_rowlo;
-            const bool kv = blk0 + (g_chunk >> 1) < p.nb;
-            const int ti = min(tok0 + r, M_end - 1);
-            const size_t tok = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti);
-            ra[ps] = kv ? *(const uint4*)(p.xq + tok * K + (size_t)blk0 * 32 + g_chunk * 16) : make_uint4(0, 0, 0, 0);
-            if (!Q4) {
-                const size_t row = (size_t)min(row0 + r, N_end - 1);
-                rb[ps] = kv ? *(const uint4*)((const int8_t*)op.wquants + row * K + (size_t)blk0 * 32 + g_chunk * 16)
-                            : make_uint4(0, 0, 0, 0);
-            }
+            ra[ps] = *(const uint4*)(p.xq + a_off[ps] + koff);
+            if (!Q4) rb[ps] = *(const uint4*)((const int8_t*)op.wquants + b_off[ps] + koff);
         }
         if (Q4) {
+            const int bq = min(blk0 + q_bi, p.nb - 1);
 #pragma unroll
-            for (int ps = 0; ps < 2; ps++) {
-                const int r = (ps * 4 + wave) * 16 + q_rowlo;
-                const bool kv = blk0 + q_bi < p.nb;
-                const size_t row = (size_t)min(row0 + r, N_end - 1);
-                rb[ps] = kv ? ((const uint4*)op.wquants)[row * p.nb + blk0 + q_bi] : make_uint4(0, 0, 0, 0);
-            }
+            for (int ps = 0; ps < 2; ps++) rb[ps] = ((const uint4*)op.wquants)[b_off[ps] + bq];
         }
-        if (tid < 128) {
-            const int row = row0 + tid;
-            const size_t base = (size_t)min(row, N_end - 1) * p.nb + blk0;
-#pragma unroll
-            for (int bi = 0; bi < KB; bi++)
-                rscale[bi] = (row < N_end && blk0 + bi < p.nb) ? h2f_(op.wscales[base + bi]) : 0.f;
+        if (nb4) {
+            rsw = *(const unsigned*)(op.wscales + scw_base + blk0 + 2 * sh);
+            rsx = *(const uint2*)(p.xd + scx_base + blk0 + 2 * sh);
         } else {
-            const int tok = tok0 + tid - 128;
-            const int ti = min(tok, M_end - 1);
-            const size_t base = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * p.nb + blk0;
-#pragma unroll
-            for (int bi = 0; bi < KB; bi++) rscale[bi] = (tok < M_end && blk0 + bi < p.nb) ? p.xd[base + bi] : 0.f;
+            const int b0 = min(blk0 + 2 * sh, p.nb - 1), b1 = min(blk0 + 2 * sh + 1, p.nb - 1);
+            rsw = (unsigned)op.wscales[scw_base + b0] | ((unsigned)op.wscales[scw_base + b1] << 16);
+            rsx = make_uint2(__float_as_uint(p.xd[scx_base + b0]), __float_as_uint(p.xd[scx_base + b1]));
         }
     };
 
-    auto store_stage = [&](int buf) {
+    auto store_stage = [&](int buf, int s) {
         char* sA = smem + buf * STAGE_BYTES;
         char* sB = sA + A_BYTES;
         float* sdw = (float*)(sB + B_BYTES);
         float* sdx = sdw + KB * 128;
+        const int blk0 = s * KB;
+        const bool tail = blk0 + KB > p.nb;  // uniform: only the last stage of a K that is not a stage multiple
 #pragma unroll
         for (int ps = 0; ps < 4; ps++) {
             const int r = (ps * 4 + wave) * 8 + g_rowlo;
             const int off = ((g_chunk >> 1) * 4 + (r >> 5)) * FRAG + (g_chunk & 1) * HPLANE + (r & 31) * 16;
-            *(uint4*)(sA + off) = ra[ps];
-            if (!Q4) *(uint4*)(sB + off) = rb[ps];
+            uint4 va = ra[ps], vb = rb[ps];
+            if (tail && blk0 + (g_chunk >> 1) >= p.nb) {
+                va = make_uint4(0, 0, 0, 0);
+                vb = va;
+            }
+            *(uint4*)(sA + off) = va;
+            if (!Q4) *(uint4*)(sB + off) = vb;
         }
         if (Q4) {
 #pragma unroll
@@ -138,13 +155,19 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
                 lo.y = sub8(q.y & 0x0f0f0f0fu); hi.y = sub8((q.y >> 4) & 0x0f0f0f0fu);
                 lo.z = sub8(q.z & 0x0f0f0f0fu); hi.z = sub8((q.z >> 4) & 0x0f0f0f0fu);
                 lo.w = sub8(q.w & 0x0f0f0f0fu); hi.w = sub8((q.w >> 4) & 0x0f0f0f0fu);
+                if (tail && blk0 + q_bi >= p.nb) {
+                    lo = make_uint4(0, 0, 0, 0);
+                    hi = lo;
+                }
                 *(uint4*)(sB + off) = lo;            // elements 0..15 of the block
                 *(uint4*)(sB + off + HPLANE) = hi;   // elements 16..31
             }
         }
-        float* sp = tid < 128 ? sdw + tid : sdx + (tid - 128);
-#pragma unroll
-        for (int bi = 0; bi < KB; bi++) sp[bi * 128] = rscale[bi];
+        const bool v0 = blk0 + 2 * sh < p.nb, v1 = blk0 + 2 * sh + 1 < p.nb;
+        sdw[(2 * sh) * 128 + sr] = (w_valid && v0) ? h2f_((uint16_t)(rsw & 0xffff)) : 0.f;
+        sdw[(2 * sh + 1) * 128 + sr] = (w_valid && v1) ? h2f_((uint16_t)(rsw >> 16)) : 0.f;
+        sdx[(2 * sh) * 128 + sr] = (x_valid && v0) ? __uint_as_float(rsx.x) : 0.f;
+        sdx[(2 * sh + 1) * 128 + sr] = (x_valid && v1) ? __uint_as_float(rsx.y) : 0.f;
     };
 
     float acc[4][16];
@@ -161,7 +184,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
 
     if (s_begin < s_end) {
         load_stage(s_begin);
-        store_stage(0);
+        store_stage(0, s_begin);
     }
     __syncthreads();
     for (int s = s_begin; s < s_end; s++) {
@@ -201,7 +224,7 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
                 }
             }
         }
-        if (s + 1 < s_end) store_stage(buf ^ 1);
+        if (s + 1 < s_end) store_stage(buf ^ 1, s + 1);
         __syncthreads();
     }
 
@@ -262,7 +285,7 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     const int T = p.tiles_m * p.tiles_n;
     p.xcd_remap = (T % 8 == 0) ? 1 : 0;
     const int nstages = (p.nb + KB - 1) / KB;
-    int Z = (dump || (m * w.N) % 4 != 0) ? 1 : pick_splitk(c, T, nstages);
+    int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(c, T, nstages));
     p.stages_per_slice = (nstages + Z - 1) / Z;
     Z = (nstages + p.stages_per_slice - 1) / p.stages_per_slice;
     p.op[0].out = y;
@@ -278,7 +301,9 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
 #define LAUNCH_GEMM(Q4, DUMP)                                                                              \
     do {                                                                                                   \
         auto k = gemm_i8_kernel<Q4, DUMP>;                                                                 \
-        SMX_HIP(c, hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
+        static size_t lds_set = 0;                                                                         \
+        int rc_ = set_dyn_lds(c, k, lds, &lds_set);                                                        \
+        if (rc_ != SMX_OK) return rc_;                                                                     \
         hipLaunchKernelGGL(k, grid, dim3(256), lds, c->stream, p);                                         \
     } while (0)
         if (w.type == kQ4_0) {
@@ -305,7 +330,9 @@ int launch_gemm_grouped(smx_ctx* c, const GemmArgs& args, int ntiles, int nops, 
     const size_t lds = 2 * STAGE_BYTES;
     ProfScope ps(c, name);
     auto k = gemm_i8_kernel<false, false>;
-    SMX_HIP(c, hipFuncSetAttribute((const void*)k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    static size_t lds_set = 0;
+    int rc = set_dyn_lds(c, k, lds, &lds_set);
+    if (rc != SMX_OK) return rc;
     hipLaunchKernelGGL(k, dim3((unsigned)ntiles, (unsigned)nops, 1), dim3(256), lds, c->stream, args);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;

@@ -9,167 +9,188 @@
 //   * v_dot4_i32_i8 integer block dots, exact i32 per block, then acc += (dw*dx)*float(isum);
 //   * cross-lane (DPP) combination of lanes that share a block, wave-wide reduction at the end.
 // HBM-bound: algorithmic bytes per row are K/32 * {18, 34} (Q4_0, Q8_0) or K/256 * 210 (Q6_K).
+#include <algorithm>
+
 #include "gemv_body.h"
 #include "smx_internal.h"
 
 namespace smx {
 
-
-template <int MT, int RPW, bool DUMP>
-__global__ __launch_bounds__(1024) void gemv_q4_0_kernel(const uint16_t* __restrict__ scales,
-                                                         const uint4* __restrict__ quants,
-                                                         const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                         const int* __restrict__ xs, float* __restrict__ y, int nb,
-                                                         int N, int m, int* __restrict__ dump) {
-    const int row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW;
-    gemv_q4_0_body<MT, RPW, DUMP>(scales, quants, xq, xd, xs, y, nb, N, m, dump, row0);
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool FUSEQ, bool DUMP, int NT>
+__global__ __launch_bounds__(NT) void gemv_kernel(GemvW W, GemvX X, float* __restrict__ y, int nblk, int N, int m,
+                                                  int* __restrict__ dump, int dump_per_row) {
+    const int nw = NT / 64;
+    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FUSEQ, DUMP>(W, X, y, N, nblk, N, m, dump, dump_per_row,
+                                                       blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
-template <int MT, int RPW, bool DUMP>
-__global__ __launch_bounds__(1024) void gemv_q8_0_kernel(const uint16_t* __restrict__ scales,
-                                                         const uint4* __restrict__ quants,
-                                                         const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                         float* __restrict__ y, int nb, int N, int m,
-                                                         int* __restrict__ dump) {
-    const int row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW;
-    gemv_q8_0_body<MT, RPW, DUMP>(scales, quants, xq, xd, y, nb, N, m, dump, row0);
-}
+namespace {
 
-template <int RPW, bool DUMP>
-__global__ __launch_bounds__(1024) void gemv_q6_k_kernel(const uint4* __restrict__ ql, const uint4* __restrict__ qh,
-                                                         const uint2* __restrict__ sc,
-                                                         const uint16_t* __restrict__ dsb,
-                                                         const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                         const int* __restrict__ xs, float* __restrict__ y, int nsb,
-                                                         int N, int* __restrict__ dump) {
-    const int row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW;
-    gemv_q6_k_body<RPW, DUMP>(ql, qh, sc, dsb, xq, xd, xs, y, nsb, N, dump, row0);
-}
+// Launch geometry: slots per wave, pipeline depth, K-split, lanes per row, threads per workgroup.
+struct Geom {
+    int rpw, pre, ks, lpr, nt;
+    unsigned grid;
+    size_t lds;
+};
 
-// ---------------------------------------------------------------- launch
-
-template <typename Kern>
-static int set_lds(smx_ctx* c, Kern kern, size_t lds) {
-    if (lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "gemv: activation needs %zu bytes of LDS (limit 163840)", lds);
-    if (lds > 48 * 1024)
-        SMX_HIP(c, hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool DUMP, int NT>
+int launch_one(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float* y, int nblk, int N, int m, int* dump,
+               int dump_per_row) {
+    // one activation row: quantiser fused into the staging; several rows: staged from rows quantised once
+    auto k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, MT == 1, DUMP, NT>;
+    static size_t lds_set = 0;
+    int rc = set_dyn_lds(c, k, g.lds, &lds_set);
+    if (rc != SMX_OK) return rc;
+    hipLaunchKernelGGL(k, dim3(g.grid), dim3(NT), g.lds, c->stream, W, X, y, nblk, N, m, dump, dump_per_row);
+    SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
 
-struct GemvGeom {
-    int rpw, nw;
-    unsigned grid;
-};
+// The compiled variants (RPW, PRE, KS, LPR):
+//   whole-wave rows   (4,2,1,64) (2,2,1,64) (1,4,1,64) (1,2,2,64) (1,2,4,64)
+//   sub-wave rows     (2,2,1,32) (1,2,1,32) (2,2,1,16) (1,2,1,16)        [one activation row only]
+template <class Ops, int MT>
+int launch_variant(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float* y, int nblk, int N, int m) {
+    // sub-wave rows: the pipeline is deep enough to put a whole short row set in flight before the
+    // activation is staged (Q6_K units are three times as wide, so half the depth)
+    constexpr bool kWide = sizeof(typename Ops::Regs) > 32;
+    if (MT == 1 && g.lpr == 32) {
+        if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 32, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+        return launch_one<Ops, 1, 1, kWide ? 2 : 4, 1, 32, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    }
+    if (MT == 1 && g.lpr == 16) {
+        if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 16, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+        return launch_one<Ops, 1, 1, kWide ? 4 : 6, 1, 16, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    }
+    if (g.ks == 4) return launch_one<Ops, MT, 1, 2, 4, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    if (g.ks == 2) return launch_one<Ops, MT, 1, 2, 2, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    if (g.rpw == 1) return launch_one<Ops, MT, 1, 4, 1, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    if (g.rpw == 4 && MT == 1) return launch_one<Ops, 1, 4, 2, 1, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    return launch_one<Ops, MT, 2, 2, 1, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+}
 
-// Rows per wave and waves per workgroup.  Small activations: 4-wave groups (many groups per CU);
-// large staged activations: 16-wave groups so one LDS copy serves a whole CU's worth of waves.
-static GemvGeom pick_geom(const smx_ctx* c, size_t N, size_t lds, size_t row_bytes, int max_rpw) {
-    GemvGeom g;
-    g.nw = lds > 40 * 1024 ? 16 : 4;
-    // keep >= ~8 waves per CU in flight when the matrix allows it, and give short rows more per wave
-    int rpw = 1;
-    const size_t want_waves = (size_t)c->num_cu * 8;
-    while (rpw < max_rpw && N / (size_t)(rpw * 2) >= want_waves && row_bytes * (size_t)rpw < 8192) rpw *= 2;
-    g.rpw = rpw;
-    const size_t rows_per_wg = (size_t)g.nw * g.rpw;
-    g.grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
+template <class Ops>
+int launch_type(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float* y, int nblk, int N, int m, int mt,
+                int* dump, int dump_per_row) {
+    if (dump) {
+        if (g.lpr == 16) return launch_one<Ops, 1, 1, 2, 1, 16, true, 256>(c, g, W, X, y, nblk, N, m, dump, dump_per_row);
+        return launch_one<Ops, 1, 1, 4, 1, 64, true, 256>(c, g, W, X, y, nblk, N, m, dump, dump_per_row);
+    }
+    switch (mt) {
+        case 1: return launch_variant<Ops, 1>(c, g, W, X, y, nblk, N, m);
+        case 2: return launch_variant<Ops, 2>(c, g, W, X, y, nblk, N, m);
+        case 4: return launch_variant<Ops, 4>(c, g, W, X, y, nblk, N, m);
+        default: return launch_variant<Ops, 8>(c, g, W, X, y, nblk, N, m);
+    }
+}
+
+}  // namespace
+
+// Geometry choice.  The small GEMVs of a decode step are bound by instruction issue and start-up
+// latency rather than by HBM, so: 16-wave workgroups (the activation is quantised and staged once
+// per 16 waves), persistent workgroups looping over chunks, lanes-per-row chosen to waste the fewest
+// lanes on short rows, and for weights with few, long rows the passes of a row are split over 2 or
+// 4 waves (K-split) so every SIMD has work.
+static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int mt, bool dump) {
+    Geom g;
+    size_t tokb, units;
+    if (type == kQ4_0) { tokb = (nblk * 40 + 15) & ~size_t(15); units = nblk; }
+    else if (type == kQ8_0) { tokb = (nblk * 36 + 15) & ~size_t(15); units = nblk * 2; }
+    else { tokb = nblk * 2 * 176; units = nblk * 4; }
+    g.nt = 1024;
+    g.lpr = 64;
+    g.ks = 1;
+    const size_t waves = (size_t)c->num_cu * 16;
+    // lanes per row: fewest wasted lanes, whole-wave rows on ties (short rows, one activation row only)
+    if (mt == 1 && units < 256) {
+        size_t best = ((units + 63) / 64) * 64;
+        for (int lpr : {32, 16}) {
+            const size_t slots = ((units + lpr - 1) / lpr) * lpr;
+            // measured: with equal waste, rows of fewer than 128 units run best two to a wave
+            if (slots < best || (slots == best && lpr == 32 && units < 128)) { best = slots; g.lpr = lpr; }
+        }
+    }
+    if (c->tune_gemv_lpr > 0 && mt == 1) g.lpr = c->tune_gemv_lpr;
+    const int P = (int)((units + g.lpr - 1) / g.lpr);
+    if (g.lpr == 64) {
+        // K-split pays for a single activation row only (batched rows are bound by their own arithmetic)
+        if (mt == 1 && P >= 4 && N * 2 <= waves) g.ks = (P >= 8 && N * 4 <= waves) ? 4 : 2;
+        else if (mt == 1 && P >= 4 && N <= waves) g.ks = 2;  // more wave-tasks than one round of waves: extra workgroups queue
+        if (g.ks > 1) { g.rpw = 1; g.pre = 2; }
+        else if (P >= 4) { g.rpw = 1; g.pre = 4; }
+        else if (mt == 1 && type != kQ6_K && P <= 2 && N >= waves * 4) { g.rpw = 4; g.pre = 2; }
+        else { g.rpw = 2; g.pre = 2; }
+        if (c->tune_gemv_rpw > 0 || c->tune_gemv_ks > 0) {
+            const int ks = c->tune_gemv_ks > 0 ? c->tune_gemv_ks : 1;
+            const int rpw = c->tune_gemv_rpw > 0 ? c->tune_gemv_rpw : 1;
+            if (ks > 1) { g.ks = ks; g.rpw = 1; g.pre = 2; }
+            else if (rpw == 1) { g.ks = 1; g.rpw = 1; g.pre = 4; }
+            else if (rpw == 4 && mt == 1) { g.ks = 1; g.rpw = 4; g.pre = 2; }
+            else { g.ks = 1; g.rpw = 2; g.pre = 2; }
+        }
+        // register budget of the 16-wave workgroup (128 VGPRs): Q6_K units are wide, batched rows multiply accumulators
+        if (g.ks == 1 && g.rpw > 1 && ((type == kQ6_K && (g.rpw > 2 || mt > 1)) || mt == 8)) {
+            g.rpw = (type == kQ6_K && mt == 1) ? 2 : 1;
+            g.pre = g.rpw == 1 ? 4 : 2;
+        }
+    } else {
+        const size_t rows_per_slot = 64 / g.lpr;
+        g.pre = 2;
+        g.rpw = (N / rows_per_slot >= waves * 2 && type != kQ6_K) ? 2 : 1;
+        if (c->tune_gemv_rpw > 0) g.rpw = c->tune_gemv_rpw >= 2 && type != kQ6_K ? 2 : 1;
+    }
+    if (dump) { g.rpw = 1; g.pre = g.lpr == 16 ? 2 : 4; g.ks = 1; g.nt = 256; if (g.lpr == 32) g.lpr = 64; }
+    const int nw = g.nt / 64;
+    const size_t rc = (size_t)g.rpw * (64 / g.lpr);
+    g.lds = tokb * (size_t)mt + (g.ks > 1 ? (size_t)nw * rc * mt * 4 : 0);
+    const size_t chunks = (N + rc - 1) / rc;
+    const size_t wgs = (chunks * g.ks + nw - 1) / nw;
+    if (g.ks > 1) {
+        g.grid = (unsigned)wgs;  // one chunk per wave group
+    } else {
+        int wpc = c->tune_gemv_wpc > 0 ? c->tune_gemv_wpc : 1;
+        if (dump) wpc = 8;
+        g.grid = (unsigned)std::min<size_t>(wgs, (size_t)c->num_cu * wpc);
+    }
     return g;
 }
 
-#define LAUNCH_Q4(MT, RPW, DUMP)                                                                                   \
-    do {                                                                                                           \
-        auto k = gemv_q4_0_kernel<MT, RPW, DUMP>;                                                                  \
-        int rc = set_lds(c, k, lds);                                                                               \
-        if (rc != SMX_OK) return rc;                                                                               \
-        hipLaunchKernelGGL(k, dim3(g.grid), dim3(g.nw * 64), lds, c->stream, w.scales, (const uint4*)w.quants, xq, \
-                           xd, (const int*)xs, y, (int)w.nblk, (int)w.N, (int)m, (int*)dump);                      \
-    } while (0)
-
-#define LAUNCH_Q8(MT, RPW, DUMP)                                                                                   \
-    do {                                                                                                           \
-        auto k = gemv_q8_0_kernel<MT, RPW, DUMP>;                                                                  \
-        int rc = set_lds(c, k, lds);                                                                               \
-        if (rc != SMX_OK) return rc;                                                                               \
-        hipLaunchKernelGGL(k, dim3(g.grid), dim3(g.nw * 64), lds, c->stream, w.scales, (const uint4*)w.quants, xq, \
-                           xd, y, (int)w.nblk, (int)w.N, (int)m, (int*)dump);                                      \
-    } while (0)
-
-#define LAUNCH_Q6(RPW, DUMP)                                                                                      \
-    do {                                                                                                          \
-        auto k = gemv_q6_k_kernel<RPW, DUMP>;                                                                     \
-        int rc = set_lds(c, k, lds);                                                                              \
-        if (rc != SMX_OK) return rc;                                                                              \
-        hipLaunchKernelGGL(k, dim3(g.grid), dim3(g.nw * 64), lds, c->stream, (const uint4*)w.quants,              \
-                           (const uint4*)w.qh, (const uint2*)w.sc, w.scales, xq, xd, (const int*)xs, y,           \
-                           (int)w.nblk, (int)w.N, (int*)dump);                                                    \
-    } while (0)
-
-#define DISPATCH_MT_RPW(L)                                  \
-    do {                                                    \
-        if (mt == 1) {                                      \
-            if (g.rpw == 1) L(1, 1, false);                 \
-            else if (g.rpw == 2) L(1, 2, false);            \
-            else L(1, 4, false);                            \
-        } else if (mt == 2) {                               \
-            if (g.rpw == 1) L(2, 1, false);                 \
-            else L(2, 2, false);                            \
-        } else if (mt == 4) {                               \
-            if (g.rpw == 1) L(4, 1, false);                 \
-            else L(4, 2, false);                            \
-        } else {                                            \
-            if (g.rpw == 1) L(8, 1, false);                 \
-            else L(8, 2, false);                            \
-        }                                                   \
-    } while (0)
-
-int launch_gemv(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, const int32_t* xs, size_t m,
-                float* y, int32_t* dump) {
+int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump) {
     if (m == 0 || m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv: %zu rows (1..%d supported)", m, SMX_GEMV_MAX_M);
     if (w.N > 0x7fffffffu / 4 || w.K > (size_t(1) << 20))
         return fail(c, SMX_ERR_LIMIT, "gemv: shape %zu x %zu exceeds the kernel's index range", w.N, w.K);
-    const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8));
-    if (w.type == kQ4_0) {
-        const size_t lds = (size_t)mt * ((w.nblk * 40 + 15) & ~size_t(15));
-        GemvGeom g = pick_geom(c, w.N, lds, w.nblk * 18, mt == 1 ? 4 : 2);
-        ProfScope ps(c, "gemv_q4_0");
-        if (dump) {
-            g.rpw = 1;
-            g.grid = (unsigned)((w.N + g.nw - 1) / g.nw);
-            LAUNCH_Q4(1, 1, true);
-        } else {
-            DISPATCH_MT_RPW(LAUNCH_Q4);
-        }
-    } else if (w.type == kQ8_0) {
-        const size_t lds = (size_t)mt * ((w.nblk * 36 + 15) & ~size_t(15));
-        GemvGeom g = pick_geom(c, w.N, lds, w.nblk * 34, mt == 1 ? 4 : 2);
-        ProfScope ps(c, "gemv_q8_0");
-        if (dump) {
-            g.rpw = 1;
-            g.grid = (unsigned)((w.N + g.nw - 1) / g.nw);
-            LAUNCH_Q8(1, 1, true);
-        } else {
-            DISPATCH_MT_RPW(LAUNCH_Q8);
-        }
-    } else {
-        if (m != 1) return fail(c, SMX_ERR_LIMIT, "gemv: Q6_K weights take one activation row per call");
-        const size_t ngrp = w.nblk * 2;
-        const size_t lds = ngrp * 9 * 16 + ngrp * 16 + ngrp * 16;
-        GemvGeom g = pick_geom(c, w.N, lds, w.nblk * 210, 4);
-        ProfScope ps(c, "gemv_q6_k");
-        if (dump) {
-            g.rpw = 1;
-            g.grid = (unsigned)((w.N + g.nw - 1) / g.nw);
-            LAUNCH_Q6(1, true);
-        } else if (g.rpw == 1) {
-            LAUNCH_Q6(1, false);
-        } else if (g.rpw == 2) {
-            LAUNCH_Q6(2, false);
-        } else {
-            LAUNCH_Q6(4, false);
-        }
+    if (w.type == kQ6_K && m > 4) {  // Q6_K keeps at most 4 activation rows in registers per launch
+        int rc = launch_gemv(c, w, x, 4, y, nullptr);
+        if (rc != SMX_OK) return rc;
+        return launch_gemv(c, w, x + 4 * w.K, m - 4, y + 4 * w.N, nullptr);
     }
-    SMX_HIP(c, hipGetLastError());
-    return SMX_OK;
+    const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8));
+    const Geom g = pick_geom(c, w.type, w.N, w.nblk, mt, dump != nullptr);
+    if (g.lds > 160 * 1024)
+        return fail(c, SMX_ERR_LIMIT, "gemv: %zu activation rows of %zu need %zu bytes of LDS (limit 163840)", m, w.K, g.lds);
+    GemvW W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
+    GemvX X = {x, nullptr, nullptr, nullptr};
+    if (mt > 1) {
+        // each of the persistent workgroups would repeat the quantiser for all m rows: do it once instead
+        int rc;
+        if ((rc = ensure(c, c->xq, m * w.K)) != SMX_OK) return rc;
+        if ((rc = ensure(c, c->xd, m * (w.K / 32) * 4)) != SMX_OK) return rc;
+        if ((rc = ensure(c, c->xs, m * (w.K / 32) * 4)) != SMX_OK) return rc;
+        rc = launch_actquant(c, x, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+        if (rc != SMX_OK) return rc;
+        X = {nullptr, (const int8_t*)c->xq.p, (const float*)c->xd.p, (const int*)c->xs.p};
+    }
+    const int nblk = (int)w.nblk, N = (int)w.N;
+    if (w.type == kQ4_0) {
+        ProfScope ps(c, "gemv_q4_0");
+        return launch_type<OpsQ4_0>(c, g, W, X, y, nblk, N, (int)m, mt, dump, (int)(w.K / 32));
+    }
+    if (w.type == kQ8_0) {
+        ProfScope ps(c, "gemv_q8_0");
+        return launch_type<OpsQ8_0>(c, g, W, X, y, nblk, N, (int)m, mt, dump, (int)(w.K / 32));
+    }
+    ProfScope ps(c, "gemv_q6_k");
+    return launch_type<OpsQ6_K>(c, g, W, X, y, nblk, N, (int)m, mt, dump, (int)(w.K / 16));
 }
 
 }  // namespace smx

@@ -1,6 +1,19 @@
-// Device bodies of the fused block-dequant GEMV (shared by the dense and the MoE launches).
-// Each body serves the RPW consecutive rows starting at `row0` for the calling wavefront; every
-// wave of the workgroup must call it (the activation staging ends in a workgroup barrier).
+// Device body of the fused block-dequant GEMV (shared by the dense and the MoE launches).
+//
+// One wavefront serves RPW consecutive output rows at a time ("chunk") and walks the rows in
+// 64-lane passes; every lane streams one 16-byte unit of packed quants per row and pass:
+//     Q4_0  unit = one 32-block   (16 B nibbles + f16 scale)
+//     Q8_0  unit = half a block   (16 B int8; lanes 2i, 2i+1 share block i and its scale)
+//     Q6_K  unit = 64 elements    (2 x 16 B ql + 16 B qh + 8 B sub-scales + f16 d; lanes 2i, 2i+1
+//                                  hold the two 16-element halves of four 32-wide blocks)
+// The (chunk, pass) items of a wave form one sequence that is software-pipelined PRE items deep:
+// the first PRE items are requested before the activation is staged, and each consumed item's
+// registers are refilled at once with the item PRE steps ahead, so HBM requests never wait for
+// arithmetic.  Waves are persistent: chunk ids advance by the total number of waves.
+//
+// The activation is staged once per workgroup in LDS, either from pre-quantised int8 rows or,
+// fused, straight from the fp32 rows through the path's quantiser (d = amax/127,
+// q = clamp(rint(x/d)), crates/strix-backend-rocm/src/kernels.rs:75-96).
 #pragma once
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
@@ -9,379 +22,460 @@
 
 namespace smx {
 
+// Optional per-wave timeline stamps (development builds only; compiled out of the library).
+#ifdef SMX_TRACE
+extern __device__ unsigned long long* g_smx_trace;
+#define SMX_STAMP_DECL unsigned long long smx_ts[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define SMX_STAMP(slot) smx_ts[slot] = wall_clock64()
+#define SMX_STAMP_FLUSH()                                                                                 \
+    do {                                                                                                  \
+        if ((threadIdx.x & 63) == 0 && g_smx_trace) {                                                     \
+            unsigned long long* o_ = g_smx_trace + ((size_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 8; \
+            for (int s_ = 0; s_ < 8; s_++) o_[s_] = smx_ts[s_];                                           \
+        }                                                                                                 \
+    } while (0)
+#else
+#define SMX_STAMP_DECL do { } while (0)
+#define SMX_STAMP(slot) do { } while (0)
+#define SMX_STAMP_FLUSH() do { } while (0)
+#endif
+
 __device__ __forceinline__ float h2f(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 __device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
 // value of the neighbouring lane (lane ^ 1)
 __device__ __forceinline__ int swap1(int v) { return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xf, 0xf, false); }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+// Cross-lane moves on the DPP path (no LDS round trip).  CTRL: 0xB1 = lane^1, 0x4E = lane^2 (quad
+// permutes), 0x141 = mirror within 8 lanes, 0x140 = mirror within a 16-lane row, 0x142 / 0x143 =
+// broadcast of lane 15 / 31 into the following row(s).
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+
+// Sum over groups of LPR (16, 32 or 64) adjacent lanes in a fixed order; the last lane of each group
+// (lane % LPR == LPR - 1) ends up holding the group's total.
+template <int LPR>
+__device__ __forceinline__ float group_sum(float v) {
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x141>(v);
+    v += dpp_f<0x140>(v);                         // all lanes of a 16-lane row hold the row's sum
+    if (LPR >= 32) v += dpp_f<0x142, 0xa>(v);     // rows 1, 3 += rows 0, 2
+    if (LPR == 64) v += dpp_f<0x143, 0xc>(v);     // rows 2, 3 += rows 0+1
     return v;
 }
 
-// ------------------------------------------------------------------ Q4_0
-// LDS: per token  lo[nb] uint4 | hi[nb] uint4 | xd[nb] f32 | xs[nb] i32
-template <int MT, int RPW, bool DUMP>
-__device__ __forceinline__ void gemv_q4_0_body(const uint16_t* __restrict__ scales,
-                                                         const uint4* __restrict__ quants,
-                                                         const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                         const int* __restrict__ xs, float* __restrict__ y, int nb,
-                                                         int N, int m, int* __restrict__ dump, const int row0) {
-    extern __shared__ __align__(16) char smem[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int tok_bytes = (nb * 40 + 15) & ~15;
+// Pointers of one resident weight (planar layout) and of the activation.
+struct GemvW {
+    const uint16_t* scales;  // Q4_0/Q8_0: f16 per block; Q6_K: f16 d per superblock
+    const uint4* quants;     // Q4_0: 1 uint4/block; Q8_0: 2 uint4/block; Q6_K: ql, 8 uint4/superblock
+    const uint4* qh;         // Q6_K: 4 uint4/superblock
+    const uint2* sc;         // Q6_K: 2 uint2/superblock
+};
+struct GemvX {
+    const float* x;      // fp32 rows [m][K] (fused quantiser) or null
+    const int8_t* xq;    // pre-quantised rows [m][K]
+    const float* xd;     // [m][K/32]
+    const int* xs;       // [m][K/32] packed 16-element sums
+};
 
-    // first pass of weight loads goes out before the activation is staged
-    uint4 wq[RPW];
-    uint16_t wsc[RPW];
-    size_t rbase[RPW];
-    {
-        const int bc = min(lane, nb - 1);
-#pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            rbase[r] = (size_t)min(row0 + r, N - 1) * nb;
-            wq[r] = quants[rbase[r] + bc];
-            wsc[r] = scales[rbase[r] + bc];
-        }
+// ---------------------------------------------------------------------------------------------
+// Per-format pieces.  `U` = units per row, `nb32` = 32-blocks per row.
+
+struct OpsQ4_0 {
+    struct Regs { uint4 q; uint16_t s; };
+    static __device__ __forceinline__ int units_per_row(int nblk) { return nblk; }
+    static __device__ __forceinline__ int nb32(int nblk) { return nblk; }
+    static __device__ __forceinline__ int tok_bytes(int nblk) { return (nblk * 40 + 15) & ~15; }
+    // LDS per token: lo[nb] uint4 | hi[nb] uint4 | {f32 d, i32 8*sum(q)}[nb]
+    static __device__ __forceinline__ int* xq_dword(char* tok, int nblk, int blk, int sub) {
+        uint4* lo = (uint4*)tok;
+        return (int*)((sub < 4 ? lo : lo + nblk) + blk) + (sub & 3);
     }
+    static __device__ __forceinline__ void put_scale(char* tok, int nblk, int blk, float d, int s_lo, int s_hi) {
+        int2* p = (int2*)(tok + nblk * 32) + blk;
+        *p = make_int2(__float_as_int(d), 8 * (s_lo + s_hi));
+    }
+    static constexpr bool kNeedsSums = true;
+    static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nblk, int u) {
+        r.q = w.quants[row * nblk + u];
+        r.s = w.scales[row * nblk + u];
+    }
+};
+
+struct OpsQ8_0 {
+    struct Regs { uint4 q; uint16_t s; };
+    static __device__ __forceinline__ int units_per_row(int nblk) { return nblk * 2; }
+    static __device__ __forceinline__ int nb32(int nblk) { return nblk; }
+    static __device__ __forceinline__ int tok_bytes(int nblk) { return (nblk * 36 + 15) & ~15; }
+    // LDS per token: xq[2nb] uint4 | sd[nb] f32
+    static __device__ __forceinline__ int* xq_dword(char* tok, int, int blk, int sub) {
+        return (int*)tok + blk * 8 + sub;
+    }
+    static __device__ __forceinline__ void put_scale(char* tok, int nblk, int blk, float d, int, int) {
+        ((float*)(tok + nblk * 32))[blk] = d;
+    }
+    static constexpr bool kNeedsSums = false;
+    static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nblk, int u) {
+        r.q = w.quants[row * nblk * 2 + u];
+        r.s = w.scales[row * nblk + (u >> 1)];
+    }
+};
+
+struct OpsQ6_K {
+    struct Regs { uint4 a, b, h; uint2 sc; uint16_t d; };
+    static __device__ __forceinline__ int units_per_row(int nsb) { return nsb * 4; }
+    static __device__ __forceinline__ int nb32(int nsb) { return nsb * 8; }
+    static __device__ __forceinline__ int tok_bytes(int nsb) { return nsb * 2 * (9 * 16 + 16 + 16); }
+    // LDS per token: xq 16-byte chunks, 8 per 128 elements padded to 9 | sd float4[2nsb] | ss int4[2nsb]
+    static __device__ __forceinline__ int* xq_dword(char* tok, int, int blk, int sub) {
+        const int ci = blk * 2 + (sub >> 2);
+        return (int*)((uint4*)tok + (ci >> 3) * 9 + (ci & 7)) + (sub & 3);
+    }
+    static __device__ __forceinline__ void put_scale(char* tok, int nsb, int blk, float d, int s_lo, int s_hi) {
+        ((float*)(tok + nsb * 2 * 144))[blk] = d;
+        ((int*)(tok + nsb * 2 * 160))[blk] = (s_lo & 0xffff) | (s_hi << 16);
+    }
+    static constexpr bool kNeedsSums = true;
+    static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nsb, int u) {
+        const size_t sb0 = row * nsb;
+        r.a = w.quants[sb0 * 8 + (u >> 1) * 4 + (u & 1)];
+        r.b = w.quants[sb0 * 8 + (u >> 1) * 4 + (u & 1) + 2];
+        r.h = w.qh[sb0 * 4 + u];
+        r.sc = w.sc[sb0 * 2 + (u >> 1)];
+        r.d = w.scales[sb0 + (u >> 2)];
+    }
+};
+
+// Q4_0: whole-block i32 = sum(nibble*xq) - 8*sum(xq)  (kernels.rs:241-250), then (dw*dx)*float(isum)
+template <int MT, bool DUMP>
+__device__ __forceinline__ void compute_unit(OpsQ4_0, const OpsQ4_0::Regs& r, const char* smem, int tokb, int nblk,
+                                             int u, bool act, float* acc, int* dump_row) {
+    unsigned lo4[4], hi4[4];
+    const unsigned w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        lo4[g] = w[g] & 0x0f0f0f0fu;         // elements 4g..4g+3
+        hi4[g] = (w[g] >> 4) & 0x0f0f0f0fu;  // elements 16+4g..
+    }
+    const float dw = act ? h2f(r.s) : 0.f;
+#pragma unroll
     for (int t = 0; t < MT; t++) {
-        uint4* lo = (uint4*)(smem + t * tok_bytes);
-        uint4* hi = lo + nb;
-        float* sd = (float*)(hi + nb);
-        int* ss = (int*)(sd + nb);
-        if (t < m) {
-            const uint4* src = (const uint4*)(xq + (size_t)t * nb * 32);
-            for (int i = tid; i < nb * 2; i += blockDim.x) ((i & 1) ? hi : lo)[i >> 1] = src[i];
-            for (int i = tid; i < nb; i += blockDim.x) {
-                sd[i] = xd[(size_t)t * nb + i];
-                ss[i] = xs[(size_t)t * nb + i];
-            }
-        } else {
-            for (int i = tid; i < nb; i += blockDim.x) {
-                lo[i] = make_uint4(0, 0, 0, 0);
-                hi[i] = make_uint4(0, 0, 0, 0);
-                sd[i] = 0.f;
-                ss[i] = 0;
-            }
+        const char* tok = smem + t * tokb;
+        const uint4 xl = ((const uint4*)tok)[u], xh = ((const uint4*)tok)[nblk + u];
+        const int2 ds = ((const int2*)(tok + nblk * 32))[u];
+        const float dx = __int_as_float(ds.x);
+        int isum = 0;
+        isum = dot4((int)lo4[0], (int)xl.x, isum);
+        isum = dot4((int)hi4[0], (int)xh.x, isum);
+        isum = dot4((int)lo4[1], (int)xl.y, isum);
+        isum = dot4((int)hi4[1], (int)xh.y, isum);
+        isum = dot4((int)lo4[2], (int)xl.z, isum);
+        isum = dot4((int)hi4[2], (int)xh.z, isum);
+        isum = dot4((int)lo4[3], (int)xl.w, isum);
+        isum = dot4((int)hi4[3], (int)xh.w, isum);
+        isum -= ds.y;  // sum((q-8)x) = sum(qx) - 8 sum(x)
+        if (DUMP) {
+            if (act && t == 0 && dump_row) dump_row[u] = isum;
         }
+        acc[t] += (dw * dx) * (float)isum;
     }
-    __syncthreads();
-
-    float acc[RPW][MT];
-#pragma unroll
-    for (int r = 0; r < RPW; r++)
-#pragma unroll
-        for (int t = 0; t < MT; t++) acc[r][t] = 0.f;
-
-    for (int b0 = 0; b0 < nb; b0 += 64) {
-        const int b = b0 + lane;
-        const bool act = b < nb;
-        const int bc = act ? b : nb - 1;
-        uint4 nq[RPW];
-        uint16_t nsc[RPW];
-        const bool more = b0 + 64 < nb;
-        if (more) {
-            const int bn = min(b + 64, nb - 1);
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                nq[r] = quants[rbase[r] + bn];
-                nsc[r] = scales[rbase[r] + bn];
-            }
-        }
-        unsigned lo4[RPW][4], hi4[RPW][4];
-        float dw[RPW];
-#pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            const unsigned w[4] = {wq[r].x, wq[r].y, wq[r].z, wq[r].w};
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                lo4[r][g] = w[g] & 0x0f0f0f0fu;         // elements 4g..4g+3
-                hi4[r][g] = (w[g] >> 4) & 0x0f0f0f0fu;  // elements 16+4g..
-            }
-            dw[r] = act ? h2f(wsc[r]) : 0.f;
-        }
-#pragma unroll
-        for (int t = 0; t < MT; t++) {
-            const uint4* lo = (const uint4*)(smem + t * tok_bytes);
-            const uint4* hi = lo + nb;
-            const float* sd = (const float*)(hi + nb);
-            const int* ss = (const int*)(sd + nb);
-            const uint4 xl = lo[bc], xh = hi[bc];
-            const float dx = sd[bc];
-            const int sp = ss[bc];
-            const int xsum = (int)(short)(sp & 0xffff) + (sp >> 16);
-            const int xlw[4] = {(int)xl.x, (int)xl.y, (int)xl.z, (int)xl.w};
-            const int xhw[4] = {(int)xh.x, (int)xh.y, (int)xh.z, (int)xh.w};
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                int isum = 0;
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    isum = dot4((int)lo4[r][g], xlw[g], isum);
-                    isum = dot4((int)hi4[r][g], xhw[g], isum);
-                }
-                isum -= 8 * xsum;  // sum((q-8)x) = sum(qx) - 8 sum(x)
-                if (DUMP) {
-                    if (act && t == 0 && row0 + r < N) dump[(size_t)(row0 + r) * nb + b] = isum;
-                }
-                acc[r][t] += (dw[r] * dx) * (float)isum;
-            }
-        }
-        if (more) {
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                wq[r] = nq[r];
-                wsc[r] = nsc[r];
-            }
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RPW; r++)
-#pragma unroll
-        for (int t = 0; t < MT; t++) {
-            const float s = wave_sum(acc[r][t]);
-            if (lane == 0 && row0 + r < N && t < m) y[(size_t)t * N + row0 + r] = s;
-        }
 }
 
-// ------------------------------------------------------------------ Q8_0
-// A lane owns a 16-byte half block; lanes 2i and 2i+1 share block i and add their i32 halves.
-// LDS: per token  xq[nb*2] uint4 | xd[nb] f32
-template <int MT, int RPW, bool DUMP>
-__device__ __forceinline__ void gemv_q8_0_body(const uint16_t* __restrict__ scales,
-                                                         const uint4* __restrict__ quants,
-                                                         const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                         float* __restrict__ y, int nb, int N, int m,
-                                                         int* __restrict__ dump, const int row0) {
-    extern __shared__ __align__(16) char smem[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int cpr = nb * 2;  // 16-byte chunks per row
-    const int tok_bytes = (nb * 36 + 15) & ~15;
-
-    uint4 wq[RPW];
-    uint16_t wsc[RPW];
-    size_t rbase[RPW];
-    {
-        const int cc = min(lane, cpr - 1);
+// Q8_0: the two half-block lanes add their i32 halves (DPP), the even lane carries the block
+template <int MT, bool DUMP>
+__device__ __forceinline__ void compute_unit(OpsQ8_0, const OpsQ8_0::Regs& r, const char* smem, int tokb, int nblk,
+                                             int u, bool act, float* acc, int* dump_row) {
+    const float dw = (act && !(u & 1)) ? h2f(r.s) : 0.f;
 #pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            rbase[r] = (size_t)min(row0 + r, N - 1) * nb;
-            wq[r] = quants[rbase[r] * 2 + cc];
-            wsc[r] = scales[rbase[r] + (cc >> 1)];
-        }
-    }
     for (int t = 0; t < MT; t++) {
-        uint4* sq = (uint4*)(smem + t * tok_bytes);
-        float* sd = (float*)(sq + cpr);
-        if (t < m) {
-            const uint4* src = (const uint4*)(xq + (size_t)t * nb * 32);
-            for (int i = tid; i < cpr; i += blockDim.x) sq[i] = src[i];
-            for (int i = tid; i < nb; i += blockDim.x) sd[i] = xd[(size_t)t * nb + i];
-        } else {
-            for (int i = tid; i < cpr; i += blockDim.x) sq[i] = make_uint4(0, 0, 0, 0);
-            for (int i = tid; i < nb; i += blockDim.x) sd[i] = 0.f;
+        const char* tok = smem + t * tokb;
+        const uint4 xv = ((const uint4*)tok)[u];
+        const float dx = ((const float*)(tok + nblk * 32))[u >> 1];
+        int isum = dot4((int)r.q.x, (int)xv.x, 0);
+        isum = dot4((int)r.q.y, (int)xv.y, isum);
+        isum = dot4((int)r.q.z, (int)xv.z, isum);
+        isum = dot4((int)r.q.w, (int)xv.w, isum);
+        isum += swap1(isum);  // whole-block i32
+        if (DUMP) {
+            if (act && !(u & 1) && t == 0 && dump_row) dump_row[u >> 1] = isum;
         }
+        acc[t] += (dw * dx) * (float)isum;
     }
-    __syncthreads();
-
-    float acc[RPW][MT];
-#pragma unroll
-    for (int r = 0; r < RPW; r++)
-#pragma unroll
-        for (int t = 0; t < MT; t++) acc[r][t] = 0.f;
-
-    for (int c0 = 0; c0 < cpr; c0 += 64) {
-        const int ch = c0 + lane;
-        const bool act = ch < cpr;
-        const int cc = act ? ch : cpr - 1;
-        const int b = cc >> 1;
-        uint4 nq[RPW];
-        uint16_t nsc[RPW];
-        const bool more = c0 + 64 < cpr;
-        if (more) {
-            const int cn = min(ch + 64, cpr - 1);
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                nq[r] = quants[rbase[r] * 2 + cn];
-                nsc[r] = scales[rbase[r] + (cn >> 1)];
-            }
-        }
-        float dw[RPW];
-#pragma unroll
-        for (int r = 0; r < RPW; r++) dw[r] = (act && !(cc & 1)) ? h2f(wsc[r]) : 0.f;  // even lane carries the block
-#pragma unroll
-        for (int t = 0; t < MT; t++) {
-            const uint4* sq = (const uint4*)(smem + t * tok_bytes);
-            const float* sd = (const float*)(sq + cpr);
-            const uint4 xv = sq[cc];
-            const float dx = sd[b];
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                int isum = dot4((int)wq[r].x, (int)xv.x, 0);
-                isum = dot4((int)wq[r].y, (int)xv.y, isum);
-                isum = dot4((int)wq[r].z, (int)xv.z, isum);
-                isum = dot4((int)wq[r].w, (int)xv.w, isum);
-                isum += swap1(isum);  // whole-block i32
-                if (DUMP) {
-                    if (act && !(cc & 1) && t == 0 && row0 + r < N) dump[(size_t)(row0 + r) * nb + b] = isum;
-                }
-                acc[r][t] += (dw[r] * dx) * (float)isum;
-            }
-        }
-        if (more) {
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                wq[r] = nq[r];
-                wsc[r] = nsc[r];
-            }
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RPW; r++)
-#pragma unroll
-        for (int t = 0; t < MT; t++) {
-            const float s = wave_sum(acc[r][t]);
-            if (lane == 0 && row0 + r < N && t < m) y[(size_t)t * N + row0 + r] = s;
-        }
 }
 
-// ------------------------------------------------------------------ Q6_K
-// A lane owns a 64-element task (superblock sb, half h, 16-lane column c): two 16-byte ql chunks
-// (c and c+2 of the half), one 16-byte qh chunk, i.e. four 16-element sub-blocks 8h + 2j + c.
-// Lanes 2i / 2i+1 (c = 0 / 1) hold the two halves of the same four 32-wide activation blocks.
-// Element map: crates/strix-models/src/ggml_quant.rs:417-426.
-// LDS: xq as 16-byte chunks, 8 per 128 elements padded to 9 | xd[K/32] f32 | xs[K/32] i32
-template <int RPW, bool DUMP>
-__device__ __forceinline__ void gemv_q6_k_body(const uint4* __restrict__ ql, const uint4* __restrict__ qh,
-                                                         const uint2* __restrict__ sc,
-                                                         const uint16_t* __restrict__ dsb,
-                                                         const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                         const int* __restrict__ xs, float* __restrict__ y, int nsb,
-                                                         int N, int* __restrict__ dump, const int row0) {
-    extern __shared__ __align__(16) char smem[];
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int tpr = nsb * 4;   // tasks per row
-    const int ngrp = nsb * 2;  // 128-element groups
-    uint4* sq = (uint4*)smem;
-    float4* sd = (float4*)(sq + ngrp * 9);
-    int4* ss = (int4*)(sd + ngrp);
-
-    uint4 wa[RPW], wb[RPW], wh[RPW];
-    uint2 wsc[RPW];
-    uint16_t wd[RPW];
-    size_t rsb[RPW];
-    {
-        const int tk = min(lane, tpr - 1);
+// Q6_K: four 16-element sub-block dots per lane (sub-blocks 8h + 2j + c of the superblock, element
+// map crates/strix-models/src/ggml_quant.rs:417-426); t_j = sc*isum summed over the lane pair is the
+// scaled i32 of 32-block 4h + j; acc += (d*dx_j)*float(t_j).
+template <int MT, bool DUMP>
+__device__ __forceinline__ void compute_unit(OpsQ6_K, const OpsQ6_K::Regs& r, const char* smem, int tokb, int nsb,
+                                             int u, bool act, float* acc, int* dump_row) {
+    const int g = u >> 1, c = u & 1;
+    const unsigned a4[4] = {r.a.x, r.a.y, r.a.z, r.a.w};
+    const unsigned b4[4] = {r.b.x, r.b.y, r.b.z, r.b.w};
+    const unsigned h4[4] = {r.h.x, r.h.y, r.h.z, r.h.w};
+    unsigned q[4][4];
 #pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            rsb[r] = (size_t)min(row0 + r, N - 1) * nsb;
-            wa[r] = ql[rsb[r] * 8 + (tk >> 1) * 4 + (tk & 1)];
-            wb[r] = ql[rsb[r] * 8 + (tk >> 1) * 4 + (tk & 1) + 2];
-            wh[r] = qh[rsb[r] * 4 + tk];
-            wsc[r] = sc[rsb[r] * 2 + (tk >> 1)];
-            wd[r] = dsb[rsb[r] + (tk >> 2)];
-        }
+    for (int i = 0; i < 4; i++) {
+        q[0][i] = (a4[i] & 0x0f0f0f0fu) | ((h4[i] << 4) & 0x30303030u);
+        q[1][i] = (b4[i] & 0x0f0f0f0fu) | ((h4[i] << 2) & 0x30303030u);
+        q[2][i] = ((a4[i] >> 4) & 0x0f0f0f0fu) | (h4[i] & 0x30303030u);
+        q[3][i] = ((b4[i] >> 4) & 0x0f0f0f0fu) | ((h4[i] >> 2) & 0x30303030u);
     }
-    {
-        const uint4* src = (const uint4*)xq;
-        for (int i = tid; i < ngrp * 8; i += blockDim.x) sq[(i >> 3) * 9 + (i & 7)] = src[i];
-        const float4* srcd = (const float4*)xd;
-        const int4* srcs = (const int4*)xs;
-        for (int i = tid; i < ngrp; i += blockDim.x) {
-            sd[i] = srcd[i];
-            ss[i] = srcs[i];
-        }
-    }
-    __syncthreads();
-
-    float acc[RPW];
+    const float d = (act && c == 0) ? h2f(r.d) : 0.f;  // even lane carries the 32-blocks
+    const unsigned long long scw = ((unsigned long long)r.sc.y << 32) | r.sc.x;
 #pragma unroll
-    for (int r = 0; r < RPW; r++) acc[r] = 0.f;
-
-    for (int t0 = 0; t0 < tpr; t0 += 64) {
-        const int tku = t0 + lane;
-        const bool act = tku < tpr;
-        const int tk = act ? tku : tpr - 1;
-        const int g = tk >> 1, c = tk & 1;
-        uint4 na[RPW], nbq[RPW], nh[RPW];
-        uint2 nsc[RPW];
-        uint16_t nd[RPW];
-        const bool more = t0 + 64 < tpr;
-        if (more) {
-            const int tn = min(tku + 64, tpr - 1);
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                na[r] = ql[rsb[r] * 8 + (tn >> 1) * 4 + (tn & 1)];
-                nbq[r] = ql[rsb[r] * 8 + (tn >> 1) * 4 + (tn & 1) + 2];
-                nh[r] = qh[rsb[r] * 4 + tn];
-                nsc[r] = sc[rsb[r] * 2 + (tn >> 1)];
-                nd[r] = dsb[rsb[r] + (tn >> 2)];
-            }
-        }
-        // activation: four 16-byte pieces (32-block j of the half, 16-half c), their scales and sums
-        uint4 xv[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) xv[j] = sq[g * 9 + 2 * j + c];
-        const float4 dx4 = sd[g];
-        const int4 sp4 = ss[g];
+    for (int t = 0; t < MT; t++) {
+        const char* tok = smem + t * tokb;
+        const uint4* sq = (const uint4*)tok;
+        const float4 dx4 = ((const float4*)(tok + nsb * 2 * 144))[g];
+        const int4 sp4 = ((const int4*)(tok + nsb * 2 * 160))[g];
         const float dxs[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
         const int sps[4] = {sp4.x, sp4.y, sp4.z, sp4.w};
-        int xs16[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) xs16[j] = c ? (sps[j] >> 16) : (int)(short)(sps[j] & 0xffff);
-#pragma unroll
-        for (int r = 0; r < RPW; r++) {
-            const unsigned a4[4] = {wa[r].x, wa[r].y, wa[r].z, wa[r].w};
-            const unsigned b4[4] = {wb[r].x, wb[r].y, wb[r].z, wb[r].w};
-            const unsigned h4[4] = {wh[r].x, wh[r].y, wh[r].z, wh[r].w};
-            int is[4] = {0, 0, 0, 0};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const unsigned q0 = (a4[i] & 0x0f0f0f0fu) | ((h4[i] << 4) & 0x30303030u);
-                const unsigned q1 = (b4[i] & 0x0f0f0f0fu) | ((h4[i] << 2) & 0x30303030u);
-                const unsigned q2 = ((a4[i] >> 4) & 0x0f0f0f0fu) | (h4[i] & 0x30303030u);
-                const unsigned q3 = ((b4[i] >> 4) & 0x0f0f0f0fu) | ((h4[i] >> 2) & 0x30303030u);
-                const int x0 = (int)(&xv[0].x)[i], x1 = (int)(&xv[1].x)[i], x2 = (int)(&xv[2].x)[i],
-                          x3 = (int)(&xv[3].x)[i];
-                is[0] = dot4((int)q0, x0, is[0]);
-                is[1] = dot4((int)q1, x1, is[1]);
-                is[2] = dot4((int)q2, x2, is[2]);
-                is[3] = dot4((int)q3, x3, is[3]);
+        for (int j = 0; j < 4; j++) {
+            const uint4 xv = sq[g * 9 + 2 * j + c];
+            int is = dot4((int)q[j][0], (int)xv.x, 0);
+            is = dot4((int)q[j][1], (int)xv.y, is);
+            is = dot4((int)q[j][2], (int)xv.z, is);
+            is = dot4((int)q[j][3], (int)xv.w, is);
+            const int xs16 = c ? (sps[j] >> 16) : (int)(short)(sps[j] & 0xffff);
+            const int isum = is - 32 * xs16;  // sum((q-32)x) = sum(qx) - 32 sum(x)
+            if (DUMP) {
+                if (act && t == 0 && dump_row) dump_row[(u >> 2) * 16 + ((u >> 1) & 1) * 8 + 2 * j + c] = isum;
             }
-            const float d = (act && c == 0) ? h2f(wd[r]) : 0.f;  // even lane carries the 32-block
-            const unsigned long long scw = ((unsigned long long)wsc[r].y << 32) | wsc[r].x;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int isum = is[j] - 32 * xs16[j];  // sum((q-32)x) = sum(qx) - 32 sum(x)
-                if (DUMP) {
-                    if (act && row0 + r < N)
-                        dump[(size_t)(row0 + r) * nsb * 16 + (size_t)(tk >> 2) * 16 + ((tk >> 1) & 1) * 8 + 2 * j + c] =
-                            isum;
-                }
-                const int s8 = (int)(signed char)((scw >> (8 * (2 * j + c))) & 0xff);
-                int tj = s8 * isum;
-                tj += swap1(tj);  // both 16-element halves of the 32-block
-                acc[r] += (d * dxs[j]) * (float)tj;
-            }
+            const int s8 = (int)(signed char)((scw >> (8 * (2 * j + c))) & 0xff);
+            int tj = s8 * isum;
+            tj += swap1(tj);
+            acc[t] += (d * dxs[j]) * (float)tj;
         }
-        if (more) {
-#pragma unroll
-            for (int r = 0; r < RPW; r++) {
-                wa[r] = na[r];
-                wb[r] = nbq[r];
-                wh[r] = nh[r];
-                wsc[r] = nsc[r];
-                wd[r] = nd[r];
-            }
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < RPW; r++) {
-        const float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < N) y[row0 + r] = s;
     }
 }
 
+// Stage one activation row into LDS.  8 lanes per 32-block, one float4 / one packed dword each;
+// reductions inside the 8 lanes go over DPP.
+template <class Ops, bool FUSEQ>
+__device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X, int t, bool zero) {
+    const int nb32 = Ops::nb32(nblk);
+    const int items = nb32 * 8;
+    constexpr int SB = 2;  // items per thread requested before any is consumed
+    for (int i0 = threadIdx.x; i0 < items; i0 += blockDim.x * SB) {
+        float4 v[SB];
+        int pk[SB];
+#pragma unroll
+        for (int j = 0; j < SB; j++) {
+            const int i = i0 + j * blockDim.x;
+            const bool live = i < items && !zero;
+            v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            pk[j] = 0;
+            if (FUSEQ) {
+                if (live) v[j] = ((const float4*)(X.x + (size_t)t * nb32 * 32))[i];
+            } else {
+                if (live) pk[j] = ((const int*)(X.xq + (size_t)t * nb32 * 32))[i];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < SB; j++) {
+            const int i = i0 + j * blockDim.x;
+            // whole 8-lane groups are live or not together (items is a multiple of 8)
+            const bool live = i < items;
+            const int blk = i >> 3, sub = i & 7;
+            int packed = pk[j], s_lo = 0, s_hi = 0;
+            float d = 0.f;
+            if (FUSEQ) {
+                const float4 w = v[j];
+                float a = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
+                a = fmaxf(a, dpp_f<0xB1>(a));
+                a = fmaxf(a, dpp_f<0x4E>(a));
+                a = fmaxf(a, dpp_f<0x141>(a));
+                d = a / 127.f;
+                const float inv = d > 0.f ? 1.f / d : 0.f;
+                const int q0 = max(-127, min(127, (int)rintf(w.x * inv)));
+                const int q1 = max(-127, min(127, (int)rintf(w.y * inv)));
+                const int q2 = max(-127, min(127, (int)rintf(w.z * inv)));
+                const int q3 = max(-127, min(127, (int)rintf(w.w * inv)));
+                packed = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+                if (Ops::kNeedsSums) {
+                    int s = q0 + q1 + q2 + q3;
+                    s += dpp_i<0xB1>(s);
+                    s += dpp_i<0x4E>(s);          // sum over this lane's 16-element half
+                    s_lo = s;
+                    s_hi = dpp_i<0x141>(s);       // the other half's sum (valid in lanes 0..3 of the group)
+                }
+            } else if (live && !zero && sub == 0) {
+                d = X.xd[(size_t)t * nb32 + blk];
+                if (Ops::kNeedsSums) {
+                    const int sp = X.xs[(size_t)t * nb32 + blk];
+                    s_lo = (int)(short)(sp & 0xffff);
+                    s_hi = sp >> 16;
+                }
+            }
+            if (live) {
+                *Ops::xq_dword(tok, nblk, blk, sub) = packed;
+                if (sub == 0) Ops::put_scale(tok, nblk, blk, d, s_lo, s_hi);
+            }
+        }
+    }
+}
+
+// Stage m pre-quantised activation rows: every global load of all rows is requested before the
+// first LDS write, so the staging costs one memory round trip, not one per row.
+template <class Ops, int MT>
+__device__ __forceinline__ void stage_prequant_all(char* smem, int tokb, int nblk, const GemvX& X, int m) {
+    const int nb32 = Ops::nb32(nblk);
+    const int items = nb32 * 8;
+    constexpr int SB = 2;
+    for (int i0 = threadIdx.x; i0 < items; i0 += blockDim.x * SB) {
+        int pk[MT][SB], sp[MT][SB];
+        float d[MT][SB];
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int j = 0; j < SB; j++) {
+                const int i = i0 + j * blockDim.x;
+                const bool live = i < items && t < m;
+                pk[t][j] = live ? ((const int*)(X.xq + (size_t)t * nb32 * 32))[i] : 0;
+                const bool head = live && (i & 7) == 0;
+                d[t][j] = head ? X.xd[(size_t)t * nb32 + (i >> 3)] : 0.f;
+                sp[t][j] = (head && Ops::kNeedsSums) ? X.xs[(size_t)t * nb32 + (i >> 3)] : 0;
+            }
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int j = 0; j < SB; j++) {
+                const int i = i0 + j * blockDim.x;
+                if (i < items) {
+                    char* tok = smem + t * tokb;
+                    *Ops::xq_dword(tok, nblk, i >> 3, i & 7) = pk[t][j];
+                    if ((i & 7) == 0)
+                        Ops::put_scale(tok, nblk, i >> 3, d[t][j], (int)(short)(sp[t][j] & 0xffff), sp[t][j] >> 16);
+                }
+            }
+    }
+}
+
+// The GEMV proper.  rows [0, N) of weight W against m <= MT activation rows; y[t*ldy + row].
+//
+// Lane mapping: LPR (16, 32 or 64) lanes walk one row, so a wave serves RS = 64/LPR rows side by
+// side ("slot") and RPW slots per chunk; a row of U units takes ceil(U/LPR) passes.  LPR is chosen
+// by the launcher to waste the fewest lanes (80-unit rows: LPR 16, five full passes for four rows).
+// `wave_id` / `n_waves`: this wave's index among all waves sharing the row range, and their number.
+// KS adjacent waves (same workgroup) form a group that shares each chunk: wave j of the group takes
+// passes j, j+KS, ...; with KS > 1 every group owns at most one chunk (the launcher guarantees
+// nchunks <= n_waves / KS) and the KS partial sums meet in LDS behind the staged activation.
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool FUSEQ, bool DUMP>
+__device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* __restrict__ y, int ldy, int nblk, int N,
+                                          int m, int* __restrict__ dump, int dump_per_row, int wave_id, int n_waves) {
+    extern __shared__ __align__(16) char smem[];
+    SMX_STAMP_DECL;
+    SMX_STAMP(0);
+    constexpr int RS = 64 / LPR;                 // rows side by side in a wave
+    constexpr int RC = RPW * RS;                 // rows per chunk
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & (LPR - 1), rsub = lane / LPR;
+    const int U = Ops::units_per_row(nblk);
+    const int P = (U + LPR - 1) / LPR;           // passes per chunk
+    const int nchunks = (N + RC - 1) / RC;
+    const int group = KS == 1 ? wave_id : wave_id / KS, ks = KS == 1 ? 0 : wave_id % KS;
+    const int n_groups = KS == 1 ? n_waves : n_waves / KS;
+    const int tokb = Ops::tok_bytes(nblk);
+
+    typename Ops::Regs ring[PRE][RPW];
+    // loader cursor (runs PRE items ahead of the consumer)
+    int l_chunk = group, l_pass = ks;
+    if (KS > 1 && l_pass >= P) l_chunk = nchunks;  // more waves in the group than passes
+    auto issue = [&](int slot) {
+        const int u = min(l_pass * LPR + sub, U - 1);
+#pragma unroll
+        for (int r = 0; r < RPW; r++) {
+            const size_t row = (size_t)min(l_chunk * RC + r * RS + rsub, N - 1);
+            Ops::load(ring[slot][r], W, row, nblk, u);
+        }
+        l_pass += KS;
+        if (l_pass >= P) {
+            l_pass = ks;
+            l_chunk += n_groups;
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; k++)
+        if (l_chunk < nchunks) issue(k);
+    SMX_STAMP(1);
+
+    if (FUSEQ) {
+        for (int t = 0; t < MT; t++) stage_token<Ops, true>(smem + t * tokb, nblk, X, t, t >= m);
+    } else {
+        stage_prequant_all<Ops, MT>(smem, tokb, nblk, X, m);
+    }
+    SMX_STAMP(2);
+    __syncthreads();
+    SMX_STAMP(3);
+
+    float acc[RPW][MT];
+#pragma unroll
+    for (int r = 0; r < RPW; r++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[r][t] = 0.f;
+    int c_chunk = group, c_pass = ks;
+    if (KS > 1 && c_pass >= P) c_chunk = nchunks;
+    float* part = (float*)(smem + MT * tokb);  // [waves of the workgroup][RC][MT], KS > 1 only
+    const int wave_in_wg = threadIdx.x >> 6;
+    while (c_chunk < nchunks) {
+#pragma unroll
+        for (int k = 0; k < PRE; k++) {
+            if (c_chunk < nchunks) {
+                const int uu = c_pass * LPR + sub;
+                const bool act = uu < U;
+                const int u = act ? uu : U - 1;
+#pragma unroll
+                for (int r = 0; r < RPW; r++) {
+                    const int row = c_chunk * RC + r * RS + rsub;
+                    int* drow = (DUMP && row < N) ? dump + (size_t)row * dump_per_row : nullptr;
+                    compute_unit<MT, DUMP>(Ops(), ring[k][r], smem, tokb, nblk, u, act, acc[r], drow);
+                }
+                if (l_chunk < nchunks) issue(k);
+                if (k == 0) SMX_STAMP(4);
+                c_pass += KS;
+                if (c_pass >= P) {
+#pragma unroll
+                    for (int r = 0; r < RPW; r++)
+#pragma unroll
+                        for (int t = 0; t < MT; t++) {
+                            const float s = group_sum<LPR>(acc[r][t]);
+                            const int row = c_chunk * RC + r * RS + rsub;
+                            if (sub == LPR - 1) {  // the lane holding the group's total
+                                if (KS == 1) {
+                                    if (row < N && t < m) y[(size_t)t * ldy + row] = s;
+                                } else {
+                                    part[wave_in_wg * (RC * MT) + (r * RS + rsub) * MT + t] = s;
+                                }
+                            }
+                            acc[r][t] = 0.f;
+                        }
+                    c_pass = ks;
+                    c_chunk += n_groups;
+                }
+            }
+        }
+    }
+    if (KS > 1) {
+        __syncthreads();
+        // the group's first wave adds the KS partials in slice order
+        if (ks == 0 && group < nchunks && lane < RC * MT) {
+            const int rr = lane / MT, t = lane % MT;
+            const int row = group * RC + rr;
+            float s = 0.f;
+            for (int j = 0; j < KS && j < P; j++) s += part[(wave_in_wg + j) * (RC * MT) + lane];
+            if (row < N && t < m) y[(size_t)t * ldy + row] = s;
+        }
+    }
+    SMX_STAMP(5);
+    SMX_STAMP_FLUSH();
+}
 
 }  // namespace smx

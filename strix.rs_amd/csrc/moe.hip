@@ -93,23 +93,21 @@ struct MoeRoute {
     float w[64];
 };
 
-template <int RPW>
-__global__ __launch_bounds__(1024) void moe_gemv_q8_kernel(const uint16_t* __restrict__ s0,
-                                                           const uint4* __restrict__ q0,
-                                                           const uint16_t* __restrict__ s1,
-                                                           const uint4* __restrict__ q1,
-                                                           const MoeRoute route, const int8_t* __restrict__ xq,
-                                                           const float* __restrict__ xd, float* __restrict__ y0,
-                                                           float* __restrict__ y1, int nb, int rows, int per_k_x) {
+template <bool FUSEQ>
+__global__ __launch_bounds__(256) void moe_gemv_q8_kernel(const uint16_t* __restrict__ s0, const uint4* __restrict__ q0,
+                                                          const uint16_t* __restrict__ s1, const uint4* __restrict__ q1,
+                                                          const MoeRoute route, const float* __restrict__ x,
+                                                          const int8_t* __restrict__ xq, const float* __restrict__ xd,
+                                                          float* __restrict__ y0, float* __restrict__ y1, int nb, int rows) {
     const int kk = blockIdx.y;
     const size_t ebase = (size_t)route.ids[kk] * rows * nb;  // in blocks
-    const uint16_t* sc = (blockIdx.z ? s1 : s0) + ebase;
-    const uint4* qu = (blockIdx.z ? q1 : q0) + ebase * 2;
+    GemvW W = {(blockIdx.z ? s1 : s0) + ebase, (blockIdx.z ? q1 : q0) + ebase * 2, nullptr, nullptr};
+    // gate/up: every expert reads the token's fp32 row (quantised while staged);
+    // down: one pre-quantised row per routed expert
+    GemvX X = {x, FUSEQ ? nullptr : xq + (size_t)kk * nb * 32, FUSEQ ? nullptr : xd + (size_t)kk * nb, nullptr};
     float* y = (blockIdx.z ? y1 : y0) + (size_t)kk * rows;
-    const int8_t* xqk = per_k_x ? xq + (size_t)kk * nb * 32 : xq;
-    const float* xdk = per_k_x ? xd + (size_t)kk * nb : xd;
-    const int row0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RPW;
-    gemv_q8_0_body<1, RPW, false>(sc, qu, xqk, xdk, y, nb, rows, 1, nullptr, row0);
+    gemv_body<OpsQ8_0, 1, 2, 2, 1, 64, FUSEQ, false>(W, X, y, rows, nb, rows, 1, nullptr, 0,
+                                                 blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
 }
 
 // out[o] = sum_k wexp[k]*dy[k][o], k ascending (kernels.rs:1875-1882)
@@ -137,20 +135,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
     y[(size_t)t * hidden + i] = s;
 }
 
-static int moe_gemv(smx_ctx* c, const Weight& a, const Weight* b, const MoeRoute& route, int k, const int8_t* xq,
-                    const float* xd, float* y0, float* y1, int rows, int per_k_x, const char* name) {
+static int moe_gemv(smx_ctx* c, const Weight& a, const Weight* b, const MoeRoute& route, int k, const float* x,
+                    const int8_t* xq, const float* xd, float* y0, float* y1, int rows, const char* name) {
     const int nb = (int)a.nblk;
     const size_t lds = ((size_t)nb * 36 + 15) & ~size_t(15);
     if (lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "moe: activation of %d blocks does not fit LDS", nb);
-    const int nw = 4, rpw = 2;
-    const unsigned gx = (unsigned)((rows + nw * rpw - 1) / (nw * rpw));
+    const unsigned gx = (unsigned)((rows + 7) / 8);  // 4 waves x 2 rows per workgroup
+    const dim3 grid(gx, (unsigned)k, b ? 2u : 1u);
     ProfScope ps(c, name);
-    auto kern = moe_gemv_q8_kernel<2>;
-    if (lds > 48 * 1024)
-        SMX_HIP(c, hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3(gx, (unsigned)k, b ? 2u : 1u), dim3(nw * 64), lds, c->stream, a.scales,
-                       (const uint4*)a.quants, b ? b->scales : a.scales, (const uint4*)(b ? b->quants : a.quants), route,
-                       xq, xd, y0, y1, nb, rows, per_k_x);
+    const uint16_t* s1 = b ? b->scales : a.scales;
+    const uint4* q1 = (const uint4*)(b ? b->quants : a.quants);
+    if (x) {
+        auto kern = moe_gemv_q8_kernel<true>;
+        static size_t lds_set = 0;
+        int rc = set_dyn_lds(c, kern, lds, &lds_set);
+        if (rc != SMX_OK) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, c->stream, a.scales, (const uint4*)a.quants, s1, q1, route, x, xq, xd,
+                           y0, y1, nb, rows);
+    } else {
+        auto kern = moe_gemv_q8_kernel<false>;
+        static size_t lds_set = 0;
+        int rc = set_dyn_lds(c, kern, lds, &lds_set);
+        if (rc != SMX_OK) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, c->stream, a.scales, (const uint4*)a.quants, s1, q1, route, x, xq, xd,
+                           y0, y1, nb, rows);
+    }
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
@@ -191,9 +200,6 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
             return fail(c, SMX_ERR_ARG, "moe_ffn: expert id %d outside 0..%zu", ids[i], L.ne - 1);
     const size_t hidden = L.hidden, eff = L.eff;
     int rc;
-    if ((rc = ensure(c, c->xq, hidden)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->xd, (hidden / 32) * 4)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->xs, (hidden / 32) * 4)) != SMX_OK) return rc;
     Carver cv;
     const size_t o_g = cv.take(k * eff * 4), o_u = cv.take(k * eff * 4), o_aq = cv.take(k * eff),
                  o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(k * hidden * 4);
@@ -209,14 +215,11 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     s.aq = (int8_t*)(c->work.p + o_aq);
     s.ad = (float*)(c->work.p + o_ad);
     s.dy = (float*)(c->work.p + o_dy);
-    rc = launch_actquant(c, x_dev, 1, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
-    if (rc != SMX_OK) return rc;
-    rc = moe_gemv(c, L.gate, &L.up, route, (int)k, (const int8_t*)c->xq.p, (const float*)c->xd.p, s.g, s.u, (int)eff, 0,
-                  "moe_gemv_gate_up");
+    rc = moe_gemv(c, L.gate, &L.up, route, (int)k, x_dev, nullptr, nullptr, s.g, s.u, (int)eff, "moe_gemv_gate_up");
     if (rc != SMX_OK) return rc;
     rc = silu_mul_quant(c, s.g, s.u, eff, k, eff, s.aq, s.ad);
     if (rc != SMX_OK) return rc;
-    rc = moe_gemv(c, L.down, nullptr, route, (int)k, s.aq, s.ad, s.dy, s.dy, (int)hidden, 1, "moe_gemv_down");
+    rc = moe_gemv(c, L.down, nullptr, route, (int)k, nullptr, s.aq, s.ad, s.dy, s.dy, (int)hidden, "moe_gemv_down");
     if (rc != SMX_OK) return rc;
     {
         ProfScope ps(c, "moe_wsum");

@@ -71,6 +71,11 @@ struct smx_ctx {
     smx::DevBuf work2;
     smx::DevBuf tab;    // small tables (ids, weights, tile tables)
 
+    // tuning overrides (0 = automatic)
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0;
+
+    bool capturing = false;  // between smx_graph_begin and smx_graph_end
+
     // profiling
     bool prof_on = false;
     std::vector<smx::ProfRec> prof;
@@ -90,6 +95,17 @@ int hip_fail(smx_ctx* c, hipError_t e, const char* what);
     } while (0)
 
 int ensure(smx_ctx* c, DevBuf& b, size_t bytes);
+
+// Raises a kernel's dynamic-LDS limit when it asks for more than the 48 KB default (remembered per
+// kernel so that replays and captured launches do not repeat the call).
+template <typename Kern>
+int set_dyn_lds(smx_ctx* c, Kern kern, size_t lds, size_t* cached) {
+    if (lds <= 48 * 1024 || lds <= *cached) return SMX_OK;
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return hip_fail(c, e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    *cached = lds;
+    return SMX_OK;
+}
 
 // Brackets one kernel launch with an event pair when profiling is on.
 struct ProfScope {
@@ -127,9 +143,9 @@ struct GemmArgs {
 // ---- launchers (all enqueue on c->stream; return SMX_OK or an error) ----
 // Activation quantiser: x[m][K] f32 -> xq[m][K], xd[m][K/32], xs[m][K/32] (two i16 sums per block).
 int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, float* xd, int32_t* xs);
-// GEMV: y[m][N], m <= SMX_GEMV_MAX_M (Q6_K: m == 1).  dump (optional): per-block i32 dots of row 0.
-int launch_gemv(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, const int32_t* xs,
-                size_t m, float* y, int32_t* dump);
+// GEMV with the activation quantiser fused into its LDS staging: x fp32 [m][K] -> y[m][N],
+// m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
+int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);
