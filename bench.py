@@ -24,6 +24,9 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+# HBM bytes per launch of the headline kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
+# the same counter's reading for a 256 MiB copy (profiles/gemv_q4_0_9728x2560_hbm_traffic.md)
+HEADLINE_TRAFFIC_BYTES = 14238020
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 Q4_0, Q8_0, Q6_K = 2, 8, 14
 BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q6_K: 210}
@@ -87,6 +90,7 @@ class Bench:
         acc.sync()
         acc.prof_enable(False)
         ms, n = acc.prof_read(prefix)
+        self.last_names = acc.prof_names()
         acc.prof_reset()
         return (ms / n * 1e3 if n else float("nan")), n
 
@@ -120,15 +124,38 @@ class Bench:
         acc.dev_free(xd)
         acc.dev_free(yd)
         gbs = algo * steps / (ms * 1e-3) / 1e9
-        kgbs = algo / (kus * 1e-6) / 1e9
+        # With one activation row the quantiser is fused: a step is exactly one launch of the GEMV
+        # kernel, so the timed region's events give that kernel's average launch duration directly
+        # (an event pair per launch adds about 2 us of its own and is reported separately).
+        single = m == 1
+        launch_us = ms / steps * 1e3 if single else kus
+        kgbs = algo / (launch_us * 1e-6) / 1e9
         return {
             "workload": name, "shape": {"N": N, "K": K, "M": m}, "weight_copies": ncopies,
             "algorithmic_bytes": algo, "weight_bytes": wbytes, "steps": steps, "ms_per_step": ms / steps,
             "wall_ms_per_step": wall_ms / steps, "GBps": gbs, "weight_only_GBps": wbytes * steps / (ms * 1e-3) / 1e9,
             "frac_hbm_peak": gbs / HBM_PEAK_GBS,
-            "kernel": KERNEL[ty], "kernel_avg_us": kus, "kernel_launches": nk, "kernel_GBps": kgbs,
-            "kernel_frac_hbm_peak": kgbs / HBM_PEAK_GBS,
+            "kernel": KERNEL[ty], "kernel_avg_us": launch_us, "kernel_avg_us_event_pair": kus, "kernel_launches": nk,
+            "kernel_GBps": kgbs, "kernel_frac_hbm_peak": kgbs / HBM_PEAK_GBS,
+            "kernel_timing": ("events around the timed region's back-to-back launches / launches" if single
+                              else "event pair around each launch"),
         }
+
+    # ------------------------------------------------------------------ copy (counter calibration)
+    def copy_calib(self, nbytes=256 << 20, steps=20):
+        """A plain copy of known size: what FETCH_SIZE / WRITE_SIZE read for it scales the counters."""
+        acc = self.acc
+        src, dst = acc.dev_alloc(nbytes), acc.dev_alloc(nbytes)
+        acc.h2d(src, np.zeros(1 << 20, np.uint8))
+
+        def step(i):
+            acc.dev_copy(dst, src, nbytes)
+
+        ms, _ = self._timed(step, steps, 2)
+        acc.dev_free(src)
+        acc.dev_free(dst)
+        return {"workload": "copy_calib", "bytes_read": nbytes, "bytes_written": nbytes, "steps": steps,
+                "ms_per_step": ms / steps, "GBps_read_plus_write": 2 * nbytes * steps / (ms * 1e-3) / 1e9}
 
     # ------------------------------------------------------------------ GEMM
     def gemm(self, name, ty, M, N, K, steps=None, warmup=None):
@@ -148,7 +175,7 @@ class Bench:
         ms, wall_ms = self._timed(step, steps, warmup)
         kname = "gemm_i8_q4_0" if ty == Q4_0 else "gemm_i8_q8_0"
         kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
-        names = acc.prof_names()
+        names = self.last_names
         acc.evict(name)
         acc.dev_free(xd)
         acc.dev_free(yd)
@@ -265,6 +292,7 @@ def main():
     work[head["workload"]] = head
     b.log(json.dumps(head))
     plans = [
+        ("copy_calib", lambda: b.copy_calib()),
         ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
         ("q6_k_gemv_15360x3840", lambda: b.gemv("q6_k_gemv_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB))),
@@ -294,9 +322,11 @@ def main():
                                f"({head['weight_copies'] * head['weight_bytes'] / 1e9:.2f} GB); "
                                "step = activation quantiser + GEMV", "frac_hbm_peak": head["frac_hbm_peak"]},
         "roofline": {"bound": "hbm", "achieved": head["kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["kernel_frac_hbm_peak"], "traffic": None, "kernel": head["kernel"],
-                     "kernel_avg_us": head["kernel_avg_us"], "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
-                     "method": "HIP event pair around every GEMV launch on the launch stream, second identical pass"},
+                     "frac": head["kernel_frac_hbm_peak"], "traffic": HEADLINE_TRAFFIC_BYTES, "kernel": head["kernel"],
+                     "kernel_avg_us": head["kernel_avg_us"], "kernel_avg_us_event_pair": head["kernel_avg_us_event_pair"],
+                     "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
+                     "method": "HIP events on the launch stream around the K back-to-back launches of the timed "
+                               "region (one fused quantise+GEMV kernel per step); traffic from rocprofv3 counters"},
         "gemm": None if not best_gemm else {
             "workload": best_gemm["workload"], "value": best_gemm["TOPS"], "unit": "TOPS",
             "frac_int8_mfma_peak": best_gemm["frac_int8_peak"],

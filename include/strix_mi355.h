@@ -118,6 +118,9 @@ int smx_dev_free(smx_ctx* ctx, void* dptr);
 int smx_h2d(smx_ctx* ctx, void* dst_dev, const void* src_host, size_t nbytes);
 int smx_d2h(smx_ctx* ctx, void* dst_host, const void* src_dev, size_t nbytes); /* syncs */
 int smx_sync(smx_ctx* ctx);
+/* Plain device-to-device copy kernel (nbytes a multiple of 16, 16-byte aligned pointers), async.
+ * Also the known-size reference kernel against which hardware traffic counters are scaled. */
+int smx_dev_copy(smx_ctx* ctx, void* dst_dev, const void* src_dev, size_t nbytes);
 int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 int smx_gemm_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,

@@ -31,7 +31,7 @@ EXPORTS = [
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
-    "smx_graph_destroy",
+    "smx_graph_destroy", "smx_dev_copy",
 ]
 
 
@@ -82,6 +82,7 @@ def load_library():
     L.smx_h2d.argtypes = [vp, vp, vp, sz]
     L.smx_d2h.argtypes = [vp, vp, vp, sz]
     L.smx_sync.argtypes = [vp]
+    L.smx_dev_copy.argtypes = [vp, vp, vp, sz]
     L.smx_gemv_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemm_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
@@ -290,6 +291,9 @@ class Mi355WeightAccel:
     def d2h(self, arr, dptr):
         self._check(self._L.smx_d2h(self._h, _p(arr), dptr, arr.nbytes))
         return arr
+
+    def dev_copy(self, dst, src, nbytes):
+        self._check(self._L.smx_dev_copy(self._h, dst, src, nbytes))
 
     def sync(self):
         self._check(self._L.smx_sync(self._h))

@@ -5,6 +5,8 @@
 // Layout differs: quants stay contiguous int8 [m][K]; the block sum the reference keeps per 32
 // (kernels.rs:93) is kept as two 16-element sums packed in one dword, which also serves the
 // 16-wide sub-blocks of Q6_K.
+#include <algorithm>
+
 #include "smx_internal.h"
 
 namespace smx {
@@ -54,4 +56,22 @@ int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, 
     return SMX_OK;
 }
 
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256) dst[i] = src[i];
+}
+
 }  // namespace smx
+
+extern "C" int smx_dev_copy(smx_ctx* c, void* dst, const void* src, size_t nbytes) {
+    using namespace smx;
+    if (!c) return SMX_ERR_ARG;
+    if (!dst || !src || nbytes % 16 != 0 || ((uintptr_t)dst | (uintptr_t)src) % 16 != 0)
+        return fail(c, SMX_ERR_ARG, "dev_copy: pointers and size must be 16-byte aligned");
+    if (nbytes == 0) return SMX_OK;
+    const size_t n16 = nbytes / 16;
+    const unsigned grid = (unsigned)std::min<size_t>((n16 + 255) / 256, (size_t)c->num_cu * 32);
+    ProfScope ps(c, "copy");
+    hipLaunchKernelGGL(copy_kernel, dim3(grid), dim3(256), 0, c->stream, (const uint4*)src, (uint4*)dst, n16);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
