@@ -27,7 +27,20 @@ def build(verbose=False, extra=()):
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+    build_selftest()
     return LIB
+
+
+def build_selftest():
+    """The C++ mirror of the accelerator trait and its driver program (host compiler only)."""
+    host = os.path.join(HERE, "host")
+    exe = os.path.join(host, "selftest")
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-Wextra", os.path.join(host, "selftest.cpp"), "-o", exe,
+           "-L" + HERE, "-lstrix_mi355", "-Wl,-rpath," + HERE, "-Wl,-rpath,/opt/rocm/lib", "-L/opt/rocm/lib"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("g++ failed on host/selftest.cpp:\n" + proc.stdout)
+    return exe
 
 
 if __name__ == "__main__":

@@ -50,3 +50,14 @@ def test_missing_library_is_an_error_not_a_fallback(pkg, monkeypatch):
     monkeypatch.setattr(pkg, "LIB_PATH", os.path.join(ROOT, "does", "not", "exist.so"))
     with pytest.raises(FileNotFoundError):
         pkg.load_library()
+
+
+def test_cpp_mirror_builds_and_declines_without_gpu():
+    import subprocess
+    if os.path.exists("/dev/kfd"):
+        pytest.skip("a GPU is present")
+    exe = os.path.join(ROOT, "strix.rs_amd", "host", "selftest")
+    if not os.path.exists(exe):
+        pytest.skip("host/selftest not built")
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert r.returncode == 77 and "no HIP device" in r.stdout

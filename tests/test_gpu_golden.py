@@ -34,3 +34,14 @@ def test_literal_blocks_through_the_device(accel, golden):
             x[i] = 1.0
             y = accel.gemv("t.lit", x, 1)[0]
             assert abs(y - g[name + "_out"][i]) <= 1e-5 * max(1.0, abs(g[name + "_out"][i]))
+
+
+def test_cpp_mirror_of_the_trait_selftest():
+    """host/selftest drives strix::Mi355WeightAccel (the C++ restatement of the WeightAccel trait)."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "strix.rs_amd", "host", "selftest")
+    assert os.path.exists(exe), "build it with python strix.rs_amd/build.py"
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout
+    assert "selftest ok" in r.stdout
