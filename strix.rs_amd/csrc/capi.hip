@@ -75,9 +75,10 @@ int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, f
 int matmul_host(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, float* y, size_t y_cap,
                 bool force_gemm, const char* who) {
     if (!c) return SMX_ERR_ARG;
-    if (!key || !xs || !y) return fail(c, SMX_ERR_ARG, "%s: null argument", who);
+    if (!key) return fail(c, SMX_ERR_ARG, "%s: null key", who);
     const Weight* w = find_weight(c, key);
-    if (!w) return SMX_NOT_RESIDENT;
+    if (!w) return SMX_NOT_RESIDENT;  // a decline comes before any look at the buffers (the caller may not know out_dim)
+    if (!xs || !y) return fail(c, SMX_ERR_ARG, "%s: null argument", who);
     if (in_dim != w->K) return fail(c, SMX_ERR_ARG, "%s: activation length %zu, weight in_dim %zu", who, in_dim, w->K);
     if (m == 0) return fail(c, SMX_ERR_ARG, "%s: zero rows", who);
     if (y_cap < m * w->N) return fail(c, SMX_ERR_ARG, "%s: output capacity %zu < %zu", who, y_cap, m * w->N);

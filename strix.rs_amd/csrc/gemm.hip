@@ -79,17 +79,17 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
     const int q_bi = lane >> 4, q_rowlo = lane & 15;
     const bool nb4 = (p.nb & 3) == 0;  // whole stages only, scale rows 8/16-byte aligned
     // per-thread row bases (fixed for the whole K loop)
-    size_t a_off[4], b_off[4];
+    unsigned a_off[4], b_off[4];  // element offsets; the launcher keeps M*K and N*K below 2^31
 #pragma unroll
     for (int ps = 0; ps < 4; ps++) {
         const int r = (ps * 4 + wave) * 8 + g_rowlo;
         const int ti = min(tok0 + r, M_end - 1);
-        a_off[ps] = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * K;
+        a_off[ps] = (unsigned)(p.a_rowmap ? p.a_rowmap[ti] : ti) * (unsigned)K;
         if (!Q4) {
-            b_off[ps] = (size_t)min(row0 + r, N_end - 1) * K;
+            b_off[ps] = (unsigned)min(row0 + r, N_end - 1) * (unsigned)K;
         } else if (ps < 2) {
             const int rq = (ps * 4 + wave) * 16 + q_rowlo;
-            b_off[ps] = (size_t)min(row0 + rq, N_end - 1) * p.nb;
+            b_off[ps] = (unsigned)min(row0 + rq, N_end - 1) * (unsigned)p.nb;
         }
     }
     // scales: thread (sr, sh) carries blocks 2*sh, 2*sh+1 of the stage for weight row sr and token sr
@@ -266,7 +266,8 @@ static int pick_splitk(const smx_ctx* c, int tiles, int nstages) {
 
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y, int32_t* dump) {
     if (w.type != kQ4_0 && w.type != kQ8_0) return fail(c, SMX_ERR_ARG, "gemm: weight type %d not supported", (int)w.type);
-    if (m > (size_t(1) << 24) || w.N > (size_t(1) << 24) || w.K > (size_t(1) << 20))
+    if (m > (size_t(1) << 24) || w.N > (size_t(1) << 24) || w.K > (size_t(1) << 20) || m * w.K >= (size_t(1) << 31) ||
+        w.N * w.K >= (size_t(1) << 31))
         return fail(c, SMX_ERR_LIMIT, "gemm: shape m=%zu N=%zu K=%zu exceeds the kernel's index range", m, w.N, w.K);
     GemmArgs p = {};
     p.op[0].wscales = w.scales;

@@ -316,7 +316,9 @@ int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const siz
     const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
     if (m == 0 || slots == 0) return fail(c, SMX_ERR_ARG, "moe_layer: m %zu, slots %zu", m, slots);  // decode.rs:1622
     if (y_cap < m * hidden) return fail(c, SMX_ERR_ARG, "moe_layer: output capacity %zu < %zu", y_cap, m * hidden);
-    if (slots > (size_t(1) << 24) || m > 65535) return fail(c, SMX_ERR_LIMIT, "moe_layer: m %zu / slots %zu exceed the launch limits", m, slots);
+    if (slots > (size_t(1) << 24) || m > 65535 || m * hidden >= (size_t(1) << 31) || slots * eff >= (size_t(1) << 31) ||
+        L.ne * eff * hidden >= (size_t(1) << 31))
+        return fail(c, SMX_ERR_LIMIT, "moe_layer: m %zu / slots %zu exceed the launch limits", m, slots);
     // the plan must tile [0, slots) with in-range experts; every slot's token must exist
     size_t covered = 0;
     for (size_t i = 0; i < nplan; i++) {

@@ -1,0 +1,126 @@
+"""Device-resident entry points, graph capture, tuning knobs, timing, copy kernel."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_dev_entry_points_match_host_ones(accel, synth):
+    N, K, m = 640, 2560, 5
+    raw = synth.make_weight(8, N, K, seed=1)
+    assert accel.upload_q8_0("t.dev", raw, K, N)
+    xs = synth.make_acts(m, K, seed=2)
+    xd, yd = accel.dev_alloc(xs.nbytes), accel.dev_alloc(m * N * 4)
+    accel.h2d(xd, xs)
+    assert accel.gemv_dev("t.dev", xd, m, yd)
+    got = accel.d2h(np.empty((m, N), np.float32), yd)
+    assert np.array_equal(got, accel.gemv_rows("t.dev", xs, N))
+    assert accel.gemm_dev("t.dev", xd, m, yd)
+    got = accel.d2h(np.empty((m, N), np.float32), yd)
+    assert np.array_equal(got, accel.prefill_q8_gemm("t.dev", xs, m, N))
+    assert accel.gemv_dev("t.absent", xd, 1, yd) is False
+    accel.dev_free(xd)
+    accel.dev_free(yd)
+
+
+def test_graph_replays_equal_eager(accel, synth):
+    """A captured chain of GEMV, GEMM and MoE-decode launches, replayed several times with eager work and
+    synchronisations in between, must reproduce the eager results every time."""
+    N, K = 512, 1024
+    raw4, raw8 = synth.make_weight(2, N, K, seed=3), synth.make_weight(8, K, N, seed=4)
+    assert accel.upload_q4_0("t.g4", raw4, K, N) and accel.upload_q8_0("t.g8", raw8, N, K)
+    gate, up, down = synth.make_moe_q8(8, K, 96, seed=5)
+    assert accel.upload_moe_q8(31, gate, up, down, K, 96, 8)
+    ids, w = synth.zipf_routing(1, 8, 2, seed=6)
+    x = synth.make_acts(4, K, seed=7)
+    xd = accel.dev_alloc(x.nbytes)
+    h1, h2, h3, h4 = (accel.dev_alloc(4 * max(N, K) * 4) for _ in range(4))
+    accel.h2d(xd, x)
+
+    def chain():
+        accel.gemv_dev("t.g4", xd, 1, h1)          # K -> N
+        accel.gemv_dev("t.g8", h1, 1, h2)          # N -> K  (dependent)
+        accel.moe_ffn_dev(31, ids[0], w[0], h2, h3)
+        accel.gemm_dev("t.g4", xd, 4, h4)
+
+    def read():
+        return [accel.d2h(np.empty(n, np.float32), p) for p, n in ((h1, N), (h2, K), (h3, K), (h4, 4 * N))]
+
+    chain()
+    eager = read()
+    accel.graph_begin()
+    chain()
+    g = accel.graph_end()
+    for rep in range(4):
+        for p in (h1, h2, h3, h4):
+            accel.h2d(p, np.zeros(4 * max(N, K), np.float32))     # eager work between replays
+        accel.gemv_dev("t.g8", xd, 1, h1)                         # an unrelated eager launch
+        accel.sync()
+        accel.graph_launch(g)
+        accel.sync()
+        for a, b in zip(read(), eager):
+            assert np.array_equal(a, b), f"replay {rep}"
+    accel.graph_destroy(g)
+    for p in (xd, h1, h2, h3, h4):
+        accel.dev_free(p)
+
+
+def test_capture_refuses_scratch_growth(accel, synth, pkg):
+    raw = synth.make_weight(8, 128, 4096, seed=8)
+    assert accel.upload_q8_0("t.grow", raw, 4096, 128)
+    m = 40000                                     # 164 MB of int8 rows: larger than any scratch grown so far
+    xd, yd = accel.dev_alloc(m * 4096 * 4), accel.dev_alloc(m * 128 * 4)
+    accel.graph_begin()
+    with pytest.raises(pkg.SmxError):
+        accel.gemm_dev("t.grow", xd, m, yd)
+    g = accel.graph_end()
+    accel.graph_destroy(g)
+    accel.dev_free(xd)
+    accel.dev_free(yd)
+
+
+def test_tuning_knobs_keep_results(accel, orc, synth, relerr, pkg):
+    N, K = 1000, 2560
+    for ty, up in ((2, accel.upload_q4_0), (8, accel.upload_q8_0), (14, accel.upload_q6_k)):
+        raw = synth.make_weight(ty, N, K, seed=ty)
+        x = synth.make_acts(1, K, seed=9)
+        assert up("t.tune", raw, K, N)
+        ref = orc.matmul_q8_from_f32(ty, raw, K, N, x)[0]
+        for knobs in ({"gemv_lpr": 16}, {"gemv_lpr": 32, "gemv_rpw": 2}, {"gemv_lpr": 64, "gemv_rpw": 4},
+                      {"gemv_lpr": 64, "gemv_ks": 2}, {"gemv_lpr": 64, "gemv_ks": 4}, {"gemv_wpc": 2}):
+            for k, v in knobs.items():
+                accel.tune(k, v)
+            assert relerr(accel.gemv("t.tune", x, N), ref) <= 1e-5, knobs
+            for k in knobs:
+                accel.tune(k, 0)
+    raw = synth.make_weight(8, 256, 4096, seed=11)
+    xs = synth.make_acts(64, 4096, seed=12)
+    assert accel.upload_q8_0("t.tune", raw, 4096, 256)
+    ref = orc.matmul_q8_from_f32(8, raw, 4096, 256, xs)
+    for sk in (1, 2, 4, 8):
+        accel.tune("gemm_splitk", sk)
+        assert relerr(accel.prefill_q8_gemm("t.tune", xs, 64, 256), ref) <= 1e-5
+    accel.tune("gemm_splitk", 0)
+    with pytest.raises(pkg.SmxError):
+        accel.tune("no_such_knob", 1)
+    with pytest.raises(pkg.SmxError):
+        accel.tune("gemv_lpr", 48)
+
+
+def test_copy_kernel_and_profiling(accel, synth):
+    a = np.random.default_rng(0).integers(0, 255, 1 << 20, dtype=np.uint8)
+    s, d = accel.dev_alloc(a.nbytes), accel.dev_alloc(a.nbytes)
+    accel.h2d(s, a)
+    accel.prof_reset()
+    accel.prof_enable(True)
+    accel.timer_begin()
+    accel.dev_copy(d, s, a.nbytes)
+    ms = accel.timer_end()
+    accel.prof_enable(False)
+    assert np.array_equal(accel.d2h(np.empty_like(a), d), a)
+    tot, n = accel.prof_read("copy")
+    assert n == 1 and 0 < tot <= ms * 1.5 + 0.1 and "copy" in accel.prof_names()
+    accel.prof_reset()
+    assert accel.prof_read("copy")[1] == 0
+    accel.dev_free(s)
+    accel.dev_free(d)
