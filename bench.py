@@ -141,6 +141,45 @@ class Bench:
                               else "event pair around each launch"),
         }
 
+    # ------------------------------------------------------------------ grouped GEMV (one launch, G weights)
+    def gemv_group(self, name, ty, N, K, G, min_total_bytes, steps=None, warmup=None):
+        """G single-token GEMVs of the same shape in one launch (the gate+up pair of a decode step for
+        G = 2), rotating through >= 1 GB of weight copies; a step is one launch."""
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
+        algo1, wbytes = gemv_bytes(ty, N, K, 1)
+        ncopies = max(2 * G, -(-min_total_bytes // wbytes))
+        ncopies = -(-ncopies // G) * G
+        src = [sy.make_weight(ty, N, K, seed=1000 + i) for i in range(2)]
+        keys = []
+        for i in range(ncopies):
+            key = f"{name}.w{i}"
+            assert getattr(acc, UPLOAD[ty])(key, src[i % 2], K, N)
+            keys.append(key)
+        del src
+        x = sy.make_acts(1, K, seed=7)
+        xd = acc.dev_alloc(x.nbytes)
+        acc.h2d(xd, x)
+        yds = [acc.dev_alloc(N * 4) for _ in range(G)]
+        ngroups = ncopies // G
+
+        def step(i):
+            g0 = (i % ngroups) * G
+            acc.gemv_batch_dev(keys[g0:g0 + G], [xd] * G, yds)
+
+        ms, wall_ms = self._timed(step, steps, warmup)
+        for k in keys:
+            acc.evict(k)
+        acc.dev_free(xd)
+        for p in yds:
+            acc.dev_free(p)
+        algo = algo1 * G
+        gbs = algo * steps / (ms * 1e-3) / 1e9
+        return {"workload": name, "shape": {"N": N, "K": K, "M": 1, "weights_per_launch": G}, "weight_copies": ncopies,
+                "algorithmic_bytes": algo, "steps": steps, "ms_per_step": ms / steps, "GBps": gbs,
+                "frac_hbm_peak": gbs / HBM_PEAK_GBS, "kernel": KERNEL[ty], "kernel_avg_us": ms / steps * 1e3,
+                "kernel_GBps": gbs, "kernel_frac_hbm_peak": gbs / HBM_PEAK_GBS}
+
     # ------------------------------------------------------------------ copy (counter calibration)
     def copy_calib(self, nbytes=256 << 20, steps=20):
         """A plain copy of known size: what FETCH_SIZE / WRITE_SIZE read for it scales the counters."""
@@ -293,6 +332,8 @@ def main():
     b.log(json.dumps(head))
     plans = [
         ("copy_calib", lambda: b.copy_calib()),
+        ("q4_0_gemv_9728x2560_gate_up_pair", lambda: b.gemv_group("q4_0_gemv_9728x2560_gate_up_pair", Q4_0, 9728, 2560, 2, int(1.1 * GB))),
+        ("q4_0_gemv_9728x2560_batch8", lambda: b.gemv_group("q4_0_gemv_9728x2560_batch8", Q4_0, 9728, 2560, 8, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
         ("q6_k_gemv_15360x3840", lambda: b.gemv("q6_k_gemv_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB))),

@@ -122,6 +122,10 @@ int smx_sync(smx_ctx* ctx);
  * Also the known-size reference kernel against which hardware traffic counters are scaled. */
 int smx_dev_copy(smx_ctx* ctx, void* dst_dev, const void* src_dev, size_t nbytes);
 int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
+/* Up to 8 single-row GEMVs of one format and in_dim in ONE launch (gate+up, q/k/v, a batch of
+ * weights against their activations); 0 if any key is not resident. */
+int smx_gemv_batch_dev(smx_ctx* ctx, size_t n, const char* const* keys, const float* const* xs_dev,
+                       float* const* ys_dev);
 int smx_gemm_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                     const float* x_dev, float* y_dev);

@@ -31,7 +31,7 @@ EXPORTS = [
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
-    "smx_graph_destroy", "smx_dev_copy",
+    "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev",
 ]
 
 
@@ -85,6 +85,7 @@ def load_library():
     L.smx_dev_copy.argtypes = [vp, vp, vp, sz]
     L.smx_gemv_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemm_dev.argtypes = [vp, cp, vp, sz, vp]
+    L.smx_gemv_batch_dev.argtypes = [vp, sz, vp, vp, vp]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_prof_enable.argtypes = [vp, i]
     L.smx_prof_reset.argtypes = [vp]
@@ -300,6 +301,13 @@ class Mi355WeightAccel:
 
     def gemv_dev(self, key, xs_dev, m, y_dev):
         return self._check(self._L.smx_gemv_dev(self._h, key.encode(), xs_dev, m, y_dev))
+
+    def gemv_batch_dev(self, keys, xs_dev, ys_dev):
+        n = len(keys)
+        k = (C.c_char_p * n)(*[s.encode() for s in keys])
+        xp = (C.c_void_p * n)(*xs_dev)
+        yp = (C.c_void_p * n)(*ys_dev)
+        return self._check(self._L.smx_gemv_batch_dev(self._h, n, k, xp, yp))
 
     def gemm_dev(self, key, xs_dev, m, y_dev):
         return self._check(self._L.smx_gemm_dev(self._h, key.encode(), xs_dev, m, y_dev))

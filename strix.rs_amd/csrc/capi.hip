@@ -144,28 +144,36 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
     int rc;
     if ((rc = ensure(c, c->xf32, xbytes)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->yf32, ybytes)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->xq, qbytes)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->xd, dbytes)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->xs, dbytes)) != SMX_OK) return rc;
-    size_t xo = 0, yo = 0, qo = 0, dofs = 0;
+    (void)qbytes; (void)dbytes;
+    size_t xo = 0, yo = 0;
     std::vector<size_t> yoff(n, 0);
+    std::vector<float*> xdev(n, nullptr), ydev(n, nullptr);
     for (size_t i = 0; i < n; i++) {
         const Weight* w = ws[i];
         if (!w) continue;
-        float* xdv = (float*)(c->xf32.p + xo);
-        int8_t* q = (int8_t*)(c->xq.p + qo);
-        float* d = (float*)(c->xd.p + dofs);
-        int32_t* s = (int32_t*)(c->xs.p + dofs);
-        float* yd = (float*)(c->yf32.p + yo);
+        xdev[i] = (float*)(c->xf32.p + xo);
+        ydev[i] = (float*)(c->yf32.p + yo);
         yoff[i] = yo;
-        SMX_HIP(c, hipMemcpyAsync(xdv, xs[i], w->K * 4, hipMemcpyHostToDevice, c->stream));
-        (void)q; (void)d; (void)s;
-        rc = launch_gemv(c, *w, xdv, 1, yd, nullptr);
-        status[i] = rc;
+        SMX_HIP(c, hipMemcpyAsync(xdev[i], xs[i], w->K * 4, hipMemcpyHostToDevice, c->stream));
         xo += (w->K * 4 + 255) & ~size_t(255);
         yo += (w->N * 4 + 255) & ~size_t(255);
-        qo += (w->K + 255) & ~size_t(255);
-        dofs += ((w->K / 32) * 4 + 255) & ~size_t(255);
+    }
+    // consecutive items of one format and row length share a launch (up to 8 per launch)
+    for (size_t i = 0; i < n;) {
+        if (!ws[i]) { i++; continue; }
+        const Weight* gw[8];
+        const float* gx[8];
+        float* gy[8];
+        size_t idx[8];
+        int g = 0;
+        size_t j = i;
+        while (j < n && g < 8 && ws[j] && ws[j]->type == ws[i]->type && ws[j]->K == ws[i]->K) {
+            gw[g] = ws[j]; gx[g] = xdev[j]; gy[g] = ydev[j]; idx[g] = j;
+            g++; j++;
+        }
+        rc = launch_gemv_group(c, gw, gx, gy, g);
+        for (int k = 0; k < g; k++) status[idx[k]] = rc;
+        i = j;
     }
     for (size_t i = 0; i < n; i++)
         if (ws[i] && status[i] == SMX_OK)
@@ -216,6 +224,19 @@ int smx_gemv_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, flo
     if (!w) return SMX_NOT_RESIDENT;
     if (m == 0 || m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv_dev: %zu rows (1..%d)", m, SMX_GEMV_MAX_M);
     return run_matmul_dev(c, *w, xs_dev, m, y_dev, false, nullptr);
+}
+
+int smx_gemv_batch_dev(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs_dev, float* const* ys_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!keys || !xs_dev || !ys_dev) return fail(c, SMX_ERR_ARG, "gemv_batch_dev: null argument");
+    if (n == 0 || n > 8) return fail(c, SMX_ERR_LIMIT, "gemv_batch_dev: %zu items (1..8 per launch)", n);
+    const Weight* ws[8];
+    for (size_t i = 0; i < n; i++) {
+        if (!keys[i] || !xs_dev[i] || !ys_dev[i]) return fail(c, SMX_ERR_ARG, "gemv_batch_dev: item %zu has a null pointer", i);
+        ws[i] = find_weight(c, keys[i]);
+        if (!ws[i]) return SMX_NOT_RESIDENT;
+    }
+    return launch_gemv_group(c, ws, xs_dev, ys_dev, (int)n);
 }
 
 int smx_gemm_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, float* y_dev) {

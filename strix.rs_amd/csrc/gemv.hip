@@ -16,11 +16,25 @@
 
 namespace smx {
 
+// One launch serves up to 8 independent GEMVs of the same format and row length (blockIdx.y picks
+// the job): the gate/up pair or the q/k/v triple of a decode step, or a caller's batch of (key, x)
+// pairs, share one kernel start-up.
+struct GemvJob {
+    GemvW W;
+    GemvX X;
+    float* y;
+    int N;
+};
+struct GemvJobs {
+    GemvJob job[8];
+};
+
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool FUSEQ, bool DUMP, int NT>
-__global__ __launch_bounds__(NT) void gemv_kernel(GemvW W, GemvX X, float* __restrict__ y, int nblk, int N, int m,
-                                                  int* __restrict__ dump, int dump_per_row) {
+__global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, int m, int* __restrict__ dump,
+                                                  int dump_per_row) {
     const int nw = NT / 64;
-    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FUSEQ, DUMP>(W, X, y, N, nblk, N, m, dump, dump_per_row,
+    const GemvJob& jb = J.job[blockIdx.y];
+    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FUSEQ, DUMP>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
@@ -34,14 +48,14 @@ struct Geom {
 };
 
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool DUMP, int NT>
-int launch_one(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float* y, int nblk, int N, int m, int* dump,
+int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump,
                int dump_per_row) {
     // one activation row: quantiser fused into the staging; several rows: staged from rows quantised once
     auto k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, MT == 1, DUMP, NT>;
     static size_t lds_set = 0;
     int rc = set_dyn_lds(c, k, g.lds, &lds_set);
     if (rc != SMX_OK) return rc;
-    hipLaunchKernelGGL(k, dim3(g.grid), dim3(NT), g.lds, c->stream, W, X, y, nblk, N, m, dump, dump_per_row);
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(NT), g.lds, c->stream, J, nblk, m, dump, dump_per_row);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
@@ -50,37 +64,37 @@ int launch_one(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float*
 //   whole-wave rows   (4,2,1,64) (2,2,1,64) (1,4,1,64) (1,2,2,64) (1,2,4,64)
 //   sub-wave rows     (2,2,1,32) (1,2,1,32) (2,2,1,16) (1,2,1,16)        [one activation row only]
 template <class Ops, int MT>
-int launch_variant(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float* y, int nblk, int N, int m) {
+int launch_variant(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m) {
     // sub-wave rows: the pipeline is deep enough to put a whole short row set in flight before the
     // activation is staged (Q6_K units are three times as wide, so half the depth)
     constexpr bool kWide = sizeof(typename Ops::Regs) > 32;
     if (MT == 1 && g.lpr == 32) {
-        if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 32, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
-        return launch_one<Ops, 1, 1, kWide ? 2 : 4, 1, 32, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+        if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+        return launch_one<Ops, 1, 1, kWide ? 2 : 4, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
     }
     if (MT == 1 && g.lpr == 16) {
-        if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 16, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
-        return launch_one<Ops, 1, 1, kWide ? 4 : 6, 1, 16, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+        if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 16, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+        return launch_one<Ops, 1, 1, kWide ? 4 : 6, 1, 16, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
     }
-    if (g.ks == 4) return launch_one<Ops, MT, 1, 2, 4, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
-    if (g.ks == 2) return launch_one<Ops, MT, 1, 2, 2, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
-    if (g.rpw == 1) return launch_one<Ops, MT, 1, 4, 1, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
-    if (g.rpw == 4 && MT == 1) return launch_one<Ops, 1, 4, 2, 1, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
-    return launch_one<Ops, MT, 2, 2, 1, 64, false, 1024>(c, g, W, X, y, nblk, N, m, nullptr, 0);
+    if (g.ks == 4) return launch_one<Ops, MT, 1, 2, 4, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+    if (g.ks == 2) return launch_one<Ops, MT, 1, 2, 2, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+    if (g.rpw == 1) return launch_one<Ops, MT, 1, 4, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+    if (g.rpw == 4 && MT == 1) return launch_one<Ops, 1, 4, 2, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+    return launch_one<Ops, MT, 2, 2, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
 }
 
 template <class Ops>
-int launch_type(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float* y, int nblk, int N, int m, int mt,
+int launch_type(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int mt,
                 int* dump, int dump_per_row) {
     if (dump) {
-        if (g.lpr == 16) return launch_one<Ops, 1, 1, 2, 1, 16, true, 256>(c, g, W, X, y, nblk, N, m, dump, dump_per_row);
-        return launch_one<Ops, 1, 1, 4, 1, 64, true, 256>(c, g, W, X, y, nblk, N, m, dump, dump_per_row);
+        if (g.lpr == 16) return launch_one<Ops, 1, 1, 2, 1, 16, true, 256>(c, g, J, njobs, nblk, m, dump, dump_per_row);
+        return launch_one<Ops, 1, 1, 4, 1, 64, true, 256>(c, g, J, njobs, nblk, m, dump, dump_per_row);
     }
     switch (mt) {
-        case 1: return launch_variant<Ops, 1>(c, g, W, X, y, nblk, N, m);
-        case 2: return launch_variant<Ops, 2>(c, g, W, X, y, nblk, N, m);
-        case 4: return launch_variant<Ops, 4>(c, g, W, X, y, nblk, N, m);
-        default: return launch_variant<Ops, 8>(c, g, W, X, y, nblk, N, m);
+        case 1: return launch_variant<Ops, 1>(c, g, J, njobs, nblk, m);
+        case 2: return launch_variant<Ops, 2>(c, g, J, njobs, nblk, m);
+        case 4: return launch_variant<Ops, 4>(c, g, J, njobs, nblk, m);
+        default: return launch_variant<Ops, 8>(c, g, J, njobs, nblk, m);
     }
 }
 
@@ -91,7 +105,7 @@ int launch_type(smx_ctx* c, const Geom& g, const GemvW& W, const GemvX& X, float
 // per 16 waves), persistent workgroups looping over chunks, lanes-per-row chosen to waste the fewest
 // lanes on short rows, and for weights with few, long rows the passes of a row are split over 2 or
 // 4 waves (K-split) so every SIMD has work.
-static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int mt, bool dump) {
+static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int mt, bool dump, int njobs) {
     Geom g;
     size_t tokb, units;
     if (type == kQ4_0) { tokb = (nblk * 40 + 15) & ~size_t(15); units = nblk; }
@@ -100,7 +114,8 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     g.nt = 1024;
     g.lpr = 64;
     g.ks = 1;
-    const size_t waves = (size_t)c->num_cu * 16;
+    const size_t cus = std::max<size_t>(1, (size_t)c->num_cu / njobs);  // this job's share of the chip
+    const size_t waves = cus * 16;
     // lanes per row: fewest wasted lanes, whole-wave rows on ties (short rows, one activation row only)
     if (mt == 1 && units < 256) {
         size_t best = ((units + 63) / 64) * 64;
@@ -150,9 +165,23 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     } else {
         int wpc = c->tune_gemv_wpc > 0 ? c->tune_gemv_wpc : 1;
         if (dump) wpc = 8;
-        g.grid = (unsigned)std::min<size_t>(wgs, (size_t)c->num_cu * wpc);
+        g.grid = (unsigned)std::min<size_t>(wgs, cus * wpc);
     }
     return g;
+}
+
+static int launch_jobs(smx_ctx* c, QType type, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int mt,
+                       int32_t* dump, int dump_per_row) {
+    if (type == kQ4_0) {
+        ProfScope ps(c, "gemv_q4_0");
+        return launch_type<OpsQ4_0>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
+    }
+    if (type == kQ8_0) {
+        ProfScope ps(c, "gemv_q8_0");
+        return launch_type<OpsQ8_0>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
+    }
+    ProfScope ps(c, "gemv_q6_k");
+    return launch_type<OpsQ6_K>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
 }
 
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump) {
@@ -165,11 +194,14 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
         return launch_gemv(c, w, x + 4 * w.K, m - 4, y + 4 * w.N, nullptr);
     }
     const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8));
-    const Geom g = pick_geom(c, w.type, w.N, w.nblk, mt, dump != nullptr);
+    const Geom g = pick_geom(c, w.type, w.N, w.nblk, mt, dump != nullptr, 1);
     if (g.lds > 160 * 1024)
         return fail(c, SMX_ERR_LIMIT, "gemv: %zu activation rows of %zu need %zu bytes of LDS (limit 163840)", m, w.K, g.lds);
-    GemvW W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
-    GemvX X = {x, nullptr, nullptr, nullptr};
+    GemvJobs J = {};
+    J.job[0].W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
+    J.job[0].X = {x, nullptr, nullptr, nullptr};
+    J.job[0].y = y;
+    J.job[0].N = (int)w.N;
     if (mt > 1) {
         // each of the persistent workgroups would repeat the quantiser for all m rows: do it once instead
         int rc;
@@ -178,19 +210,31 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
         if ((rc = ensure(c, c->xs, m * (w.K / 32) * 4)) != SMX_OK) return rc;
         rc = launch_actquant(c, x, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
         if (rc != SMX_OK) return rc;
-        X = {nullptr, (const int8_t*)c->xq.p, (const float*)c->xd.p, (const int*)c->xs.p};
+        J.job[0].X = {nullptr, (const int8_t*)c->xq.p, (const float*)c->xd.p, (const int*)c->xs.p};
     }
-    const int nblk = (int)w.nblk, N = (int)w.N;
-    if (w.type == kQ4_0) {
-        ProfScope ps(c, "gemv_q4_0");
-        return launch_type<OpsQ4_0>(c, g, W, X, y, nblk, N, (int)m, mt, dump, (int)(w.K / 32));
+    return launch_jobs(c, w.type, g, J, 1, (int)w.nblk, (int)m, mt, dump, (int)(w.type == kQ6_K ? w.K / 16 : w.K / 32));
+}
+
+// n <= 8 single-row GEMVs of one format and row length in one launch.
+int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n) {
+    if (n < 1 || n > 8) return fail(c, SMX_ERR_ARG, "gemv group of %d", n);
+    size_t maxN = 0;
+    GemvJobs J = {};
+    for (int i = 0; i < n; i++) {
+        const Weight& w = *ws[i];
+        if (w.type != ws[0]->type || w.K != ws[0]->K) return fail(c, SMX_ERR_ARG, "gemv group mixes formats or row lengths");
+        if (w.N > 0x7fffffffu / 4 || w.K > (size_t(1) << 20))
+            return fail(c, SMX_ERR_LIMIT, "gemv: shape %zu x %zu exceeds the kernel's index range", w.N, w.K);
+        maxN = std::max(maxN, w.N);
+        J.job[i].W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
+        J.job[i].X = {xs[i], nullptr, nullptr, nullptr};
+        J.job[i].y = ys[i];
+        J.job[i].N = (int)w.N;
     }
-    if (w.type == kQ8_0) {
-        ProfScope ps(c, "gemv_q8_0");
-        return launch_type<OpsQ8_0>(c, g, W, X, y, nblk, N, (int)m, mt, dump, (int)(w.K / 32));
-    }
-    ProfScope ps(c, "gemv_q6_k");
-    return launch_type<OpsQ6_K>(c, g, W, X, y, nblk, N, (int)m, mt, dump, (int)(w.K / 16));
+    const Weight& w0 = *ws[0];
+    Geom g = pick_geom(c, w0.type, maxN, w0.nblk, 1, false, n);
+    if (g.lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "gemv: activation of %zu needs %zu bytes of LDS", w0.K, g.lds);
+    return launch_jobs(c, w0.type, g, J, n, (int)w0.nblk, 1, 1, nullptr, 0);
 }
 
 }  // namespace smx

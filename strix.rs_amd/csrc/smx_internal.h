@@ -146,6 +146,8 @@ int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, 
 // GEMV with the activation quantiser fused into its LDS staging: x fp32 [m][K] -> y[m][N],
 // m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);
+// n <= 8 single-row GEMVs of one format and row length in one launch (device pointers).
+int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);

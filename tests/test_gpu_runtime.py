@@ -124,3 +124,29 @@ def test_copy_kernel_and_profiling(accel, synth):
     assert accel.prof_read("copy")[1] == 0
     accel.dev_free(s)
     accel.dev_free(d)
+
+
+def test_grouped_gemv_launch(accel, orc, synth, relerr):
+    """gemv_batch puts items of one format and row length in one launch (q/k/v: same K, different N)."""
+    K = 2560
+    for ty, up in ((2, accel.upload_q4_0), (8, accel.upload_q8_0), (14, accel.upload_q6_k)):
+        Ns = [4096, 1024, 1024, 9728, 130]
+        raws = [synth.make_weight(ty, n, K, seed=ty * 10 + i) for i, n in enumerate(Ns)]
+        for i, (n, r) in enumerate(zip(Ns, raws)):
+            assert up(f"t.grp{i}", r, K, n)
+        xs = [synth.make_acts(1, K, seed=70 + i)[0] for i in range(len(Ns))]
+        out = accel.gemv_batch([(f"t.grp{i}", xs[i]) for i in range(len(Ns))], Ns)
+        for i, n in enumerate(Ns):
+            assert relerr(out[i], orc.matmul_q8_from_f32(ty, raws[i], K, n, xs[i])[0]) <= 1e-5
+            assert np.array_equal(out[i], accel.gemv(f"t.grp{i}", xs[i], n)) or relerr(out[i], accel.gemv(f"t.grp{i}", xs[i], n)) <= 1e-5
+    # device-pointer form: gate + up share the activation
+    xd = accel.dev_alloc(K * 4)
+    accel.h2d(xd, xs[0])
+    y0, y1 = accel.dev_alloc(4096 * 4), accel.dev_alloc(9728 * 4)
+    assert accel.gemv_batch_dev(["t.grp0", "t.grp3"], [xd, xd], [y0, y1])
+    a = accel.d2h(np.empty(4096, np.float32), y0)
+    b = accel.d2h(np.empty(9728, np.float32), y1)
+    assert relerr(a, accel.gemv("t.grp0", xs[0], 4096)) <= 1e-5 and relerr(b, accel.gemv("t.grp3", xs[0], 9728)) <= 1e-5
+    assert accel.gemv_batch_dev(["t.grp0", "t.absent"], [xd, xd], [y0, y1]) is False
+    for p in (xd, y0, y1):
+        accel.dev_free(p)
