@@ -317,6 +317,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-headline", action="store_true", help="skip the headline GEMV when --only names other workloads")
+    ap.add_argument("--tune", default="", help="launch-geometry overrides for sweeps, e.g. gemm_nw=4,gemm_splitk=2")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X "
@@ -325,11 +327,17 @@ def main():
     want = lambda n: not only or n in only
     b = Bench(a.steps, a.warmup)
     b.log("device:", b.acc.name())
+    for kv in filter(None, a.tune.split(",")):
+        knob, value = kv.split("=")
+        b.acc.tune(knob, int(value))
     GB = 1 << 30
     work = {}
-    head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB))
-    work[head["workload"]] = head
-    b.log(json.dumps(head))
+    if a.no_headline and only:
+        head = None
+    else:
+        head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB))
+        work[head["workload"]] = head
+        b.log(json.dumps(head))
     plans = [
         ("copy_calib", lambda: b.copy_calib()),
         ("q4_0_gemv_9728x2560_gate_up_pair", lambda: b.gemv_group("q4_0_gemv_9728x2560_gate_up_pair", Q4_0, 9728, 2560, 2, int(1.1 * GB))),
@@ -351,6 +359,9 @@ def main():
             r = fn()
             work[name] = r
             b.log(json.dumps(r))
+    if head is None:  # sweep mode: per-workload records only, no headline line
+        print(json.dumps({"workloads": work}), flush=True)
+        return
     gemms = [w for n, w in work.items() if n.startswith("gemm_")]
     best_gemm = max(gemms, key=lambda w: w["TOPS"]) if gemms else None
     line = {

@@ -407,6 +407,9 @@ int smx_tune(smx_ctx* c, const char* knob, int value) {
     } else if (k == "gemm_splitk") {
         if (value > 16) return fail(c, SMX_ERR_ARG, "tune: gemm_splitk must be 0..16");
         c->tune_gemm_splitk = value;
+    } else if (k == "gemm_nw") {
+        if (value != 0 && value != 4 && value != 8) return fail(c, SMX_ERR_ARG, "tune: gemm_nw must be 0, 4 or 8");
+        c->tune_gemm_nw = value;
     } else {
         return fail(c, SMX_ERR_ARG, "tune: unknown knob %s", knob);
     }

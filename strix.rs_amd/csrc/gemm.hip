@@ -27,26 +27,51 @@ namespace smx {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, KB = 4;
-constexpr int HPLANE = 528;                 // bytes between the two k-halves of a fragment (512 + 16 pad)
-constexpr int FRAG = 1040;                  // one 32 x 32 int8 fragment
-constexpr int A_BYTES = KB * 4 * FRAG;      // 4 token tiles
-constexpr int B_BYTES = KB * 4 * FRAG;      // 4 row tiles
-constexpr int S_BYTES = KB * 128 * 4;       // one scale plane
-constexpr int STAGE_BYTES = A_BYTES + B_BYTES + 2 * S_BYTES;
+constexpr int BN = 128, KB = 4;
+constexpr int GRP = 1024;                   // 8 rows x 128 B of one stage: row r at r * 128, its 16-byte chunk c at slot (c + r) % 8
+constexpr int B_BYTES = 16 * GRP;           // 128 weight rows
+// A workgroup of NW waves covers 32 * NW tokens x 128 weight rows (NW = 8: 256 x 128, one workgroup
+// per CU; NW = 4: 128 x 128, two per CU).  The larger tile reads 25 % fewer operand bytes per
+// operation through L2, which is what bounds the kernel after the epilogue FMAs.
+constexpr int a_bytes(int NW) { return 4 * NW * GRP; }
+constexpr int stage_bytes(int NW) { return a_bytes(NW) + B_BYTES + KB * 128 * 4 + KB * 32 * NW * 4; }
 constexpr float MAGIC_F = 12582912.f;       // 1.5 * 2^23
 constexpr int MAGIC_I = 0x4B400000;
 
 __device__ __forceinline__ float h2f_(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 __device__ __forceinline__ unsigned sub8(unsigned x) { return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
 
-// (moved to smx_internal.h: GemmOperand, GemmTile, GemmArgs)
+// 64 lanes x 16 bytes from global memory straight into LDS (no register round trip): lane i's
+// bytes land at LDS byte address lds_base + 16 * i; lds_base is wave-uniform (M0).  Completion is
+// counted by vmcnt.  Written as inline assembly so that the compiler's wait-count insertion does
+// not put vmcnt(0) in front of every later LDS read (it cannot tell the two stage buffers apart);
+// the kernel waits for vmcnt(0) itself before the barrier that publishes a stage.
+__device__ __forceinline__ void load_to_lds16(const void* g, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_base), "v"(g)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
+}
 
-template <bool Q4, bool DUMP>
-__global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
+struct GemmFrag {
+    v4i a;         // this wave's 32 tokens x 32 k
+    v4i b[4];      // 4 x (32 weight rows x 32 k)
+    float4 dx[4];  // activation scales of the 16 tokens this lane accumulates
+    float dw[4];   // weight scale of this lane's row in each of the 4 row tiles
+};
+
+template <bool Q4, bool DUMP, int NW>
+__global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmArgs p) {
+    constexpr int BM = 32 * NW, A_BYTES = a_bytes(NW), STAGE_BYTES = stage_bytes(NW);
+    constexpr int BG = 16 / NW;  // 8-row groups of B each wave stages
+    constexpr int WS = 8 / NW;   // weight scales per thread per stage
     extern __shared__ __align__(16) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = p.nb * 32;
+    const unsigned smem_base = lds_addr(smem);
 
     // tile coordinates; consecutive logical tiles share a weight strip, and each XCD (blockIdx % 8)
     // gets a contiguous range of logical tiles so its L2 holds few strips
@@ -67,107 +92,96 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
     const int s_begin = blockIdx.z * p.stages_per_slice;
     const int s_end = min(nstage_total, s_begin + p.stages_per_slice);
 
-    // ---- global -> register staging: branch-free (clamped addresses, masks applied when the
-    //      registers are written to LDS) so the loads of stage s+1 stay in flight during stage s ----
-    uint4 ra[4], rb[4];
-    unsigned rsw;  // raw weight scales: two f16 (blocks 2*sh, 2*sh+1 of the stage) of row sr
-    uint2 rsx;     // raw activation scales: two f32 of token sr
-    // A (and Q8_0 B): lane = [chunk_hi:2][row_lo:3][chunk_lo:1], 8 rows x 128 B per wave load
-    const int g_chunk = ((lane >> 4) << 1) | (lane & 1);  // 16-byte chunk 0..7 within the 128-byte stage row
-    const int g_rowlo = (lane >> 1) & 7;
-    // Q4_0 B: lane = [bi:2][row_lo:4]
-    const int q_bi = lane >> 4, q_rowlo = lane & 15;
-    const bool nb4 = (p.nb & 3) == 0;  // whole stages only, scale rows 8/16-byte aligned
-    // per-thread row bases (fixed for the whole K loop)
-    unsigned a_off[4], b_off[4];  // element offsets; the launcher keeps M*K and N*K below 2^31
+    // ---- staging.  int8 operands go global -> LDS directly, one 8-row x 128-byte group per wave
+    //      instruction, lane = [row:3][slot:3]: the 8 lanes of a row fetch its whole 128-byte line
+    //      (scattered 16-byte fetches run at a fraction of the L2 -> CU rate), and lane (r, slot)
+    //      fetches chunk (slot - r) % 8, so that chunk c of the 8 rows of a group lies in 8 different
+    //      bank groups and every MFMA fragment read below is a conflict-free 128-bit load.
+    //      Rows past the tile's end and blocks past K re-read valid memory (clamped addresses) and
+    //      are neutralised by zero scales.  Q4_0 weights pass through registers to be widened. ----
+    const int g_rowlo = lane >> 3, g_chunk = ((lane & 7) - g_rowlo) & 7;
+    const int q_bi = lane & 3, q_rowlo = lane >> 2;   // Q4_0 B: lane = [row:4][block:2], 64 contiguous bytes per row
+    constexpr int QG = Q4 ? 8 / NW : 1;  // Q4_0 B: 16-byte blocks per thread per stage
+    unsigned a_off[4], b_off[Q4 ? QG : BG];  // element offsets; the launcher keeps M*K and N*K below 2^31
 #pragma unroll
     for (int ps = 0; ps < 4; ps++) {
-        const int r = (ps * 4 + wave) * 8 + g_rowlo;
-        const int ti = min(tok0 + r, M_end - 1);
+        const int ti = min(tok0 + (ps * NW + wave) * 8 + g_rowlo, M_end - 1);
         a_off[ps] = (unsigned)(p.a_rowmap ? p.a_rowmap[ti] : ti) * (unsigned)K;
-        if (!Q4) {
-            b_off[ps] = (unsigned)min(row0 + r, N_end - 1) * (unsigned)K;
-        } else if (ps < 2) {
-            const int rq = (ps * 4 + wave) * 16 + q_rowlo;
-            b_off[ps] = (unsigned)min(row0 + rq, N_end - 1) * (unsigned)p.nb;
-        }
     }
-    // scales: thread (sr, sh) carries blocks 2*sh, 2*sh+1 of the stage for weight row sr and token sr
-    const int sr = tid & 127, sh = tid >> 7;
-    const bool w_valid = row0 + sr < N_end, x_valid = tok0 + sr < M_end;
-    const size_t scw_base = (size_t)min(row0 + sr, N_end - 1) * p.nb;
+    if (!Q4) {
+#pragma unroll
+        for (int ps = 0; ps < BG; ps++)
+            b_off[ps] = (unsigned)min(row0 + (ps * NW + wave) * 8 + g_rowlo, N_end - 1) * (unsigned)K;
+    } else {
+#pragma unroll
+        for (int ps = 0; ps < QG; ps++)
+            b_off[ps] = (unsigned)min(row0 + (ps * NW + wave) * 16 + q_rowlo, N_end - 1) * (unsigned)p.nb;
+    }
+    // scales: thread (sr, sh) carries blocks 2*sh, 2*sh+1 of the stage for token sr, and thread
+    // (wr, wh) blocks wh*WS .. wh*WS+WS-1 for weight row wr
+    const int sr = tid & (BM - 1), sh = tid / BM;
+    const int wr = tid & 127, wh = tid >> 7;
+    const bool w_valid = row0 + wr < N_end, x_valid = tok0 + sr < M_end;
+    const size_t scw_base = (size_t)min(row0 + wr, N_end - 1) * p.nb;
     size_t scx_base;
     {
         const int ti = min(tok0 + sr, M_end - 1);
         scx_base = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * p.nb;
     }
+    uint4 rb[QG];       // Q4_0 only
+    uint16_t rsw[WS];   // raw weight scales (f16), row wr
+    float rsx0, rsx1;   // activation scales of blocks 2*sh, 2*sh+1, token sr
 
-    auto load_stage = [&](int s) {
+    // issue every global read of stage s; the register-staged parts are written by finish_stage
+    // all global reads of stage s (issuing them piecemeal between the blocks measures slower)
+    auto issue_stage = [&](int buf, int s) {
+        const unsigned sA = __builtin_amdgcn_readfirstlane(smem_base + buf * STAGE_BYTES + wave * GRP);
+        const unsigned sB = sA + A_BYTES;
         const int blk0 = s * KB;
-        const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);  // clamped: a K tail is zeroed at store time
+        const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
 #pragma unroll
-        for (int ps = 0; ps < 4; ps++) {
-            ra[ps] = *(const uint4*)(p.xq + a_off[ps] + koff);
-            if (!Q4) rb[ps] = *(const uint4*)((const int8_t*)op.wquants + b_off[ps] + koff);
-        }
-        if (Q4) {
+        for (int ps = 0; ps < 4; ps++) load_to_lds16(p.xq + a_off[ps] + koff, sA + ps * NW * GRP);
+        if (!Q4) {
+#pragma unroll
+            for (int ps = 0; ps < BG; ps++)
+                load_to_lds16((const int8_t*)op.wquants + b_off[ps] + koff, sB + ps * NW * GRP);
+        } else {
             const int bq = min(blk0 + q_bi, p.nb - 1);
 #pragma unroll
-            for (int ps = 0; ps < 2; ps++) rb[ps] = ((const uint4*)op.wquants)[b_off[ps] + bq];
+            for (int ps = 0; ps < QG; ps++) rb[ps] = ((const uint4*)op.wquants)[b_off[ps] + bq];
         }
-        if (nb4) {
-            rsw = *(const unsigned*)(op.wscales + scw_base + blk0 + 2 * sh);
-            rsx = *(const uint2*)(p.xd + scx_base + blk0 + 2 * sh);
-        } else {
-            const int b0 = min(blk0 + 2 * sh, p.nb - 1), b1 = min(blk0 + 2 * sh + 1, p.nb - 1);
-            rsw = (unsigned)op.wscales[scw_base + b0] | ((unsigned)op.wscales[scw_base + b1] << 16);
-            rsx = make_uint2(__float_as_uint(p.xd[scx_base + b0]), __float_as_uint(p.xd[scx_base + b1]));
-        }
+        // branch-free and unconverted, so that nothing here waits for a load before the MFMA work
+#pragma unroll
+        for (int j = 0; j < WS; j++) rsw[j] = op.wscales[scw_base + min(blk0 + wh * WS + j, p.nb - 1)];
+        rsx0 = p.xd[scx_base + min(blk0 + 2 * sh, p.nb - 1)];
+        rsx1 = p.xd[scx_base + min(blk0 + 2 * sh + 1, p.nb - 1)];
     };
 
-    auto store_stage = [&](int buf, int s) {
-        char* sA = smem + buf * STAGE_BYTES;
-        char* sB = sA + A_BYTES;
+    auto finish_stage = [&](int buf, int s) {
+        char* sB = smem + buf * STAGE_BYTES + A_BYTES;
         float* sdw = (float*)(sB + B_BYTES);
         float* sdx = sdw + KB * 128;
         const int blk0 = s * KB;
-        const bool tail = blk0 + KB > p.nb;  // uniform: only the last stage of a K that is not a stage multiple
-#pragma unroll
-        for (int ps = 0; ps < 4; ps++) {
-            const int r = (ps * 4 + wave) * 8 + g_rowlo;
-            const int off = ((g_chunk >> 1) * 4 + (r >> 5)) * FRAG + (g_chunk & 1) * HPLANE + (r & 31) * 16;
-            uint4 va = ra[ps], vb = rb[ps];
-            if (tail && blk0 + (g_chunk >> 1) >= p.nb) {
-                va = make_uint4(0, 0, 0, 0);
-                vb = va;
-            }
-            *(uint4*)(sA + off) = va;
-            if (!Q4) *(uint4*)(sB + off) = vb;
-        }
         if (Q4) {
 #pragma unroll
-            for (int ps = 0; ps < 2; ps++) {
-                const int r = (ps * 4 + wave) * 16 + q_rowlo;
-                const int off = (q_bi * 4 + (r >> 5)) * FRAG + (r & 31) * 16;
+            for (int ps = 0; ps < QG; ps++) {
+                const int r = (ps * NW + wave) * 16 + q_rowlo;
+                const int off = (r >> 3) * GRP + (r & 7) * 128;  // + slot * 16
                 const uint4 q = rb[ps];
                 uint4 lo, hi;
                 lo.x = sub8(q.x & 0x0f0f0f0fu); hi.x = sub8((q.x >> 4) & 0x0f0f0f0fu);
                 lo.y = sub8(q.y & 0x0f0f0f0fu); hi.y = sub8((q.y >> 4) & 0x0f0f0f0fu);
                 lo.z = sub8(q.z & 0x0f0f0f0fu); hi.z = sub8((q.z >> 4) & 0x0f0f0f0fu);
                 lo.w = sub8(q.w & 0x0f0f0f0fu); hi.w = sub8((q.w >> 4) & 0x0f0f0f0fu);
-                if (tail && blk0 + q_bi >= p.nb) {
-                    lo = make_uint4(0, 0, 0, 0);
-                    hi = lo;
-                }
-                *(uint4*)(sB + off) = lo;            // elements 0..15 of the block
-                *(uint4*)(sB + off + HPLANE) = hi;   // elements 16..31
+                *(uint4*)(sB + off + ((2 * q_bi + r) & 7) * 16) = lo;      // elements 0..15 of the block
+                *(uint4*)(sB + off + ((2 * q_bi + 1 + r) & 7) * 16) = hi;  // elements 16..31
             }
         }
-        const bool v0 = blk0 + 2 * sh < p.nb, v1 = blk0 + 2 * sh + 1 < p.nb;
-        sdw[(2 * sh) * 128 + sr] = (w_valid && v0) ? h2f_((uint16_t)(rsw & 0xffff)) : 0.f;
-        sdw[(2 * sh + 1) * 128 + sr] = (w_valid && v1) ? h2f_((uint16_t)(rsw >> 16)) : 0.f;
-        sdx[(2 * sh) * 128 + sr] = (x_valid && v0) ? __uint_as_float(rsx.x) : 0.f;
-        sdx[(2 * sh + 1) * 128 + sr] = (x_valid && v1) ? __uint_as_float(rsx.y) : 0.f;
+#pragma unroll
+        for (int j = 0; j < WS; j++)
+            sdw[(wh * WS + j) * 128 + wr] = (w_valid && blk0 + wh * WS + j < p.nb) ? h2f_(rsw[j]) : 0.f;
+        sdx[(2 * sh) * BM + sr] = (x_valid && blk0 + 2 * sh < p.nb) ? rsx0 : 0.f;
+        sdx[(2 * sh + 1) * BM + sr] = (x_valid && blk0 + 2 * sh + 1 < p.nb) ? rsx1 : 0.f;
     };
 
     float acc[4][16];
@@ -179,52 +193,90 @@ __global__ __launch_bounds__(256, 2) void gemm_i8_kernel(GemmArgs p) {
 #pragma unroll
     for (int i = 0; i < 16; i++) cmagic[i] = MAGIC_I;
 
-    const int frag_lane = (lane >> 5) * HPLANE + (lane & 31) * 16;
     const int half = lane >> 5, col = lane & 31;
+    // fragment (tile, block bi): lane -> row lane % 32 of the tile, k-half lane / 32
+    int frag_lane[KB];
+#pragma unroll
+    for (int bi = 0; bi < KB; bi++) frag_lane[bi] = (col >> 3) * GRP + (col & 7) * 128 + ((2 * bi + half + col) & 7) * 16;
 
-    if (s_begin < s_end) {
-        load_stage(s_begin);
-        store_stage(0, s_begin);
-    }
-    __syncthreads();
-    for (int s = s_begin; s < s_end; s++) {
-        const int buf = (s - s_begin) & 1;
-        if (s + 1 < s_end) load_stage(s + 1);
+    auto read_frag = [&](GemmFrag& f, int buf, int bi) {
         const char* sA = smem + buf * STAGE_BYTES;
         const char* sB = sA + A_BYTES;
         const float* sdw = (const float*)(sB + B_BYTES);
         const float* sdx = sdw + KB * 128;
-#pragma unroll 1
-        for (int bi = 0; bi < KB; bi++) {
-            const v4i a = *(const v4i*)(sA + (bi * 4 + wave) * FRAG + frag_lane);
-            float dxr[16];
+        f.a = *(const v4i*)(sA + wave * 4 * GRP + frag_lane[bi]);
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4 v = *(const float4*)(sdx + bi * 128 + wave * 32 + g * 8 + half * 4);
-                dxr[g * 4 + 0] = v.x; dxr[g * 4 + 1] = v.y; dxr[g * 4 + 2] = v.z; dxr[g * 4 + 3] = v.w;
+        for (int g = 0; g < 4; g++) f.dx[g] = *(const float4*)(sdx + bi * BM + wave * 32 + g * 8 + half * 4);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+            f.b[nt] = *(const v4i*)(sB + nt * 4 * GRP + frag_lane[bi]);
+            f.dw[nt] = sdw[bi * 128 + nt * 32 + col];
+        }
+    };
+
+    // One block: 4 MFMAs, each followed by its 32 epilogue FMAs; MFMA nt + 1 is issued before the
+    // FMAs of nt so that the matrix pipe and the vector ALU overlap within the wave.  The empty asm
+    // statements pin the order: without them the FMAs of a whole stage sink below its 16 MFMAs,
+    // whose results (256 registers) then spill.
+    auto compute = [&](const GemmFrag& f, int blk) {
+        const float dxr[16] = {f.dx[0].x, f.dx[0].y, f.dx[0].z, f.dx[0].w, f.dx[1].x, f.dx[1].y, f.dx[1].z, f.dx[1].w,
+                               f.dx[2].x, f.dx[2].y, f.dx[2].z, f.dx[2].w, f.dx[3].x, f.dx[3].y, f.dx[3].z, f.dx[3].w};
+        v16i d[2];
+        d[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a, f.b[0], cmagic, 0, 0, 0);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+            if (nt + 1 < 4) {
+                d[(nt + 1) & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a, f.b[nt + 1], cmagic, 0, 0, 0);
+                asm volatile("" : "+v"(d[(nt + 1) & 1]));
             }
+            const v16i dn = d[nt & 1];
+            const float dw = f.dw[nt];
+            const float ndw = -dw * MAGIC_F;  // exact: dw has an 11-bit significand
 #pragma unroll
-            for (int nt = 0; nt < 4; nt++) {
-                const v4i b = *(const v4i*)(sB + (bi * 4 + nt) * FRAG + frag_lane);
-                const float dw = sdw[bi * 128 + nt * 32 + col];
-                const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, cmagic, 0, 0, 0);
-                const float ndw = -dw * MAGIC_F;  // exact: dw has an 11-bit significand
+            for (int i = 0; i < 16; i++) acc[nt][i] = fmaf(dxr[i], fmaf(dw, __int_as_float(dn[i]), ndw), acc[nt][i]);
+            asm volatile("" : "+v"(acc[nt][0]), "+v"(acc[nt][1]), "+v"(acc[nt][2]), "+v"(acc[nt][3]), "+v"(acc[nt][4]),
+                              "+v"(acc[nt][5]), "+v"(acc[nt][6]), "+v"(acc[nt][7]), "+v"(acc[nt][8]), "+v"(acc[nt][9]),
+                              "+v"(acc[nt][10]), "+v"(acc[nt][11]), "+v"(acc[nt][12]), "+v"(acc[nt][13]),
+                              "+v"(acc[nt][14]), "+v"(acc[nt][15]));
+            if (DUMP) {
+                const int row = row0 + nt * 32 + col;
 #pragma unroll
-                for (int i = 0; i < 16; i++)
-                    acc[nt][i] = fmaf(dxr[i], fmaf(dw, __int_as_float(d[i]), ndw), acc[nt][i]);
-                if (DUMP) {
-                    const int blk = s * KB + bi;
-                    const int row = row0 + nt * 32 + col;
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const int tok = tok0 + wave * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-                        if (tok < M_end && row < N_end && blk < p.nb)
-                            p.dump[((size_t)tok * p.N + row) * p.nb + blk] = d[i] - MAGIC_I;
-                    }
+                for (int i = 0; i < 16; i++) {
+                    const int tok = tok0 + wave * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                    if (tok < M_end && row < N_end && blk < p.nb)
+                        p.dump[((size_t)tok * p.N + row) * p.nb + blk] = dn[i] - MAGIC_I;
                 }
             }
         }
-        if (s + 1 < s_end) store_stage(buf ^ 1, s + 1);
+    };
+
+    if (s_begin < s_end) {
+        issue_stage(0, s_begin);
+        finish_stage(0, s_begin);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int s = s_begin; s < s_end; s++) {
+        const int buf = (s - s_begin) & 1;
+        if (s + 1 < s_end) issue_stage(buf ^ 1, s + 1);
+        GemmFrag f0, f1;
+        read_frag(f0, buf, 0);
+        read_frag(f1, buf, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(f0, s * KB + 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frag(f0, buf, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(f1, s * KB + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frag(f1, buf, 3);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(f0, s * KB + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(f1, s * KB + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        if (s + 1 < s_end) finish_stage(buf ^ 1, s + 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
@@ -254,14 +306,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4* __rest
 }
 
 // Split-K factor: the reference splits only the long-K shapes (in_dim >= 12288, decode.rs:5658) to
-// fill its grid; here: split when the tile grid alone leaves most of the 2-per-CU workgroup slots
-// empty, into whole stages, and never so far that a slice has fewer than 8 stages.
-static int pick_splitk(const smx_ctx* c, int tiles, int nstages) {
-    const int slots = c->num_cu * 2;
+// fill its grid; here: split when the tile grid alone leaves most of the workgroup slots empty,
+// into whole stages, and never so far that a slice has fewer than 8 stages.
+static int pick_splitk(int slots, int tiles, int nstages) {
     if (tiles * 2 > slots) return 1;
     int z = (slots + tiles - 1) / tiles;
     z = std::min(z, std::max(1, nstages / 8));
     return std::min(z, 16);
+}
+
+template <bool Q4, bool DUMP, int NW>
+static int launch_gemm_variant(smx_ctx* c, const GemmArgs& p, dim3 grid) {
+    auto k = gemm_i8_kernel<Q4, DUMP, NW>;
+    static size_t lds_set = 0;
+    const size_t lds = 2 * stage_bytes(NW);
+    int rc = set_dyn_lds(c, k, lds, &lds_set);
+    if (rc != SMX_OK) return rc;
+    hipLaunchKernelGGL(k, grid, dim3(64 * NW), lds, c->stream, p);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
 }
 
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y, int32_t* dump) {
@@ -281,12 +344,17 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     p.N = (int)w.N;
     p.ldo = (int)w.N;
     p.nb = (int)w.nblk;
-    p.tiles_m = (p.M + BM - 1) / BM;
+    // 128 x 128 tiles, two workgroups per CU; 256 x 128 (one 8-wave workgroup per CU) measures slower
+    int nw = 4;
+    if (c->tune_gemm_nw == 4 || c->tune_gemm_nw == 8) nw = c->tune_gemm_nw;
+    const int bm = 32 * nw;
+    p.tiles_m = (p.M + bm - 1) / bm;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int T = p.tiles_m * p.tiles_n;
     p.xcd_remap = (T % 8 == 0) ? 1 : 0;
     const int nstages = (p.nb + KB - 1) / KB;
-    int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(c, T, nstages));
+    const int slots = c->num_cu * (nw == 8 ? 1 : 2);
+    int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(slots, T, nstages));
     p.stages_per_slice = (nstages + Z - 1) / Z;
     Z = (nstages + p.stages_per_slice - 1) / p.stages_per_slice;
     p.op[0].out = y;
@@ -295,24 +363,18 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
         if (rc != SMX_OK) return rc;
         p.op[0].out = (float*)c->work.p;
     }
-    const size_t lds = 2 * STAGE_BYTES;
     const dim3 grid((unsigned)T, 1, (unsigned)Z);
     {
         ProfScope ps(c, w.type == kQ4_0 ? "gemm_i8_q4_0" : "gemm_i8_q8_0");
-#define LAUNCH_GEMM(Q4, DUMP)                                                                              \
-    do {                                                                                                   \
-        auto k = gemm_i8_kernel<Q4, DUMP>;                                                                 \
-        static size_t lds_set = 0;                                                                         \
-        int rc_ = set_dyn_lds(c, k, lds, &lds_set);                                                        \
-        if (rc_ != SMX_OK) return rc_;                                                                     \
-        hipLaunchKernelGGL(k, grid, dim3(256), lds, c->stream, p);                                         \
-    } while (0)
+        int rc;
         if (w.type == kQ4_0) {
-            if (dump) LAUNCH_GEMM(true, true); else LAUNCH_GEMM(true, false);
+            if (dump) rc = nw == 8 ? launch_gemm_variant<true, true, 8>(c, p, grid) : launch_gemm_variant<true, true, 4>(c, p, grid);
+            else rc = nw == 8 ? launch_gemm_variant<true, false, 8>(c, p, grid) : launch_gemm_variant<true, false, 4>(c, p, grid);
         } else {
-            if (dump) LAUNCH_GEMM(false, true); else LAUNCH_GEMM(false, false);
+            if (dump) rc = nw == 8 ? launch_gemm_variant<false, true, 8>(c, p, grid) : launch_gemm_variant<false, true, 4>(c, p, grid);
+            else rc = nw == 8 ? launch_gemm_variant<false, false, 8>(c, p, grid) : launch_gemm_variant<false, false, 4>(c, p, grid);
         }
-        SMX_HIP(c, hipGetLastError());
+        if (rc != SMX_OK) return rc;
     }
     if (Z > 1) {
         const size_t n = m * w.N;
@@ -328,15 +390,8 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
 // one of `nops` weight/output pairs that share the activation rows (gate and up).
 int launch_gemm_grouped(smx_ctx* c, const GemmArgs& args, int ntiles, int nops, const char* name) {
     if (ntiles <= 0) return SMX_OK;
-    const size_t lds = 2 * STAGE_BYTES;
     ProfScope ps(c, name);
-    auto k = gemm_i8_kernel<false, false>;
-    static size_t lds_set = 0;
-    int rc = set_dyn_lds(c, k, lds, &lds_set);
-    if (rc != SMX_OK) return rc;
-    hipLaunchKernelGGL(k, dim3((unsigned)ntiles, (unsigned)nops, 1), dim3(256), lds, c->stream, args);
-    SMX_HIP(c, hipGetLastError());
-    return SMX_OK;
+    return launch_gemm_variant<false, false, 4>(c, args, dim3((unsigned)ntiles, (unsigned)nops, 1));
 }
 
 }  // namespace smx

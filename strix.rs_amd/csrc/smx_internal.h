@@ -72,7 +72,7 @@ struct smx_ctx {
     smx::DevBuf tab;    // small tables (ids, weights, tile tables)
 
     // tuning overrides (0 = automatic)
-    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0;
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
 
     bool capturing = false;  // between smx_graph_begin and smx_graph_end
 
