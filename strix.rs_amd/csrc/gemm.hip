@@ -192,6 +192,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     v16i cmagic;
 #pragma unroll
     for (int i = 0; i < 16; i++) cmagic[i] = MAGIC_I;
+    asm volatile("" : "+v"(cmagic));  // keep the constant in vector registers: re-materialising it costs 8 moves per block
 
     const int half = lane >> 5, col = lane & 31;
     // fragment (tile, block bi): lane -> row lane % 32 of the tile, k-half lane / 32
@@ -256,9 +257,13 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    // a wave whose 32 tokens all lie past the tile's end (ragged expert groups, M tails) only helps
+    // with the staging: its SIMD time goes to the other workgroup on the CU
+    const bool wave_live = tok0 + wave * 32 < M_end;
     for (int s = s_begin; s < s_end; s++) {
         const int buf = (s - s_begin) & 1;
         if (s + 1 < s_end) issue_stage(buf ^ 1, s + 1);
+        if (wave_live) {
         GemmFrag f0, f1;
         read_frag(f0, buf, 0);
         read_frag(f1, buf, 1);
@@ -275,6 +280,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         __builtin_amdgcn_sched_barrier(0);
         compute(f1, s * KB + 3);
         __builtin_amdgcn_sched_barrier(0);
+        }
         if (s + 1 < s_end) finish_stage(buf ^ 1, s + 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
