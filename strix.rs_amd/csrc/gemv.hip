@@ -26,7 +26,7 @@ struct GemvJob {
     int N;
 };
 struct GemvJobs {
-    GemvJob job[8];
+    GemvJob job[SMX_GEMV_GROUP_MAX];
 };
 
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool FUSEQ, bool DUMP, int NT>
@@ -171,16 +171,16 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
 }
 
 static int launch_jobs(smx_ctx* c, QType type, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int mt,
-                       int32_t* dump, int dump_per_row) {
+                       int32_t* dump, int dump_per_row, const char* name = nullptr) {
     if (type == kQ4_0) {
-        ProfScope ps(c, "gemv_q4_0");
+        ProfScope ps(c, name ? name : "gemv_q4_0");
         return launch_type<OpsQ4_0>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
     }
     if (type == kQ8_0) {
-        ProfScope ps(c, "gemv_q8_0");
+        ProfScope ps(c, name ? name : "gemv_q8_0");
         return launch_type<OpsQ8_0>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
     }
-    ProfScope ps(c, "gemv_q6_k");
+    ProfScope ps(c, name ? name : "gemv_q6_k");
     return launch_type<OpsQ6_K>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
 }
 
@@ -215,9 +215,10 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
     return launch_jobs(c, w.type, g, J, 1, (int)w.nblk, (int)m, mt, dump, (int)(w.type == kQ6_K ? w.K / 16 : w.K / 32));
 }
 
-// n <= 8 single-row GEMVs of one format and row length in one launch.
-int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n) {
-    if (n < 1 || n > 8) return fail(c, SMX_ERR_ARG, "gemv group of %d", n);
+// n <= SMX_GEMV_GROUP_MAX single-row GEMVs of one format and row length in one launch.
+int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
+                      const char* name) {
+    if (n < 1 || n > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "gemv group of %d", n);
     size_t maxN = 0;
     GemvJobs J = {};
     for (int i = 0; i < n; i++) {
@@ -234,7 +235,7 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
     const Weight& w0 = *ws[0];
     Geom g = pick_geom(c, w0.type, maxN, w0.nblk, 1, false, n);
     if (g.lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "gemv: activation of %zu needs %zu bytes of LDS", w0.K, g.lds);
-    return launch_jobs(c, w0.type, g, J, n, (int)w0.nblk, 1, 1, nullptr, 0);
+    return launch_jobs(c, w0.type, g, J, n, (int)w0.nblk, 1, 1, nullptr, 0, name);
 }
 
 }  // namespace smx

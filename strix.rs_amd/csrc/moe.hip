@@ -10,6 +10,7 @@
 // combine walks each token's slots in ascending slot order instead of fp32 atomics, so results do
 // not depend on scheduling.
 #include <algorithm>
+#include <vector>
 
 #include "gemv_body.h"
 #include "smx_internal.h"
@@ -44,21 +45,9 @@ __device__ __forceinline__ float det_silu(float x) {
     return x / (1.0f + det_expf(-x));
 }
 
-// a = silu(g)*u, then the activation quantiser (kernels.rs:879-892, 1174-1187).  g and u are rows
-// of `eff` floats at strides ldg; 8 lanes per 32-block.
-__global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float* __restrict__ g, const float* __restrict__ u,
-                                                             size_t ldg, int eff, int* __restrict__ xq4,
-                                                             float* __restrict__ xd, size_t nblocks) {
-    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t blk = gid >> 3;
-    const bool live = blk < nblocks;
-    float4 gv = make_float4(0.f, 0.f, 0.f, 0.f), uv = gv;
-    if (live) {
-        const int bpr = eff / 32;
-        const size_t row = blk / bpr, e0 = (blk % bpr) * 32 + (gid & 7) * 4;
-        gv = *(const float4*)(g + row * ldg + e0);
-        uv = *(const float4*)(u + row * ldg + e0);
-    }
+// a = silu(g)*u for 4 consecutive elements, then the activation quantiser over the 32-block that
+// 8 adjacent lanes hold (kernels.rs:879-892, 1174-1187): packed quants and the block scale.
+__device__ __forceinline__ void silu_mul_quant4(float4 gv, float4 uv, int* packed, float* scale) {
     float4 v;
     {
 #pragma clang fp contract(off)
@@ -77,47 +66,138 @@ __global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float* __rest
     const int q1 = max(-127, min(127, (int)rintf(v.y * inv)));
     const int q2 = max(-127, min(127, (int)rintf(v.z * inv)));
     const int q3 = max(-127, min(127, (int)rintf(v.w * inv)));
+    *packed = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+    *scale = d;
+}
+
+// Rows of `eff` floats g, u at stride ldg -> quantised silu(g)*u; 8 lanes per 32-block.
+__global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                             size_t ldg, int eff, int* __restrict__ xq4,
+                                                             float* __restrict__ xd, size_t nblocks) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t blk = gid >> 3;
+    const bool live = blk < nblocks;
+    float4 gv = make_float4(0.f, 0.f, 0.f, 0.f), uv = gv;
     if (live) {
-        xq4[gid] = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+        const int bpr = eff / 32;
+        const size_t row = blk / bpr, e0 = (blk % bpr) * 32 + (gid & 7) * 4;
+        gv = *(const float4*)(g + row * ldg + e0);
+        uv = *(const float4*)(u + row * ldg + e0);
+    }
+    int packed;
+    float d;
+    silu_mul_quant4(gv, uv, &packed, &d);
+    if (live) {
+        xq4[gid] = packed;
         if ((gid & 7) == 0) xd[blk] = d;
     }
 }
 
-// Decode GEMV over the routed experts of stacked planar Q8_0 tensors.
-//   grid = (row groups, k, ntens);  tensor z in {0,1} (gate, up) or {0} (down).
-//   expert e's rows are rows [e*rows, (e+1)*rows) of the stacked tensor.
-//   x: shared by all experts (per_k_x = 0) or one quantised row per routed expert (1).
 // Routed expert ids and weights travel as kernel arguments (no table upload on the decode path).
 struct MoeRoute {
     int ids[64];
     float w[64];
 };
 
-template <bool FUSEQ>
-__global__ __launch_bounds__(256) void moe_gemv_q8_kernel(const uint16_t* __restrict__ s0, const uint4* __restrict__ q0,
-                                                          const uint16_t* __restrict__ s1, const uint4* __restrict__ q1,
-                                                          const MoeRoute route, const float* __restrict__ x,
-                                                          const int8_t* __restrict__ xq, const float* __restrict__ xd,
-                                                          float* __restrict__ y0, float* __restrict__ y1, int nb, int rows) {
-    const int kk = blockIdx.y;
-    const size_t ebase = (size_t)route.ids[kk] * rows * nb;  // in blocks
-    GemvW W = {(blockIdx.z ? s1 : s0) + ebase, (blockIdx.z ? q1 : q0) + ebase * 2, nullptr, nullptr};
-    // gate/up: every expert reads the token's fp32 row (quantised while staged);
-    // down: one pre-quantised row per routed expert
-    GemvX X = {x, FUSEQ ? nullptr : xq + (size_t)kk * nb * 32, FUSEQ ? nullptr : xd + (size_t)kk * nb, nullptr};
-    float* y = (blockIdx.z ? y1 : y0) + (size_t)kk * rows;
-    gemv_body<OpsQ8_0, 1, 2, 2, 1, 64, FUSEQ, false>(W, X, y, rows, nb, rows, 1, nullptr, 0,
-                                                 blockIdx.x * 4 + (threadIdx.x >> 6), gridDim.x * 4);
-}
+// Decode, second half, in one launch: a_k = quantised silu(g_k)*u_k is rebuilt in LDS by every
+// workgroup (k*eff elements; measured faster than a launch of its own), then each wave computes
+// output rows y[r] = sum_k w_k * sum_b dw*dx*I over the k routed experts' down-projection rows,
+// k ascending (the roles of silu_quant, q8i_moe_down and moe_wsum, kernels.rs:879-892, 972-996,
+// 1875-1882).  A lane owns 16-byte half blocks; the k*eff/16 units of a row are walked 64*UNR at
+// a time with all UNR loads issued before the first use.  Workgroup 0 also writes the quantised
+// activation out for the stage-by-stage checks.
+template <int UNR>
+__global__ __launch_bounds__(512) void moe_down_fused_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                             const uint16_t* __restrict__ scales,
+                                                             const uint4* __restrict__ quants, const MoeRoute route,
+                                                             int k, int eff, int hidden, float* __restrict__ y,
+                                                             int* __restrict__ aq_out, float* __restrict__ ad_out) {
+    extern __shared__ __align__(16) char smem[];
+    const int nbe = eff / 32;  // blocks per expert row
+    int* sxq = (int*)smem;                          // [k][eff] int8
+    float* sxd = (float*)(smem + (size_t)k * eff);  // [k][nbe]
+    int* sid = (int*)(sxd + k * nbe);               // [k] expert ids
+    float* sw = (float*)(sid + k);                  // [k] routing weights
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < k) {
+        sid[tid] = route.ids[tid];
+        sw[tid] = route.w[tid];
+    }
+    __syncthreads();
 
-// out[o] = sum_k wexp[k]*dy[k][o], k ascending (kernels.rs:1875-1882)
-__global__ __launch_bounds__(256) void moe_wsum_kernel(const float* __restrict__ dy, const MoeRoute route,
-                                                       float* __restrict__ out, int n, int k) {
-    const int o = blockIdx.x * 256 + threadIdx.x;
-    if (o >= n) return;
-    float s = 0.f;
-    for (int e = 0; e < k; e++) s += route.w[e] * dy[(size_t)e * n + o];
-    out[o] = s;
+    const int upe = eff / 16;  // 16-byte units per expert row
+    const int units = k * upe;
+    uint4 q[UNR];
+    uint16_t sc[UNR];
+    int uu[UNR];
+    auto load_chunk = [&](int r, int base) {
+#pragma unroll
+        for (int j = 0; j < UNR; j++) {
+            const int uidx = base + j * 64 + lane;
+            const int uc = min(uidx, units - 1);
+            const int kk = uc / upe, j16 = uc - kk * upe;
+            const size_t rowblk = ((size_t)sid[kk] * hidden + r) * nbe;
+            q[j] = quants[rowblk * 2 + j16];
+            sc[j] = scales[rowblk + (j16 >> 1)];
+            uu[j] = uidx < units ? uc : -1;
+        }
+    };
+    const int items = k * eff / 4;  // float4 items, 8 per block; whole 8-lane groups are live or dead together
+    for (int it0 = 0; it0 < items; it0 += 512 * 4) {
+        float4 gv[4], uv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int it = it0 + j * 512 + tid;
+            gv[j] = uv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (it < items) {
+                gv[j] = ((const float4*)g)[it];
+                uv[j] = ((const float4*)u)[it];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int it = it0 + j * 512 + tid;
+            int packed;
+            float d;
+            silu_mul_quant4(gv[j], uv[j], &packed, &d);
+            if (it < items) {
+                sxq[it] = packed;
+                if ((it & 7) == 0) sxd[it >> 3] = d;
+                if (blockIdx.x == 0 && aq_out) {
+                    aq_out[it] = packed;
+                    if ((it & 7) == 0) ad_out[it >> 3] = d;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    int r = blockIdx.x * 8 + wave;
+    if (r < hidden) load_chunk(r, 0);
+
+    const uint4* sx16 = (const uint4*)smem;
+    for (; r < hidden; r += gridDim.x * 8) {
+        float acc = 0.f;
+        for (int base = 0; base < units; base += 64 * UNR) {
+            if (base > 0) load_chunk(r, base);
+#pragma unroll
+            for (int j = 0; j < UNR; j++) {
+                const int uc = max(uu[j], 0);
+                const int kk = uc / upe, j16 = uc - kk * upe;
+                const uint4 xv = sx16[uc];
+                int isum = dot4((int)q[j].x, (int)xv.x, 0);
+                isum = dot4((int)q[j].y, (int)xv.y, isum);
+                isum = dot4((int)q[j].z, (int)xv.z, isum);
+                isum = dot4((int)q[j].w, (int)xv.w, isum);
+                isum += swap1(isum);  // the other half of the block sits in the neighbouring lane
+                const float dx = sxd[kk * nbe + (j16 >> 1)];
+                const float term = sw[kk] * ((h2f(sc[j]) * dx) * (float)isum);
+                acc += (uu[j] >= 0 && (lane & 1) == 0) ? term : 0.f;
+            }
+        }
+        acc = group_sum<64>(acc);
+        if (lane == 63) y[r] = acc;
+        if (r + (int)gridDim.x * 8 < hidden) load_chunk(r + gridDim.x * 8, 0);
+    }
 }
 
 // y[t][i] = sum over the token's slots (ascending slot index) of wslot[s]*dy[s][i]
@@ -133,35 +213,6 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
         s += wslot[sl] * dy[(size_t)sl * hidden + i];
     }
     y[(size_t)t * hidden + i] = s;
-}
-
-static int moe_gemv(smx_ctx* c, const Weight& a, const Weight* b, const MoeRoute& route, int k, const float* x,
-                    const int8_t* xq, const float* xd, float* y0, float* y1, int rows, const char* name) {
-    const int nb = (int)a.nblk;
-    const size_t lds = ((size_t)nb * 36 + 15) & ~size_t(15);
-    if (lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "moe: activation of %d blocks does not fit LDS", nb);
-    const unsigned gx = (unsigned)((rows + 7) / 8);  // 4 waves x 2 rows per workgroup
-    const dim3 grid(gx, (unsigned)k, b ? 2u : 1u);
-    ProfScope ps(c, name);
-    const uint16_t* s1 = b ? b->scales : a.scales;
-    const uint4* q1 = (const uint4*)(b ? b->quants : a.quants);
-    if (x) {
-        auto kern = moe_gemv_q8_kernel<true>;
-        static size_t lds_set = 0;
-        int rc = set_dyn_lds(c, kern, lds, &lds_set);
-        if (rc != SMX_OK) return rc;
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, c->stream, a.scales, (const uint4*)a.quants, s1, q1, route, x, xq, xd,
-                           y0, y1, nb, rows);
-    } else {
-        auto kern = moe_gemv_q8_kernel<false>;
-        static size_t lds_set = 0;
-        int rc = set_dyn_lds(c, kern, lds, &lds_set);
-        if (rc != SMX_OK) return rc;
-        hipLaunchKernelGGL(kern, grid, dim3(256), lds, c->stream, a.scales, (const uint4*)a.quants, s1, q1, route, x, xq, xd,
-                           y0, y1, nb, rows);
-    }
-    SMX_HIP(c, hipGetLastError());
-    return SMX_OK;
 }
 
 static int silu_mul_quant(smx_ctx* c, const float* g, const float* u, size_t ldg, size_t rows, size_t eff, int8_t* xq,
@@ -185,9 +236,10 @@ struct Carver {
 };
 
 // One token through k routed experts; x_dev fp32 [hidden] on the device, y_dev fp32 [hidden].
-// Intermediates live in c->work: g[k][eff], u[k][eff], aq[k][eff], ad[k][eff/32], dy[k][hidden].
+// Intermediates live in c->work: g[k][eff], u[k][eff], and a copy of the quantised activation
+// aq[k][eff], ad[k][eff/32] for the stage-by-stage checks.
 struct MoeScratch {
-    float *g, *u, *dy;
+    float *g, *u;
     int8_t* aq;
     float* ad;
 };
@@ -202,7 +254,7 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     int rc;
     Carver cv;
     const size_t o_g = cv.take(k * eff * 4), o_u = cv.take(k * eff * 4), o_aq = cv.take(k * eff),
-                 o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(k * hidden * 4);
+                 o_ad = cv.take(k * (eff / 32) * 4);
     if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
     MoeRoute route = {};
     for (size_t i = 0; i < k; i++) {
@@ -214,17 +266,43 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     s.u = (float*)(c->work.p + o_u);
     s.aq = (int8_t*)(c->work.p + o_aq);
     s.ad = (float*)(c->work.p + o_ad);
-    s.dy = (float*)(c->work.p + o_dy);
-    rc = moe_gemv(c, L.gate, &L.up, route, (int)k, x_dev, nullptr, nullptr, s.g, s.u, (int)eff, "moe_gemv_gate_up");
-    if (rc != SMX_OK) return rc;
-    rc = silu_mul_quant(c, s.g, s.u, eff, k, eff, s.aq, s.ad);
-    if (rc != SMX_OK) return rc;
-    rc = moe_gemv(c, L.down, nullptr, route, (int)k, nullptr, s.aq, s.ad, s.dy, s.dy, (int)hidden, "moe_gemv_down");
-    if (rc != SMX_OK) return rc;
+    // gate and up of every routed expert: 2k single-row GEMVs over the same activation, grouped
+    // SMX_GEMV_GROUP_MAX to a launch (the activation quantiser runs inside the GEMV's staging)
     {
-        ProfScope ps(c, "moe_wsum");
-        hipLaunchKernelGGL(moe_wsum_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, c->stream, s.dy, route,
-                           y_dev, (int)hidden, (int)k);
+        const size_t nb = hidden / 32;
+        std::vector<Weight> views(2 * k);
+        std::vector<const Weight*> ws(2 * k);
+        std::vector<const float*> xs(2 * k, x_dev);
+        std::vector<float*> ys(2 * k);
+        for (size_t i = 0; i < k; i++)
+            for (int z = 0; z < 2; z++) {
+                const Weight& src = z ? L.up : L.gate;
+                Weight& v = views[2 * i + z];
+                v = src;
+                v.N = eff;
+                v.scales = src.scales + (size_t)ids[i] * eff * nb;
+                v.quants = (const char*)src.quants + (size_t)ids[i] * eff * nb * 32;
+                ws[2 * i + z] = &v;
+                ys[2 * i + z] = (z ? s.u : s.g) + i * eff;
+            }
+        for (size_t i = 0; i < 2 * k; i += SMX_GEMV_GROUP_MAX) {
+            const int n = (int)std::min<size_t>(SMX_GEMV_GROUP_MAX, 2 * k - i);
+            rc = launch_gemv_group(c, &ws[i], &xs[i], &ys[i], n, "moe_gemv_gate_up");
+            if (rc != SMX_OK) return rc;
+        }
+    }
+    {
+        const size_t lds = k * eff + k * (eff / 32) * 4 + k * 8;
+        if (lds > 160 * 1024)
+            return fail(c, SMX_ERR_LIMIT, "moe_ffn: %zu experts x %zu intermediate values need %zu bytes of LDS (limit 163840)",
+                        k, eff, lds);
+        ProfScope ps(c, "moe_gemv_down");
+        auto kern = moe_down_fused_kernel<6>;
+        static size_t lds_set = 0;
+        if ((rc = set_dyn_lds(c, kern, lds, &lds_set)) != SMX_OK) return rc;
+        const unsigned grid = (unsigned)std::min<size_t>((hidden + 7) / 8, (size_t)c->num_cu * 2);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, c->stream, s.g, s.u, L.down.scales, (const uint4*)L.down.quants,
+                           route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad);
         SMX_HIP(c, hipGetLastError());
     }
     if (out_scratch) *out_scratch = s;

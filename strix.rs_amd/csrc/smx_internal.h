@@ -88,6 +88,8 @@ namespace smx {
 
 int fail(smx_ctx* c, int code, const char* fmt, ...);
 int hip_fail(smx_ctx* c, hipError_t e, const char* what);
+#define SMX_GEMV_GROUP_MAX 16  // single-row GEMVs that may share one launch
+
 #define SMX_HIP(c, call)                                                   \
     do {                                                                   \
         hipError_t e_ = (call);                                            \
@@ -147,7 +149,8 @@ int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, 
 // m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);
 // n <= 8 single-row GEMVs of one format and row length in one launch (device pointers).
-int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n);
+int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
+                      const char* name = nullptr);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);

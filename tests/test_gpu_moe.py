@@ -12,7 +12,8 @@ def _layer(accel, synth, layer, ne, hidden, eff, seed):
     return gate, up, down
 
 
-@pytest.mark.parametrize("ne,hidden,eff,k", [(4, 64, 32, 2), (8, 256, 96, 3), (64, 2048, 768, 8)])
+# k = 12: the 24 gate/up GEMVs exceed one grouped launch; eff = 416: down-projection units with a ragged tail
+@pytest.mark.parametrize("ne,hidden,eff,k", [(4, 64, 32, 2), (8, 256, 96, 3), (64, 2048, 768, 8), (16, 320, 416, 12)])
 def test_moe_ffn_stagewise(accel, orc, synth, relerr, ne, hidden, eff, k):
     gate, up, down = _layer(accel, synth, 3, ne, hidden, eff, seed=ne + hidden)
     ids, w = synth.zipf_routing(1, ne, k, seed=5)
