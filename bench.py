@@ -144,9 +144,10 @@ class Bench:
         }
 
     # ------------------------------------------------------------------ grouped GEMV (one launch, G weights)
-    def gemv_group(self, name, ty, N, K, G, min_total_bytes, steps=None, warmup=None):
+    def gemv_group(self, name, ty, N, K, G, min_total_bytes, steps=None, warmup=None, act=0):
         """G single-token GEMVs of the same shape in one launch (the gate+up pair of a decode step for
-        G = 2), rotating through >= 1 GB of weight copies; a step is one launch."""
+        G = 2), rotating through >= 1 GB of weight copies; a step is one launch.  act = 1: the rmsnorm
+        of the activation runs inside the same launch (norm + quantiser + G GEMVs)."""
         acc, sy = self.acc, self.synth
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
         algo1, wbytes = gemv_bytes(ty, N, K, 1)
@@ -164,15 +165,24 @@ class Bench:
         acc.h2d(xd, x)
         yds = [acc.dev_alloc(N * 4) for _ in range(G)]
         ngroups = ncopies // G
+        wd = 0
+        if act:
+            wd = acc.dev_alloc(K * 4)
+            acc.h2d(wd, np.ones(K, np.float32) + 0.01 * x[0])
 
         def step(i):
             g0 = (i % ngroups) * G
-            acc.gemv_batch_dev(keys[g0:g0 + G], [xd] * G, yds)
+            if act:
+                acc.gemv_fused_dev(keys[g0:g0 + G], act, xd, wd, yds, 1e-6)
+            else:
+                acc.gemv_batch_dev(keys[g0:g0 + G], [xd] * G, yds)
 
         ms, wall_ms = self._timed(step, steps, warmup)
         for k in keys:
             acc.evict(k)
         acc.dev_free(xd)
+        if wd:
+            acc.dev_free(wd)
         for p in yds:
             acc.dev_free(p)
         algo = algo1 * G
@@ -343,6 +353,7 @@ def main():
     plans = [
         ("copy_calib", lambda: b.copy_calib()),
         ("q4_0_gemv_9728x2560_gate_up_pair", lambda: b.gemv_group("q4_0_gemv_9728x2560_gate_up_pair", Q4_0, 9728, 2560, 2, int(1.1 * GB))),
+        ("q4_0_rmsnorm_gate_up_pair", lambda: b.gemv_group("q4_0_rmsnorm_gate_up_pair", Q4_0, 9728, 2560, 2, int(1.1 * GB), act=1)),
         ("q4_0_gemv_9728x2560_batch8", lambda: b.gemv_group("q4_0_gemv_9728x2560_batch8", Q4_0, 9728, 2560, 8, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),

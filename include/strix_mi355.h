@@ -127,6 +127,25 @@ int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, f
 int smx_gemv_batch_dev(smx_ctx* ctx, size_t n, const char* const* keys, const float* const* xs_dev,
                        float* const* ys_dev);
 int smx_gemm_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
+
+/* ---- the step BEFORE a decode GEMV fused into it: the reference's rmsnorm_xquant / silu_xquant /
+ *      geglu_xquant (crates/strix-backend-rocm/src/kernels.rs:101-147, 191-226, 151-187) write the
+ *      quantised activation for the GEMVs that follow; here the producer runs inside the GEMV's own
+ *      activation staging, so norm + quantiser + up to 16 GEMVs of one format and in_dim (q/k/v,
+ *      gate+up, down) are ONE launch and no fp32 or int8 activation goes through HBM.
+ *      RMSNORM : x = (a * 1/sqrt(mean(a^2) + eps)) * b   (b = norm weight, may be NULL; ops.rs:15-27.
+ *                The mean is formed in double and rounded once, where the reference uses rsqrtf.)
+ *      SILU_MUL: x = silu(a) * b        (ops.rs:74-87)     GEGLU: x = gelu_tanh(a) * b  (ops.rs:110-121)
+ *      a, b: fp32 [in_dim].  1 done, 0 if any key is not resident, <0 error. ---- */
+#define SMX_ACT_NONE 0
+#define SMX_ACT_RMSNORM 1
+#define SMX_ACT_SILU_MUL 2
+#define SMX_ACT_GEGLU 3
+int smx_gemv_fused_dev(smx_ctx* ctx, size_t n, const char* const* keys, int act, const float* a_dev,
+                       const float* b_dev, float eps, float* const* ys_dev);
+int smx_gemv_fused(smx_ctx* ctx, const char* key, int act, const float* a, const float* b, size_t in_len,
+                   float eps, float* y, size_t out_cap);
+
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                     const float* x_dev, float* y_dev);
 

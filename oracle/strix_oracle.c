@@ -390,6 +390,45 @@ float orc_expf(float x) {
 
 float orc_silu(float x) { return x / (1.0f + orc_expf(-x)); }
 
+/* tanh(z) = 1 - 2/(exp(2z) + 1) on the fixed-sequence exp above (saturates to +-1 through its clamps) */
+float orc_tanhf(float z) { return 1.0f - 2.0f / (orc_expf(2.0f * z) + 1.0f); }
+
+/* 0.5*x*(1 + tanh(sqrt(2/pi)*(x + 0.044715 x^3))), ops.rs:110-113; kernels.rs:162-163 */
+float orc_gelu_tanh(float x) {
+    float x3 = x * x * x;
+    float inner = 0.7978845608f * (x + 0.044715f * x3);
+    return 0.5f * x * (1.0f + orc_tanhf(inner));
+}
+
+/* Activation producers of the step before a GEMV (kernels.rs:101-226; ops.rs:15-27, 74-87, 110-121).
+ *   ORC_ACT_RMSNORM : out = (a * scale) * b, scale = 1/sqrt(mean(a^2) + eps); b == NULL: unit weight.
+ *                     The mean and the scale are formed in double and rounded once, so the result does
+ *                     not depend on the order in which the squares are summed.
+ *   ORC_ACT_SILU_MUL: out = silu(a) * b
+ *   ORC_ACT_GEGLU   : out = gelu_tanh(a) * b */
+int orc_act_produce(int act, const float* a, const float* b, int n, float eps, float* out) {
+    if (act == ORC_ACT_NONE) {
+        for (int i = 0; i < n; i++) out[i] = a[i];
+    } else if (act == ORC_ACT_RMSNORM) {
+        double ss = 0.0;
+        for (int i = 0; i < n; i++) ss += (double)a[i] * (double)a[i];
+        float scale = (float)(1.0 / sqrt(ss / (double)n + (double)eps));
+        for (int i = 0; i < n; i++) {
+            float v = a[i] * scale;
+            out[i] = b ? v * b[i] : v;
+        }
+    } else if (act == ORC_ACT_SILU_MUL) {
+        if (!b) return -1;
+        for (int i = 0; i < n; i++) out[i] = orc_silu(a[i]) * b[i];
+    } else if (act == ORC_ACT_GEGLU) {
+        if (!b) return -1;
+        for (int i = 0; i < n; i++) out[i] = orc_gelu_tanh(a[i]) * b[i];
+    } else {
+        return -1;
+    }
+    return 0;
+}
+
 int orc_moe_ffn_q8(const uint8_t* gate, const uint8_t* up, const uint8_t* down, int hidden, int eff,
                    int ne, const int32_t* ids, const float* wexp, int k, const float* x, float* y,
                    float* gu, int8_t* aq, float* ad, const int8_t* aq_in, const float* ad_in) {

@@ -92,6 +92,11 @@ int orc_matmul_q8(int type, const uint8_t* w, int K, int N, const int8_t* xq, co
  * fp32 operations, so both sides produce the same bits from the same input. */
 float orc_expf(float x);
 float orc_silu(float x); /* x / (1 + exp(-x)), ops.rs:73-76 */
+float orc_tanhf(float z);
+float orc_gelu_tanh(float x); /* ops.rs:110-113 */
+enum { ORC_ACT_NONE = 0, ORC_ACT_RMSNORM = 1, ORC_ACT_SILU_MUL = 2, ORC_ACT_GEGLU = 3 };
+/* activation producers in front of a GEMV (kernels.rs:101-226): rmsnorm(a)*b, silu(a)*b, gelu_tanh(a)*b */
+int orc_act_produce(int act, const float* a, const float* b, int n, float eps, float* out);
 
 /* One token through k routed experts, crates/strix-backend-cpu/src/mellum.rs:1623-1669
  * with the integer arithmetic of kernels.rs:942-996, 1875-1882:

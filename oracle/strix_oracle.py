@@ -19,7 +19,9 @@ BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q6_K: 210}
 
 def build(force=False):
     """Compile the oracle with gcc (strict IEEE, no FMA contraction)."""
-    if force or not os.path.exists(_LIB_PATH):
+    srcs = [os.path.join(_HERE, f) for f in ("strix_oracle.c", "strix_oracle.h", "Makefile")]
+    stale = not os.path.exists(_LIB_PATH) or any(os.path.getmtime(f) > os.path.getmtime(_LIB_PATH) for f in srcs)
+    if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B", "libstrix_oracle.so"],
                               stdout=subprocess.DEVNULL)
     return _LIB_PATH
@@ -49,6 +51,11 @@ def lib():
         L.orc_expf.argtypes = [C.c_float]
         L.orc_silu.restype = C.c_float
         L.orc_silu.argtypes = [C.c_float]
+        L.orc_gelu_tanh.restype = C.c_float
+        L.orc_gelu_tanh.argtypes = [C.c_float]
+        L.orc_tanhf.restype = C.c_float
+        L.orc_tanhf.argtypes = [C.c_float]
+        L.orc_act_produce.argtypes = [i, vp, vp, i, C.c_float, vp]
         L.orc_moe_ffn_q8.argtypes = [vp, vp, vp, i, i, i, vp, vp, i, vp, vp, vp, vp, vp, vp, vp]
         L.orc_route_topk.argtypes = [vp, i, i, vp, vp]
         L.orc_lcg_fill.argtypes = [vp, vp, sz]
@@ -154,6 +161,25 @@ def expf(x):
 
 def silu(x):
     return float(lib().orc_silu(float(x)))
+
+
+def gelu_tanh(x):
+    return float(lib().orc_gelu_tanh(float(x)))
+
+
+ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
+
+
+def act_produce(act, a, b=None, eps=0.0):
+    """The fp32 activation a GEMV's quantiser sees: rmsnorm(a)*b, silu(a)*b or gelu_tanh(a)*b."""
+    a = _c(a, np.float32)
+    if b is not None:
+        b = _c(b, np.float32)
+    out = np.empty_like(a)
+    rc = lib().orc_act_produce(int(act), _p(a), _p(b), a.size, float(eps), _p(out))
+    if rc != 0:
+        raise ValueError("act_produce failed")
+    return out
 
 
 def moe_ffn_q8(gate, up, down, hidden, eff, ne, ids, wexp, x, aq_in=None, ad_in=None):

@@ -31,8 +31,9 @@ EXPORTS = [
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
-    "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev",
+    "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused",
 ]
+ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
 
 class SmxError(RuntimeError):
@@ -86,6 +87,8 @@ def load_library():
     L.smx_gemv_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemm_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemv_batch_dev.argtypes = [vp, sz, vp, vp, vp]
+    L.smx_gemv_fused_dev.argtypes = [vp, sz, vp, i, vp, vp, C.c_float, vp]
+    L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_prof_enable.argtypes = [vp, i]
     L.smx_prof_reset.argtypes = [vp]
@@ -186,6 +189,15 @@ class Mi355WeightAccel:
         x = _c(x, np.float32).reshape(-1)
         y = np.empty(out_dim, np.float32)
         ok = self._check(self._L.smx_gemv(self._h, key.encode(), _p(x), x.size, _p(y), y.size))
+        return y if ok else None
+
+    def gemv_fused(self, key, act, a, b, out_dim, eps=0.0):
+        """GEMV of producer(a, b): rmsnorm(a)*b, silu(a)*b or gelu_tanh(a)*b (kernels.rs:101-226), one launch."""
+        a = _c(a, np.float32).reshape(-1)
+        b = None if b is None else _c(b, np.float32).reshape(-1)
+        y = np.empty(out_dim, np.float32)
+        ok = self._check(self._L.smx_gemv_fused(self._h, key.encode(), int(act), _p(a), _p(b), a.size, float(eps),
+                                                _p(y), y.size))
         return y if ok else None
 
     def gemv_rows(self, key, xs, out_dim):
@@ -308,6 +320,12 @@ class Mi355WeightAccel:
         xp = (C.c_void_p * n)(*xs_dev)
         yp = (C.c_void_p * n)(*ys_dev)
         return self._check(self._L.smx_gemv_batch_dev(self._h, n, k, xp, yp))
+
+    def gemv_fused_dev(self, keys, act, a_dev, b_dev, ys_dev, eps=0.0):
+        n = len(keys)
+        k = (C.c_char_p * n)(*[s.encode() for s in keys])
+        yp = (C.c_void_p * n)(*ys_dev)
+        return self._check(self._L.smx_gemv_fused_dev(self._h, n, k, int(act), a_dev, b_dev, float(eps), yp))
 
     def gemm_dev(self, key, xs_dev, m, y_dev):
         return self._check(self._L.smx_gemm_dev(self._h, key.encode(), xs_dev, m, y_dev))

@@ -239,6 +239,61 @@ int smx_gemv_batch_dev(smx_ctx* c, size_t n, const char* const* keys, const floa
     return launch_gemv_group(c, ws, xs_dev, ys_dev, (int)n);
 }
 
+// Activation producer + quantiser + GEMV(s) in one launch.
+static int gemv_fused_check(smx_ctx* c, int act, const float* a, const float* b, const char* who) {
+    if (act < SMX_ACT_NONE || act > SMX_ACT_GEGLU) return fail(c, SMX_ERR_ARG, "%s: unknown activation producer %d", who, act);
+    if (!a) return fail(c, SMX_ERR_ARG, "%s: null activation", who);
+    if ((act == SMX_ACT_SILU_MUL || act == SMX_ACT_GEGLU) && !b) return fail(c, SMX_ERR_ARG, "%s: the producer needs its second operand", who);
+    if (act == SMX_ACT_NONE && b) return fail(c, SMX_ERR_ARG, "%s: second operand without a producer", who);
+    return SMX_OK;
+}
+
+int smx_gemv_fused_dev(smx_ctx* c, size_t n, const char* const* keys, int act, const float* a_dev, const float* b_dev,
+                       float eps, float* const* ys_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!keys || !ys_dev) return fail(c, SMX_ERR_ARG, "gemv_fused_dev: null argument");
+    if (n == 0 || n > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_LIMIT, "gemv_fused_dev: %zu weights (1..%d per launch)", n, SMX_GEMV_GROUP_MAX);
+    int rc = gemv_fused_check(c, act, a_dev, b_dev, "gemv_fused_dev");
+    if (rc != SMX_OK) return rc;
+    const Weight* ws[SMX_GEMV_GROUP_MAX];
+    const float* xs[SMX_GEMV_GROUP_MAX];
+    for (size_t i = 0; i < n; i++) {
+        if (!keys[i] || !ys_dev[i]) return fail(c, SMX_ERR_ARG, "gemv_fused_dev: item %zu has a null pointer", i);
+        ws[i] = find_weight(c, keys[i]);
+        if (!ws[i]) return SMX_NOT_RESIDENT;
+        xs[i] = a_dev;
+    }
+    const ActProd prod = {act, b_dev, eps};
+    return launch_gemv_group(c, ws, xs, ys_dev, (int)n, nullptr, &prod);
+}
+
+int smx_gemv_fused(smx_ctx* c, const char* key, int act, const float* a, const float* b, size_t in_len, float eps,
+                   float* y, size_t out_cap) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key) return fail(c, SMX_ERR_ARG, "gemv_fused: null key");
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (!y) return fail(c, SMX_ERR_ARG, "gemv_fused: null output");
+    int rc = gemv_fused_check(c, act, a, b, "gemv_fused");
+    if (rc != SMX_OK) return rc;
+    if (in_len != w->K) return fail(c, SMX_ERR_ARG, "gemv_fused: activation length %zu, weight in_dim %zu", in_len, w->K);
+    if (out_cap < w->N) return fail(c, SMX_ERR_ARG, "gemv_fused: output capacity %zu < %zu", out_cap, w->N);
+    SMX_HIP(c, hipSetDevice(c->device));
+    if ((rc = ensure(c, c->xf32, 2 * w->K * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->yf32, w->N * 4)) != SMX_OK) return rc;
+    float* a_dev = (float*)c->xf32.p;
+    float* b_dev = b ? a_dev + w->K : nullptr;
+    SMX_HIP(c, hipMemcpyAsync(a_dev, a, w->K * 4, hipMemcpyHostToDevice, c->stream));
+    if (b) SMX_HIP(c, hipMemcpyAsync(b_dev, b, w->K * 4, hipMemcpyHostToDevice, c->stream));
+    const float* xs[1] = {a_dev};
+    float* ys[1] = {(float*)c->yf32.p};
+    const ActProd prod = {act, b_dev, eps};
+    if ((rc = launch_gemv_group(c, &w, xs, ys, 1, nullptr, &prod)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, w->N * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
 int smx_gemm_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, float* y_dev) {
     if (!c) return SMX_ERR_ARG;
     if (!key || !xs_dev || !y_dev) return fail(c, SMX_ERR_ARG, "gemm_dev: null argument");

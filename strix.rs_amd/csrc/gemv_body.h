@@ -20,6 +20,9 @@
 
 #include <cstdint>
 
+#include "../../include/strix_mi355.h"
+#include "detmath.h"
+
 namespace smx {
 
 // Optional per-wave timeline stamps (development builds only; compiled out of the library).
@@ -82,6 +85,10 @@ struct GemvX {
     const int8_t* xq;    // pre-quantised rows [m][K]
     const float* xd;     // [m][K/32]
     const int* xs;       // [m][K/32] packed 16-element sums
+    // activation producer applied to x before the fused quantiser (one row only):
+    const float* x2;     // rmsnorm: weight or null; silu_mul / geglu: the `up` operand
+    int prod;            // SMX_ACT_*
+    float eps;           // rmsnorm
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -257,15 +264,43 @@ __device__ __forceinline__ void compute_unit(OpsQ6_K, const OpsQ6_K::Regs& r, co
     }
 }
 
+// 1/sqrt(mean(x^2) + eps) of one row for the rmsnorm producer (kernels.rs:101-113).  The squares are
+// summed in double by the whole workgroup (per thread, per wave, then over the waves in index order)
+// and the scale is rounded to fp32 once, so it does not depend on the workgroup's shape.  `scratch`
+// is LDS the caller has not written yet; every thread of the workgroup must call this.
+__device__ __forceinline__ float rms_scale(char* scratch, const float* x, int n, float eps) {
+#pragma clang fp contract(off)
+    double ss = 0.0;
+    for (int i = threadIdx.x; i < n / 4; i += blockDim.x) {
+        const float4 v = ((const float4*)x)[i];
+        ss += (double)v.x * (double)v.x;
+        ss += (double)v.y * (double)v.y;
+        ss += (double)v.z * (double)v.z;
+        ss += (double)v.w * (double)v.w;
+    }
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    double* red = (double*)scratch;
+    const int nwaves = blockDim.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    double tot = 0.0;
+    for (int w = 0; w < nwaves; w++) tot += red[w];
+    __syncthreads();  // the caller overwrites the scratch next
+    return (float)(1.0 / sqrt(tot / (double)n + (double)eps));
+}
+
 // Stage one activation row into LDS.  8 lanes per 32-block, one float4 / one packed dword each;
-// reductions inside the 8 lanes go over DPP.
+// reductions inside the 8 lanes go over DPP.  With the quantiser fused, an activation producer
+// (X.prod: rmsnorm(x)*x2, silu(x)*x2, gelu_tanh(x)*x2; kernels.rs:101-226) runs on the values first.
 template <class Ops, bool FUSEQ>
 __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X, int t, bool zero) {
     const int nb32 = Ops::nb32(nblk);
     const int items = nb32 * 8;
     constexpr int SB = 2;  // items per thread requested before any is consumed
+    float rs = 1.f;
+    if (FUSEQ && X.prod == SMX_ACT_RMSNORM) rs = rms_scale(tok, X.x + (size_t)t * nb32 * 32, nb32 * 32, X.eps);
     for (int i0 = threadIdx.x; i0 < items; i0 += blockDim.x * SB) {
-        float4 v[SB];
+        float4 v[SB], v2[SB];
         int pk[SB];
 #pragma unroll
         for (int j = 0; j < SB; j++) {
@@ -274,7 +309,11 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
             v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
             pk[j] = 0;
             if (FUSEQ) {
-                if (live) v[j] = ((const float4*)(X.x + (size_t)t * nb32 * 32))[i];
+                v2[j] = make_float4(1.f, 1.f, 1.f, 1.f);
+                if (live) {
+                    v[j] = ((const float4*)(X.x + (size_t)t * nb32 * 32))[i];
+                    if (X.x2) v2[j] = ((const float4*)(X.x2 + (size_t)t * nb32 * 32))[i];
+                }
             } else {
                 if (live) pk[j] = ((const int*)(X.xq + (size_t)t * nb32 * 32))[i];
             }
@@ -288,7 +327,19 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
             int packed = pk[j], s_lo = 0, s_hi = 0;
             float d = 0.f;
             if (FUSEQ) {
-                const float4 w = v[j];
+                float4 w = v[j];
+                if (X.prod != SMX_ACT_NONE) {
+#pragma clang fp contract(off)
+                    const float4 g = v2[j];
+                    if (X.prod == SMX_ACT_RMSNORM) {
+                        w.x = (w.x * rs) * g.x; w.y = (w.y * rs) * g.y; w.z = (w.z * rs) * g.z; w.w = (w.w * rs) * g.w;
+                    } else if (X.prod == SMX_ACT_SILU_MUL) {
+                        w.x = det_silu(w.x) * g.x; w.y = det_silu(w.y) * g.y; w.z = det_silu(w.z) * g.z; w.w = det_silu(w.w) * g.w;
+                    } else {
+                        w.x = det_gelu_tanh(w.x) * g.x; w.y = det_gelu_tanh(w.y) * g.y;
+                        w.z = det_gelu_tanh(w.z) * g.z; w.w = det_gelu_tanh(w.w) * g.w;
+                    }
+                }
                 float a = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
                 a = fmaxf(a, dpp_f<0xB1>(a));
                 a = fmaxf(a, dpp_f<0x4E>(a));

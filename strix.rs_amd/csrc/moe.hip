@@ -12,38 +12,11 @@
 #include <algorithm>
 #include <vector>
 
+#include "detmath.h"
 #include "gemv_body.h"
 #include "smx_internal.h"
 
 namespace smx {
-
-// exp() as a fixed sequence of IEEE fp32 operations (no contraction), so that the quantised
-// silu(g)*u is reproducible bit for bit on any conforming implementation.
-__device__ __forceinline__ float det_expf(float x) {
-#pragma clang fp contract(off)
-    x = x > 88.0f ? 88.0f : x;
-    x = x < -87.0f ? -87.0f : x;
-    const float n = rintf(x * 1.44269504088896341f);
-    float r = x - n * 0.693359375f;
-    r = r - n * -2.12194440e-4f;
-    float p = 1.9875691500e-4f;
-    p = p * r + 1.3981999507e-3f;
-    p = p * r + 8.3334519073e-3f;
-    p = p * r + 4.1665795894e-2f;
-    p = p * r + 1.6666665459e-1f;
-    p = p * r + 5.0000001201e-1f;
-    const float r2 = r * r;
-    p = p * r2;
-    p = p + r;
-    p = p + 1.0f;
-    return ldexpf(p, (int)n);
-}
-
-// silu(x) = x / (1 + exp(-x)), crates/strix-backend-cpu/src/ops.rs:73-76
-__device__ __forceinline__ float det_silu(float x) {
-#pragma clang fp contract(off)
-    return x / (1.0f + det_expf(-x));
-}
 
 // a = silu(g)*u for 4 consecutive elements, then the activation quantiser over the 32-block that
 // 8 adjacent lanes hold (kernels.rs:879-892, 1174-1187): packed quants and the block scale.

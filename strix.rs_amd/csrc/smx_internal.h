@@ -149,8 +149,14 @@ int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, 
 // m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);
 // n <= 8 single-row GEMVs of one format and row length in one launch (device pointers).
+// prod (optional): activation producer applied to every job's x before the fused quantiser.
+struct ActProd {
+    int kind;        // SMX_ACT_*
+    const float* b;  // rmsnorm weight (or null) / the `up` operand of silu_mul, geglu
+    float eps;
+};
 int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
-                      const char* name = nullptr);
+                      const char* name = nullptr, const ActProd* prod = nullptr);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);

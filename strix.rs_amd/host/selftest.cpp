@@ -56,6 +56,19 @@ int main() {
         return 6;
     } catch (const strix::BackendError&) {
     }
+    {   // rmsnorm fused into the GEMV == GEMV of the normalised row computed here
+        double ss = 0;
+        for (size_t i = 0; i < K; i++) ss += (double)x[i] * (double)x[i];
+        const float scale = (float)(1.0 / std::sqrt(ss / (double)K + 1e-6));
+        std::vector<float> xn(K);
+        for (size_t i = 0; i < K; i++) xn[i] = x[i] * scale;
+        auto yf = acc->gemv_fused("blk.0.attn_q.weight", SMX_ACT_RMSNORM, x, nullptr, 1e-6f);
+        auto yn = acc->gemv("blk.0.attn_q.weight", xn);
+        if (!yf || !yn) return 7;
+        for (size_t r = 0; r < N; r++)
+            if (std::fabs((*yf)[r] - (*yn)[r]) > 1e-5 * maxref * scale) return 8;
+        if (acc->gemv_fused("never.adopted", SMX_ACT_RMSNORM, x, nullptr, 1e-6f)) return 9;
+    }
     std::printf("selftest ok\n");
     return 0;
 }

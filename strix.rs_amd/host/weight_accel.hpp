@@ -116,6 +116,18 @@ class Mi355WeightAccel final : public WeightAccel {
         }
         return out;
     }
+    // Beyond the trait: the producer of the step before the GEMV (rmsnorm / SwiGLU / GeGLU, the
+    // reference's rmsnorm_xquant, silu_xquant, geglu_xquant, kernels.rs:101-226) fused into it.
+    // b: norm weight (may be null) or the `up` operand.
+    std::optional<std::vector<float>> gemv_fused(const std::string& key, int act, const std::vector<float>& a,
+                                                 const std::vector<float>* b, float eps) {
+        if (b && b->size() != a.size()) throw BackendError(SMX_ERR_ARG, "gemv_fused: operand lengths differ");
+        std::vector<float> y(out_of(key, /*required=*/false));
+        if (!ok(smx_gemv_fused(ctx_, key.c_str(), act, a.data(), b ? b->data() : nullptr, a.size(), eps,
+                               y.empty() ? &dummy_ : y.data(), y.size())))
+            return std::nullopt;
+        return y;
+    }
     std::optional<std::vector<float>> prefill_q8_gemm(const std::string& key, const std::vector<float>& xs, size_t m) override {
         if (m == 0) throw BackendError(SMX_ERR_ARG, "prefill_q8_gemm: m == 0");
         std::vector<float> y(m * out_of(key));

@@ -279,6 +279,46 @@ def test_expf_and_silu_accuracy(orc):
     assert np.abs(g - xs / (1 + np.exp(-xs.astype(np.float64)))).max() < 3e-6
 
 
+def test_activation_producers_known_values(orc):
+    """The reference's own literal checks: ops.rs:204-232 (rmsnorm), 260-276 (silu, swiglu), 287-294 (gelu_tanh)."""
+    out = orc.act_produce(orc.ACT_RMSNORM, [1.0, 2.0, 3.0, 4.0], [1.0] * 4, 0.0)
+    assert abs(out[0] - 0.365148) <= 1e-5 and abs(out[3] - 1.460593) <= 1e-5
+    out = orc.act_produce(orc.ACT_RMSNORM, [2.0, 2.0], [3.0, 0.5], 0.0)
+    assert abs(out[0] - 3.0) <= 1e-6 and abs(out[1] - 0.5) <= 1e-6
+    assert np.array_equal(orc.act_produce(orc.ACT_RMSNORM, [2.0, 2.0], None, 0.0), np.ones(2, np.float32))
+    assert abs(orc.silu(1.0) - 0.731059) <= 1e-5 and abs(orc.silu(20.0) - 20.0) <= 1e-3
+    out = orc.act_produce(orc.ACT_SILU_MUL, [0.0, 1.0], [5.0, 2.0])
+    assert abs(out[0]) <= 1e-6 and abs(out[1] - 0.731059 * 2.0) <= 1e-5
+    assert abs(orc.gelu_tanh(0.0)) <= 1e-7 and abs(orc.gelu_tanh(1.0) - 0.8412) <= 1e-3
+    assert abs(orc.gelu_tanh(10.0) - 10.0) <= 1e-3 and abs(orc.gelu_tanh(-10.0)) < 1e-3
+    out = orc.act_produce(orc.ACT_GEGLU, [1.0, -10.0], [2.0, 3.0])
+    assert abs(out[0] - 2 * 0.8412) <= 2e-3 and abs(out[1]) < 3e-3
+
+
+def test_activation_producers_against_float64(orc):
+    """What the literals leave open: the whole range against numpy float64 formulas, and rmsnorm's
+    independence of the summation order (the double-precision mean is rounded once)."""
+    rng = np.random.default_rng(3)
+    g = np.concatenate([rng.normal(0, 3, 4000), np.linspace(-30, 30, 601), [88.0, -88.0, 1e-8, -1e-8]]).astype(np.float32)
+    u = rng.normal(0, 1, g.size).astype(np.float32)
+    g64, u64 = g.astype(np.float64), u.astype(np.float64)
+    ref_gelu = 0.5 * g64 * (1 + np.tanh(np.float64(np.float32(0.7978845608)) * (g64 + 0.044715 * g64 ** 3)))
+    got = orc.act_produce(orc.ACT_GEGLU, g, u).astype(np.float64)
+    assert np.max(np.abs(got - ref_gelu * u64) / (1 + np.abs(ref_gelu * u64))) <= 2e-6
+    got = orc.act_produce(orc.ACT_SILU_MUL, g, u).astype(np.float64)
+    ref = g64 / (1 + np.exp(-g64)) * u64
+    assert np.max(np.abs(got - ref) / (1 + np.abs(ref))) <= 1e-6
+    x = rng.normal(0, 2, 2560).astype(np.float32)
+    w = rng.normal(1, 0.1, 2560).astype(np.float32)
+    for eps in (0.0, 1e-6, 1e-5):
+        got = orc.act_produce(orc.ACT_RMSNORM, x, w, eps)
+        scale = np.float32(1.0 / np.sqrt(np.mean(x.astype(np.float64) ** 2) + np.float64(np.float32(eps))))
+        assert np.array_equal(got, (x * scale) * w)
+        perm = rng.permutation(x.size)   # summing the squares in another order changes nothing
+        assert np.array_equal(orc.act_produce(orc.ACT_RMSNORM, x[perm], w[perm], eps), got[perm])
+    assert np.array_equal(orc.act_produce(orc.ACT_NONE, x), x)
+
+
 def test_route_topk_ties_lowest_index(orc):
     ids, w = orc.route_topk(np.array([0.5, 2.0, 2.0, -1.0, 2.0], np.float32), 2)
     assert list(ids) == [1, 2] and abs(w.sum() - 1) < 1e-6 and abs(w[0] - 0.5) < 1e-6
