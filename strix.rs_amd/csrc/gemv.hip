@@ -109,7 +109,7 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     Geom g;
     size_t tokb, units;
     if (type == kQ4_0) { tokb = (nblk * 40 + 15) & ~size_t(15); units = nblk; }
-    else if (type == kQ8_0) { tokb = (nblk * 36 + 15) & ~size_t(15); units = nblk * 2; }
+    else if (type == kQ8_0) { tokb = (nblk * 36 + 15) & ~size_t(15); units = (mt >= 4 && !dump) ? nblk : nblk * 2; }
     else { tokb = nblk * 2 * 176; units = nblk * 4; }
     g.nt = 1024;
     g.lpr = 64;
@@ -178,6 +178,8 @@ static int launch_jobs(smx_ctx* c, QType type, const Geom& g, const GemvJobs& J,
     }
     if (type == kQ8_0) {
         ProfScope ps(c, name ? name : "gemv_q8_0");
+        // 4 or 8 activation rows: a lane takes whole blocks (the per-row scale work halves)
+        if (mt >= 4 && !dump) return launch_type<OpsQ8_0W>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
         return launch_type<OpsQ8_0>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
     }
     ProfScope ps(c, name ? name : "gemv_q6_k");

@@ -134,6 +134,18 @@ struct OpsQ8_0 {
     }
 };
 
+// Q8_0 with a whole 32-byte block per lane: used for several activation rows, where the per-row
+// scale arithmetic and LDS scale read of a unit are paid once per block instead of once per half block.
+struct OpsQ8_0W : OpsQ8_0 {
+    struct Regs { uint4 q0, q1; uint16_t s; };
+    static __device__ __forceinline__ int units_per_row(int nblk) { return nblk; }
+    static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nblk, int u) {
+        r.q0 = w.quants[(row * nblk + u) * 2];
+        r.q1 = w.quants[(row * nblk + u) * 2 + 1];
+        r.s = w.scales[row * nblk + u];
+    }
+};
+
 struct OpsQ6_K {
     struct Regs { uint4 a, b, h; uint2 sc; uint16_t d; };
     static __device__ __forceinline__ int units_per_row(int nsb) { return nsb * 4; }
@@ -211,6 +223,30 @@ __device__ __forceinline__ void compute_unit(OpsQ8_0, const OpsQ8_0::Regs& r, co
         isum += swap1(isum);  // whole-block i32
         if (DUMP) {
             if (act && !(u & 1) && t == 0 && dump_row) dump_row[u >> 1] = isum;
+        }
+        acc[t] += (dw * dx) * (float)isum;
+    }
+}
+
+template <int MT, bool DUMP>
+__device__ __forceinline__ void compute_unit(OpsQ8_0W, const OpsQ8_0W::Regs& r, const char* smem, int tokb, int nblk,
+                                             int u, bool act, float* acc, int* dump_row) {
+    const float dw = act ? h2f(r.s) : 0.f;
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        const char* tok = smem + t * tokb;
+        const uint4 x0 = ((const uint4*)tok)[u * 2], x1 = ((const uint4*)tok)[u * 2 + 1];
+        const float dx = ((const float*)(tok + nblk * 32))[u];
+        int isum = dot4((int)r.q0.x, (int)x0.x, 0);
+        isum = dot4((int)r.q0.y, (int)x0.y, isum);
+        isum = dot4((int)r.q0.z, (int)x0.z, isum);
+        isum = dot4((int)r.q0.w, (int)x0.w, isum);
+        isum = dot4((int)r.q1.x, (int)x1.x, isum);
+        isum = dot4((int)r.q1.y, (int)x1.y, isum);
+        isum = dot4((int)r.q1.z, (int)x1.z, isum);
+        isum = dot4((int)r.q1.w, (int)x1.w, isum);
+        if (DUMP) {
+            if (act && t == 0 && dump_row) dump_row[u] = isum;
         }
         acc[t] += (dw * dx) * (float)isum;
     }
