@@ -68,6 +68,12 @@ int smx_upload_q6_k(smx_ctx* ctx, const char* key, const void* bytes, size_t nby
 int smx_upload_moe_q8(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_nbytes,
                       const void* up, size_t up_nbytes, const void* down, size_t down_nbytes,
                       size_t hidden, size_t eff, size_t ne);
+/* WeightAccel::upload_moe_q6, accel.rs:185-196; decode.rs:2793-2831: the same tensors as Q6_K
+ * superblocks (hidden and eff multiples of 256).  Such a layer is served by smx_moe_ffn (one token);
+ * smx_moe_layer returns an error for it. */
+int smx_upload_moe_q6(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_nbytes,
+                      const void* up, size_t up_nbytes, const void* down, size_t down_nbytes,
+                      size_t hidden, size_t eff, size_t ne);
 /* Drop one resident weight (the reference never frees, decode.rs:458-460). */
 int smx_evict(smx_ctx* ctx, const char* key);
 

@@ -432,9 +432,17 @@ int orc_act_produce(int act, const float* a, const float* b, int n, float eps, f
 int orc_moe_ffn_q8(const uint8_t* gate, const uint8_t* up, const uint8_t* down, int hidden, int eff,
                    int ne, const int32_t* ids, const float* wexp, int k, const float* x, float* y,
                    float* gu, int8_t* aq, float* ad, const int8_t* aq_in, const float* ad_in) {
-    if (hidden % 32 || eff % 32) return -1;
-    size_t gate_eb = (size_t)(hidden / 32) * 34 * (size_t)eff; /* decode.rs:2730 */
-    size_t down_eb = (size_t)(eff / 32) * 34 * (size_t)hidden; /* decode.rs:2731 */
+    return orc_moe_ffn(ORC_Q8_0, gate, up, down, hidden, eff, ne, ids, wexp, k, x, y, gu, aq, ad, aq_in, ad_in);
+}
+
+int orc_moe_ffn(int type, const uint8_t* gate, const uint8_t* up, const uint8_t* down, int hidden, int eff,
+                int ne, const int32_t* ids, const float* wexp, int k, const float* x, float* y,
+                float* gu, int8_t* aq, float* ad, const int8_t* aq_in, const float* ad_in) {
+    if (type != ORC_Q8_0 && type != ORC_Q6_K) return -1;
+    const int be = type == ORC_Q6_K ? 256 : 32, bb = type == ORC_Q6_K ? 210 : 34;
+    if (hidden % be || eff % be) return -1;
+    size_t gate_eb = (size_t)(hidden / be) * bb * (size_t)eff; /* decode.rs:2730, 2806 */
+    size_t down_eb = (size_t)(eff / be) * bb * (size_t)hidden; /* decode.rs:2731, 2807 */
     int8_t* xq = (int8_t*)malloc((size_t)hidden);
     float* xd = (float*)malloc((size_t)(hidden / 32) * 4);
     float* g = (float*)malloc((size_t)eff * 4);
@@ -449,8 +457,8 @@ int orc_moe_ffn_q8(const uint8_t* gate, const uint8_t* up, const uint8_t* down, 
     for (int kk = 0; kk < k; kk++) {
         int e = ids[kk];
         if (e < 0 || e >= ne) { rc = -1; break; }
-        orc_matmul_q8(ORC_Q8_0, gate + (size_t)e * gate_eb, hidden, eff, xq, xd, 1, g, 1);
-        orc_matmul_q8(ORC_Q8_0, up + (size_t)e * gate_eb, hidden, eff, xq, xd, 1, u, 1);
+        orc_matmul_q8(type, gate + (size_t)e * gate_eb, hidden, eff, xq, xd, 1, g, 1);
+        orc_matmul_q8(type, up + (size_t)e * gate_eb, hidden, eff, xq, xd, 1, u, 1);
         if (gu) {
             memcpy(gu + ((size_t)kk * 2) * eff, g, (size_t)eff * 4);
             memcpy(gu + ((size_t)kk * 2 + 1) * eff, u, (size_t)eff * 4);
@@ -461,7 +469,7 @@ int orc_moe_ffn_q8(const uint8_t* gate, const uint8_t* up, const uint8_t* down, 
         if (ad) memcpy(ad + (size_t)kk * (eff / 32), adk, (size_t)(eff / 32) * 4);
         const int8_t* q = aq_in ? aq_in + (size_t)kk * eff : aqk;
         const float* d = ad_in ? ad_in + (size_t)kk * (eff / 32) : adk;
-        orc_matmul_q8(ORC_Q8_0, down + (size_t)e * down_eb, eff, hidden, q, d, 1, dy, 1);
+        orc_matmul_q8(type, down + (size_t)e * down_eb, eff, hidden, q, d, 1, dy, 1);
         for (int i = 0; i < hidden; i++) y[i] += wexp[kk] * dy[i]; /* mellum.rs:1666-1668; kernels.rs:1880 */
     }
     free(xq); free(xd); free(g); free(u); free(a); free(aqk); free(adk); free(dy);

@@ -108,6 +108,11 @@ int orc_act_produce(int act, const float* a, const float* b, int n, float eps, f
 int orc_moe_ffn_q8(const uint8_t* gate, const uint8_t* up, const uint8_t* down, int hidden, int eff,
                    int ne, const int32_t* ids, const float* wexp, int k, const float* x, float* y,
                    float* gu, int8_t* aq, float* ad, const int8_t* aq_in, const float* ad_in);
+/* The same with the expert tensors in `type` = ORC_Q8_0 or ORC_Q6_K (decode.rs:2793-2852: Q6_K expert
+ * layers; hidden and eff multiples of 256, 210-byte superblocks). */
+int orc_moe_ffn(int type, const uint8_t* gate, const uint8_t* up, const uint8_t* down, int hidden, int eff,
+                int ne, const int32_t* ids, const float* wexp, int k, const float* x, float* y,
+                float* gu, int8_t* aq, float* ad, const int8_t* aq_in, const float* ad_in);
 
 /* Top-k routing, mellum.rs:1178-1192: softmax over all experts, k largest
  * (ties -> lowest index, kernels.rs:1843-1845), renormalise. */

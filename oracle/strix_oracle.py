@@ -57,6 +57,7 @@ def lib():
         L.orc_tanhf.argtypes = [C.c_float]
         L.orc_act_produce.argtypes = [i, vp, vp, i, C.c_float, vp]
         L.orc_moe_ffn_q8.argtypes = [vp, vp, vp, i, i, i, vp, vp, i, vp, vp, vp, vp, vp, vp, vp]
+        L.orc_moe_ffn.argtypes = [i, vp, vp, vp, i, i, i, vp, vp, i, vp, vp, vp, vp, vp, vp, vp]
         L.orc_route_topk.argtypes = [vp, i, i, vp, vp]
         L.orc_lcg_fill.argtypes = [vp, vp, sz]
         _lib = L
@@ -182,8 +183,8 @@ def act_produce(act, a, b=None, eps=0.0):
     return out
 
 
-def moe_ffn_q8(gate, up, down, hidden, eff, ne, ids, wexp, x, aq_in=None, ad_in=None):
-    """Returns (y[hidden], gu[k][2][eff], aq[k][eff], ad[k][eff/32])."""
+def moe_ffn_q8(gate, up, down, hidden, eff, ne, ids, wexp, x, aq_in=None, ad_in=None, ty=Q8_0):
+    """Returns (y[hidden], gu[k][2][eff], aq[k][eff], ad[k][eff/32]).  ty: Q8_0 or Q6_K expert tensors."""
     gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
     ids = _c(ids, np.int32)
     wexp = _c(wexp, np.float32)
@@ -195,8 +196,8 @@ def moe_ffn_q8(gate, up, down, hidden, eff, ne, ids, wexp, x, aq_in=None, ad_in=
     ad = np.empty((k, eff // 32), np.float32)
     if aq_in is not None:
         aq_in, ad_in = _c(aq_in, np.int8), _c(ad_in, np.float32)
-    rc = lib().orc_moe_ffn_q8(_p(gate), _p(up), _p(down), hidden, eff, ne, _p(ids), _p(wexp), k,
-                              _p(x), _p(y), _p(gu), _p(aq), _p(ad), _p(aq_in), _p(ad_in))
+    rc = lib().orc_moe_ffn(ty, _p(gate), _p(up), _p(down), hidden, eff, ne, _p(ids), _p(wexp), k,
+                           _p(x), _p(y), _p(gu), _p(aq), _p(ad), _p(aq_in), _p(ad_in))
     if rc != 0:
         raise ValueError("moe_ffn_q8 failed")
     return y, gu, aq, ad

@@ -32,6 +32,7 @@ EXPORTS = [
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
     "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused",
+    "smx_upload_moe_q6",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -70,6 +71,7 @@ def load_library():
     for n in ("smx_upload_q4_0", "smx_upload_q8_0", "smx_upload_q6_k"):
         getattr(L, n).argtypes = [vp, cp, vp, sz, sz, sz]
     L.smx_upload_moe_q8.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz, sz, sz, sz]
+    L.smx_upload_moe_q6.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz, sz, sz, sz]
     L.smx_evict.argtypes = [vp, cp]
     L.smx_gemv.argtypes = [vp, cp, vp, sz, vp, sz]
     L.smx_gemv_rows.argtypes = [vp, cp, vp, sz, sz, vp, sz]
@@ -180,6 +182,11 @@ class Mi355WeightAccel:
     def upload_moe_q8(self, layer, gate, up, down, hidden, eff, ne):
         gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
         return self._check(self._L.smx_upload_moe_q8(self._h, layer, _p(gate), gate.size, _p(up), up.size,
+                                                     _p(down), down.size, hidden, eff, ne))
+
+    def upload_moe_q6(self, layer, gate, up, down, hidden, eff, ne):
+        gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
+        return self._check(self._L.smx_upload_moe_q6(self._h, layer, _p(gate), gate.size, _p(up), up.size,
                                                      _p(down), down.size, hidden, eff, ne))
 
     def evict(self, key):

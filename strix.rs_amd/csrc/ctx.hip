@@ -254,29 +254,31 @@ int smx_upload_q6_k(smx_ctx* c, const char* key, const void* bytes, size_t nbyte
     return upload(c, kQ6_K, key, bytes, nbytes, in_dim, out_dim);
 }
 
-int smx_upload_moe_q8(smx_ctx* c, size_t layer, const void* gate, size_t gate_n, const void* up, size_t up_n,
-                      const void* down, size_t down_n, size_t hidden, size_t eff, size_t ne) {
+static int upload_moe(smx_ctx* c, QType type, const char* who, size_t layer, const void* gate, size_t gate_n, const void* up,
+                      size_t up_n, const void* down, size_t down_n, size_t hidden, size_t eff, size_t ne) {
     if (!c) return SMX_ERR_ARG;
-    if (!gate || !up || !down) return fail(c, SMX_ERR_ARG, "upload_moe_q8: null tensor");
-    if (hidden == 0 || eff == 0 || ne == 0 || hidden % 32 != 0 || eff % 32 != 0)
-        return fail(c, SMX_ERR_ARG, "upload_moe_q8: hidden %zu / eff %zu must be positive multiples of 32", hidden, eff);
-    const size_t gate_eb = (hidden / 32) * 34 * eff, down_eb = (eff / 32) * 34 * hidden;  // decode.rs:2730-2731
+    if (!gate || !up || !down) return fail(c, SMX_ERR_ARG, "%s: null tensor", who);
+    const size_t be = type == kQ6_K ? 256 : 32, bb = type == kQ6_K ? 210 : 34;
+    if (hidden == 0 || eff == 0 || ne == 0 || hidden % be != 0 || eff % be != 0)
+        return fail(c, SMX_ERR_ARG, "%s: hidden %zu / eff %zu must be positive multiples of %zu", who, hidden, eff, be);
+    const size_t gate_eb = (hidden / be) * bb * eff, down_eb = (eff / be) * bb * hidden;  // decode.rs:2730-2731, 2806-2807
     if (gate_n != gate_eb * ne || up_n != gate_eb * ne || down_n != down_eb * ne)
-        return fail(c, SMX_ERR_ARG, "upload_moe_q8: byte lengths (%zu, %zu, %zu) do not match %zu experts of %zu/%zu",
-                    gate_n, up_n, down_n, ne, gate_eb, down_eb);
+        return fail(c, SMX_ERR_ARG, "%s: byte lengths (%zu, %zu, %zu) do not match %zu experts of %zu/%zu", who, gate_n, up_n,
+                    down_n, ne, gate_eb, down_eb);
     SMX_HIP(c, hipSetDevice(c->device));
     MoeLayer L;
+    L.type = type;
     L.hidden = hidden;
     L.eff = eff;
     L.ne = ne;
-    int rc = build_weight(c, kQ8_0, (const uint8_t*)gate, gate_n, hidden, ne * eff, &L.gate);
+    int rc = build_weight(c, type, (const uint8_t*)gate, gate_n, hidden, ne * eff, &L.gate);
     if (rc != SMX_OK) return rc;
-    rc = build_weight(c, kQ8_0, (const uint8_t*)up, up_n, hidden, ne * eff, &L.up);
+    rc = build_weight(c, type, (const uint8_t*)up, up_n, hidden, ne * eff, &L.up);
     if (rc != SMX_OK) {
         free_weight(L.gate);
         return rc;
     }
-    rc = build_weight(c, kQ8_0, (const uint8_t*)down, down_n, eff, ne * hidden, &L.down);
+    rc = build_weight(c, type, (const uint8_t*)down, down_n, eff, ne * hidden, &L.down);
     if (rc != SMX_OK) {
         free_weight(L.gate);
         free_weight(L.up);
@@ -293,6 +295,16 @@ int smx_upload_moe_q8(smx_ctx* c, size_t layer, const void* gate, size_t gate_n,
         c->moe.emplace(layer, L);
     }
     return SMX_OK;
+}
+
+int smx_upload_moe_q8(smx_ctx* c, size_t layer, const void* gate, size_t gate_n, const void* up, size_t up_n,
+                      const void* down, size_t down_n, size_t hidden, size_t eff, size_t ne) {
+    return upload_moe(c, kQ8_0, "upload_moe_q8", layer, gate, gate_n, up, up_n, down, down_n, hidden, eff, ne);
+}
+
+int smx_upload_moe_q6(smx_ctx* c, size_t layer, const void* gate, size_t gate_n, const void* up, size_t up_n,
+                      const void* down, size_t down_n, size_t hidden, size_t eff, size_t ne) {
+    return upload_moe(c, kQ6_K, "upload_moe_q6", layer, gate, gate_n, up, up_n, down, down_n, hidden, eff, ne);
 }
 
 int smx_evict(smx_ctx* c, const char* key) {

@@ -219,7 +219,7 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
 
 // n <= SMX_GEMV_GROUP_MAX single-row GEMVs of one format and row length in one launch.
 int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
-                      const char* name, const ActProd* prod) {
+                      const char* name, const ActProd* prod, const float* const* x2s) {
     if (n < 1 || n > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "gemv group of %d", n);
     size_t maxN = 0;
     GemvJobs J = {};
@@ -232,7 +232,7 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
         J.job[i].W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
         J.job[i].X = {xs[i], nullptr, nullptr, nullptr};
         if (prod) {
-            J.job[i].X.x2 = prod->b;
+            J.job[i].X.x2 = x2s ? x2s[i] : prod->b;
             J.job[i].X.prod = prod->kind;
             J.job[i].X.eps = prod->eps;
         }

@@ -198,6 +198,32 @@ static int silu_mul_quant(smx_ctx* c, const float* g, const float* u, size_t ldg
     return SMX_OK;
 }
 
+// out[o] = sum_k wexp[k]*dy[k][o], k ascending (kernels.rs:1875-1882); used by the Q6_K expert path
+__global__ __launch_bounds__(256) void moe_wsum_kernel(const float* __restrict__ dy, const MoeRoute route,
+                                                       float* __restrict__ out, int n, int k) {
+    const int o = blockIdx.x * 256 + threadIdx.x;
+    if (o >= n) return;
+    float s = 0.f;
+    for (int e = 0; e < k; e++) s += route.w[e] * dy[(size_t)e * n + o];
+    out[o] = s;
+}
+
+// Rows [e*rows, (e+1)*rows) of a stacked expert tensor as a weight of its own (planes are row-major).
+static Weight expert_view(const Weight& src, size_t e, size_t rows) {
+    Weight v = src;
+    v.N = rows;
+    const size_t b0 = e * rows * src.nblk;  // first block / superblock of the expert
+    v.scales = src.scales + b0;
+    if (src.type == kQ6_K) {
+        v.quants = (const char*)src.quants + b0 * 128;
+        v.qh = (const char*)src.qh + b0 * 64;
+        v.sc = src.sc + b0 * 16;
+    } else {
+        v.quants = (const char*)src.quants + b0 * (src.type == kQ4_0 ? 16 : 32);
+    }
+    return v;
+}
+
 // Scratch carve-up helper: 256-byte aligned bump allocation inside one DevBuf.
 struct Carver {
     size_t off = 0;
@@ -227,7 +253,7 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     int rc;
     Carver cv;
     const size_t o_g = cv.take(k * eff * 4), o_u = cv.take(k * eff * 4), o_aq = cv.take(k * eff),
-                 o_ad = cv.take(k * (eff / 32) * 4);
+                 o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(L.type == kQ6_K ? k * hidden * 4 : 0);
     if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
     MoeRoute route = {};
     for (size_t i = 0; i < k; i++) {
@@ -242,20 +268,14 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     // gate and up of every routed expert: 2k single-row GEMVs over the same activation, grouped
     // SMX_GEMV_GROUP_MAX to a launch (the activation quantiser runs inside the GEMV's staging)
     {
-        const size_t nb = hidden / 32;
         std::vector<Weight> views(2 * k);
         std::vector<const Weight*> ws(2 * k);
         std::vector<const float*> xs(2 * k, x_dev);
         std::vector<float*> ys(2 * k);
         for (size_t i = 0; i < k; i++)
             for (int z = 0; z < 2; z++) {
-                const Weight& src = z ? L.up : L.gate;
-                Weight& v = views[2 * i + z];
-                v = src;
-                v.N = eff;
-                v.scales = src.scales + (size_t)ids[i] * eff * nb;
-                v.quants = (const char*)src.quants + (size_t)ids[i] * eff * nb * 32;
-                ws[2 * i + z] = &v;
+                views[2 * i + z] = expert_view(z ? L.up : L.gate, (size_t)ids[i], eff);
+                ws[2 * i + z] = &views[2 * i + z];
                 ys[2 * i + z] = (z ? s.u : s.g) + i * eff;
             }
         for (size_t i = 0; i < 2 * k; i += SMX_GEMV_GROUP_MAX) {
@@ -264,7 +284,38 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
             if (rc != SMX_OK) return rc;
         }
     }
-    {
+    if (L.type == kQ6_K) {
+        // Q6_K experts (decode.rs:2839-2852, moe6_launches): the down projections are k more jobs of the
+        // grouped GEMV, each quantising silu(g_k)*u_k inside its staging; then the weighted sum
+        float* dy = (float*)(c->work.p + o_dy);
+        std::vector<Weight> views(k);
+        std::vector<const Weight*> ws(k);
+        std::vector<const float*> gs(k), us(k);
+        std::vector<float*> ys(k);
+        for (size_t i = 0; i < k; i++) {
+            views[i] = expert_view(L.down, (size_t)ids[i], hidden);
+            ws[i] = &views[i];
+            gs[i] = s.g + i * eff;
+            us[i] = s.u + i * eff;
+            ys[i] = dy + i * hidden;
+        }
+        const ActProd prod = {SMX_ACT_SILU_MUL, nullptr, 0.f};
+        for (size_t i = 0; i < k; i += SMX_GEMV_GROUP_MAX) {
+            const int n = (int)std::min<size_t>(SMX_GEMV_GROUP_MAX, k - i);
+            rc = launch_gemv_group(c, &ws[i], &gs[i], &ys[i], n, "moe_gemv_down", &prod, &us[i]);
+            if (rc != SMX_OK) return rc;
+        }
+        {
+            ProfScope ps(c, "moe_wsum");
+            hipLaunchKernelGGL(moe_wsum_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, c->stream, dy, route,
+                               y_dev, (int)hidden, (int)k);
+            SMX_HIP(c, hipGetLastError());
+        }
+        if (out_scratch) {  // the quantised activation is never materialised on this path: rebuild it for the checks
+            rc = silu_mul_quant(c, s.g, s.u, eff, k, eff, s.aq, s.ad);
+            if (rc != SMX_OK) return rc;
+        }
+    } else {
         const size_t lds = k * eff + k * (eff / 32) * 4 + k * 8;
         if (lds > 160 * 1024)
             return fail(c, SMX_ERR_LIMIT, "moe_ffn: %zu experts x %zu intermediate values need %zu bytes of LDS (limit 163840)",
@@ -365,6 +416,8 @@ int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const siz
     if (it == c->moe.end()) return SMX_NOT_RESIDENT;
     const MoeLayer& L = it->second;
     const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
+    if (L.type != kQ8_0)
+        return fail(c, SMX_ERR_LIMIT, "moe_layer: layer %zu holds Q6_K experts, which only the one-token path (moe_ffn) serves", layer);
     if (m == 0 || slots == 0) return fail(c, SMX_ERR_ARG, "moe_layer: m %zu, slots %zu", m, slots);  // decode.rs:1622
     if (y_cap < m * hidden) return fail(c, SMX_ERR_ARG, "moe_layer: output capacity %zu < %zu", y_cap, m * hidden);
     if (slots > (size_t(1) << 24) || m > 65535 || m * hidden >= (size_t(1) << 31) || slots * eff >= (size_t(1) << 31) ||

@@ -33,9 +33,10 @@ struct Weight {
     const int8_t* sc = nullptr;        // Q6_K sub-scales
 };
 
-// A resident MoE layer (Q8_0 experts): three planar Q8_0 tensors whose rows are
+// A resident MoE layer (Q8_0 or Q6_K experts): three planar tensors whose rows are
 // the experts' rows back to back (expert e, row r -> row e*rows + r).
 struct MoeLayer {
+    QType type = kQ8_0;
     size_t hidden = 0, eff = 0, ne = 0;
     Weight gate, up, down;  // gate/up: N = ne*eff, K = hidden; down: N = ne*hidden, K = eff
 };
@@ -155,8 +156,9 @@ struct ActProd {
     const float* b;  // rmsnorm weight (or null) / the `up` operand of silu_mul, geglu
     float eps;
 };
+// x2s (optional, with prod): a second operand per job instead of prod->b.
 int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
-                      const char* name = nullptr, const ActProd* prod = nullptr);
+                      const char* name = nullptr, const ActProd* prod = nullptr, const float* const* x2s = nullptr);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);

@@ -77,6 +77,11 @@ class Mi355WeightAccel final : public WeightAccel {
     bool upload_q8_0(const std::string& key, const uint8_t* b, size_t n, size_t in_dim, size_t out_dim) override {
         return ok(smx_upload_q8_0(ctx_, key.c_str(), b, n, in_dim, out_dim));
     }
+    // accel.rs:185-196
+    bool upload_moe_q6(size_t layer, const uint8_t* gate, size_t gate_n, const uint8_t* up, size_t up_n, const uint8_t* down,
+                       size_t down_n, size_t hidden, size_t eff, size_t ne) {
+        return ok(smx_upload_moe_q6(ctx_, layer, gate, gate_n, up, up_n, down, down_n, hidden, eff, ne));
+    }
     bool upload_moe_q8(size_t layer, const uint8_t* gate, size_t gate_n, const uint8_t* up, size_t up_n, const uint8_t* down,
                        size_t down_n, size_t hidden, size_t eff, size_t ne) override {
         hidden_[layer] = hidden;

@@ -64,6 +64,14 @@ def make_moe_q8(ne, hidden, eff, seed):
     return gate, up, down
 
 
+def make_moe_q6(ne, hidden, eff, seed):
+    """The same tensors as Q6_K superblocks (hidden and eff multiples of 256)."""
+    gate = make_q6_k(ne * eff, hidden, seed)
+    up = make_q6_k(ne * eff, hidden, seed + 1)
+    down = make_q6_k(ne * hidden, eff, seed + 2)
+    return gate, up, down
+
+
 def zipf_routing(m, ne, k, seed, s=1.1):
     """Per token: k distinct experts drawn without replacement with Zipf(s) popularity,
     weights = renormalised softmax of N(0,1) logits.  Returns ids[m][k] i32, w[m][k] f32."""

@@ -35,6 +35,32 @@ def test_moe_ffn_stagewise(accel, orc, synth, relerr, ne, hidden, eff, k):
     assert np.array_equal(accel.moe_ffn(3, ids[0], w[0], x), y)
 
 
+@pytest.mark.parametrize("ne,hidden,eff,k", [(4, 256, 256, 2), (8, 512, 768, 3), (16, 2048, 768, 8), (32, 256, 512, 20)])
+def test_moe_ffn_q6k_experts_stagewise(accel, orc, synth, relerr, pkg, ne, hidden, eff, k):
+    """Q6_K expert layers (upload_moe_q6, decode.rs:2793-2852): same stages, Q6_K integer sub-block dots."""
+    gate, up, down = synth.make_moe_q6(ne, hidden, eff, seed=ne + eff)
+    assert accel.upload_moe_q6(7, gate, up, down, hidden, eff, ne)
+    ids, w = synth.zipf_routing(1, ne, k, seed=11)
+    x = synth.make_acts(1, hidden, seed=12)[0]
+    y, gu, aq, ad = accel.moe_ffn_stages(7, ids[0], w[0], x, eff)
+    ry, rgu, raq, rad = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[0], w[0], x, ty=14)
+    assert relerr(gu, rgu) <= TOL
+    a = np.array([[orc.silu(g) * u for g, u in zip(gu[kk, 0], gu[kk, 1])] for kk in range(k)], np.float32)
+    q2, d2, _ = orc.actquant(a, eff)
+    assert np.array_equal(aq, q2)
+    assert np.array_equal(ad.view(np.uint32), d2.view(np.uint32))
+    ry2, _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[0], w[0], x, aq_in=aq, ad_in=ad, ty=14)
+    assert relerr(y, ry2) <= TOL
+    assert relerr(y, ry) <= 2e-2
+    assert np.array_equal(accel.moe_ffn(7, ids[0], w[0], x), y)
+    # the grouped prefill entry point does not take Q6_K layers
+    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
+    with pytest.raises(pkg.SmxError):
+        accel.moe_layer_q8_dev(7, x[None, :], 1, plan, slot_tok, wslot)
+    with pytest.raises(pkg.SmxError):
+        accel.upload_moe_q6(8, gate[:-1], up, down, hidden, eff, ne)
+
+
 def test_moe_ffn_declines_and_errors(accel, synth, pkg):
     x = np.zeros(64, np.float32)
     assert accel.moe_ffn(999, [0], [1.0], x) is None

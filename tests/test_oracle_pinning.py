@@ -330,28 +330,31 @@ def test_route_topk_ties_lowest_index(orc):
     assert np.allclose(w, p[ids] / p[ids].sum(), rtol=1e-5)
 
 
-def test_moe_ffn_equals_sum_of_dense_experts(orc, synth):
-    """mellum.rs:1623-1669: y = sum_k w_k * down_k(silu(gate_k x) * up_k x), routed order."""
-    ne, hidden, eff, k = 6, 128, 64, 3
-    gate, up, down = synth.make_moe_q8(ne, hidden, eff, seed=81)
+@pytest.mark.parametrize("TY", [Q8_0, Q6_K])
+def test_moe_ffn_equals_sum_of_dense_experts(orc, synth, TY):
+    """mellum.rs:1623-1669: y = sum_k w_k * down_k(silu(gate_k x) * up_k x), routed order; Q8_0 and
+    Q6_K expert tensors (decode.rs:2717-2831)."""
+    ne, hidden, eff, k = (6, 128, 64, 3) if TY == Q8_0 else (5, 256, 512, 3)
+    gate, up, down = (synth.make_moe_q8 if TY == Q8_0 else synth.make_moe_q6)(ne, hidden, eff, seed=81)
     ids, w = synth.zipf_routing(1, ne, k, seed=82)
     x = synth.make_acts(1, hidden, seed=83)[0]
-    y, gu, aq, ad = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[0], w[0], x)
-    geb, deb = (hidden // 32) * 34 * eff, (eff // 32) * 34 * hidden
+    y, gu, aq, ad = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[0], w[0], x, ty=TY)
+    be, bb = (32, 34) if TY == Q8_0 else (256, 210)
+    geb, deb = (hidden // be) * bb * eff, (eff // be) * bb * hidden
     acc = np.zeros(hidden, np.float32)
     for kk, e in enumerate(ids[0]):
-        g = orc.matmul_q8_from_f32(Q8_0, gate[e * geb:(e + 1) * geb], hidden, eff, x)[0]
-        u = orc.matmul_q8_from_f32(Q8_0, up[e * geb:(e + 1) * geb], hidden, eff, x)[0]
+        g = orc.matmul_q8_from_f32(TY, gate[e * geb:(e + 1) * geb], hidden, eff, x)[0]
+        u = orc.matmul_q8_from_f32(TY, up[e * geb:(e + 1) * geb], hidden, eff, x)[0]
         assert np.array_equal(gu[kk, 0], g) and np.array_equal(gu[kk, 1], u)
         a = np.array([orc.silu(float(a_)) for a_ in g], np.float32) * u
-        dy = orc.matmul_q8_from_f32(Q8_0, down[e * deb:(e + 1) * deb], eff, hidden, a)[0]
+        dy = orc.matmul_q8_from_f32(TY, down[e * deb:(e + 1) * deb], eff, hidden, a)[0]
         acc = (acc + w[0][kk] * dy).astype(np.float32)
     assert np.array_equal(y, acc)
     # against the f32 path end to end: only quantisation noise
     accf = np.zeros(hidden, np.float64)
     for kk, e in enumerate(ids[0]):
-        g = orc.matmul_f32(Q8_0, gate[e * geb:(e + 1) * geb], hidden, eff, x, 1)[0].astype(np.float64)
-        u = orc.matmul_f32(Q8_0, up[e * geb:(e + 1) * geb], hidden, eff, x, 1)[0].astype(np.float64)
+        g = orc.matmul_f32(TY, gate[e * geb:(e + 1) * geb], hidden, eff, x, 1)[0].astype(np.float64)
+        u = orc.matmul_f32(TY, up[e * geb:(e + 1) * geb], hidden, eff, x, 1)[0].astype(np.float64)
         a = (g / (1 + np.exp(-g)) * u).astype(np.float32)
-        accf += w[0][kk] * orc.matmul_f32(Q8_0, down[e * deb:(e + 1) * deb], eff, hidden, a, 1)[0]
+        accf += w[0][kk] * orc.matmul_f32(TY, down[e * deb:(e + 1) * deb], eff, hidden, a, 1)[0]
     assert np.abs(y - accf).max() / np.abs(accf).max() < 5e-2
