@@ -192,6 +192,43 @@ class Bench:
                 "frac_hbm_peak": gbs / HBM_PEAK_GBS, "kernel": KERNEL[ty], "kernel_avg_us": ms / steps * 1e3,
                 "kernel_GBps": gbs, "kernel_frac_hbm_peak": gbs / HBM_PEAK_GBS}
 
+    # ------------------------------------------------------------------ dense FFN decode step (2 launches)
+    def ffn_block(self, name, ty, H, F, min_total_bytes, steps=None, warmup=None):
+        """One token through a dense FFN: launch 1 = rmsnorm + quantiser + gate and up GEMVs, launch 2 =
+        SwiGLU + quantiser + down GEMV; rotating through >= 1 GB of (gate, up, down) sets."""
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
+        a1, w1 = gemv_bytes(ty, F, H, 1)
+        a2, w2 = gemv_bytes(ty, H, F, 1)
+        nsets = max(2, -(-min_total_bytes // (2 * w1 + w2)))
+        srcs = [(sy.make_weight(ty, F, H, seed=1500 + i), sy.make_weight(ty, H, F, seed=1600 + i)) for i in range(2)]
+        for i in range(nsets):
+            up_fn = getattr(acc, UPLOAD[ty])
+            assert up_fn(f"{name}.g{i}", srcs[i % 2][0], H, F) and up_fn(f"{name}.u{i}", srcs[(i + 1) % 2][0], H, F)
+            assert up_fn(f"{name}.d{i}", srcs[i % 2][1], F, H)
+        del srcs
+        x = sy.make_acts(1, H, seed=7)
+        xd, wd, gd, ud, yd = (acc.dev_alloc(n * 4) for n in (H, H, F, F, H))
+        acc.h2d(xd, x)
+        acc.h2d(wd, np.ones(H, np.float32))
+
+        def step(i):
+            j = i % nsets
+            acc.gemv_fused_dev([f"{name}.g{j}", f"{name}.u{j}"], 1, xd, wd, [gd, ud], 1e-6)
+            acc.gemv_fused_dev([f"{name}.d{j}"], 2, gd, ud, [yd])
+
+        ms, wall_ms = self._timed(step, steps, warmup)
+        for i in range(nsets):
+            for t in "gud":
+                acc.evict(f"{name}.{t}{i}")
+        for p in (xd, wd, gd, ud, yd):
+            acc.dev_free(p)
+        algo = 2 * a1 + a2
+        gbs = algo * steps / (ms * 1e-3) / 1e9
+        return {"workload": name, "shape": {"hidden": H, "ffn": F, "M": 1, "launches_per_step": 2}, "weight_sets": nsets,
+                "algorithmic_bytes": algo, "steps": steps, "ms_per_step": ms / steps, "GBps": gbs,
+                "frac_hbm_peak": gbs / HBM_PEAK_GBS}
+
     # ------------------------------------------------------------------ copy (counter calibration)
     def copy_calib(self, nbytes=256 << 20, steps=20):
         """A plain copy of known size: what FETCH_SIZE / WRITE_SIZE read for it scales the counters."""
@@ -355,6 +392,7 @@ def main():
         ("q4_0_gemv_9728x2560_gate_up_pair", lambda: b.gemv_group("q4_0_gemv_9728x2560_gate_up_pair", Q4_0, 9728, 2560, 2, int(1.1 * GB))),
         ("q4_0_rmsnorm_gate_up_pair", lambda: b.gemv_group("q4_0_rmsnorm_gate_up_pair", Q4_0, 9728, 2560, 2, int(1.1 * GB), act=1)),
         ("q4_0_gemv_9728x2560_batch8", lambda: b.gemv_group("q4_0_gemv_9728x2560_batch8", Q4_0, 9728, 2560, 8, int(1.1 * GB))),
+        ("q4_0_ffn_decode_block_2560x9728", lambda: b.ffn_block("q4_0_ffn_decode_block_2560x9728", Q4_0, 2560, 9728, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
         ("q6_k_gemv_15360x3840", lambda: b.gemv("q6_k_gemv_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB))),

@@ -150,3 +150,45 @@ def test_grouped_gemv_launch(accel, orc, synth, relerr):
     assert accel.gemv_batch_dev(["t.grp0", "t.absent"], [xd, xd], [y0, y1]) is False
     for p in (xd, y0, y1):
         accel.dev_free(p)
+
+
+@pytest.mark.parametrize("act", [2, 3])
+def test_ffn_block_two_launches_in_a_graph(accel, orc, synth, relerr, act):
+    """A dense FFN decode step as two launches (norm + quantiser + gate/up; SwiGLU or GeGLU + quantiser
+    + down), captured in a graph and replayed: equal to the eager run every time and to the oracle chain."""
+    H, F = 1024, 2560
+    rg, ru, rd = synth.make_weight(2, F, H, seed=21), synth.make_weight(2, F, H, seed=22), synth.make_weight(2, H, F, seed=23)
+    assert accel.upload_q4_0("t.ffn.gate", rg, H, F) and accel.upload_q4_0("t.ffn.up", ru, H, F)
+    assert accel.upload_q4_0("t.ffn.down", rd, F, H)
+    x = synth.make_acts(1, H, seed=24)[0] * 2.0
+    nw = synth.make_acts(1, H, seed=25)[0] * 0.1 + 1.0
+    xd, wd, gd, ud, yd = (accel.dev_alloc(n * 4) for n in (H, H, F, F, H))
+    accel.h2d(xd, x)
+    accel.h2d(wd, nw)
+
+    def block():
+        accel.gemv_fused_dev(["t.ffn.gate", "t.ffn.up"], 1, xd, wd, [gd, ud], 1e-6)
+        accel.gemv_fused_dev(["t.ffn.down"], act, gd, ud, [yd])
+
+    block()
+    eager = accel.d2h(np.empty(H, np.float32), yd)
+    xn = orc.act_produce(1, x, nw, 1e-6)
+    g = orc.matmul_q8_from_f32(2, rg, H, F, xn)[0]
+    u = orc.matmul_q8_from_f32(2, ru, H, F, xn)[0]
+    gdev, udev = accel.d2h(np.empty(F, np.float32), gd), accel.d2h(np.empty(F, np.float32), ud)
+    assert relerr(gdev, g) <= 1e-5 and relerr(udev, u) <= 1e-5
+    # the second stage is checked on the device's own g/u (a rounding flip in g would move a quant)
+    assert relerr(eager, orc.matmul_q8_from_f32(2, rd, F, H, orc.act_produce(act, gdev, udev))[0]) <= 1e-5
+    accel.graph_begin()
+    block()
+    graph = accel.graph_end()
+    for rep in range(3):
+        accel.h2d(yd, np.zeros(H, np.float32))
+        accel.gemv_dev("t.ffn.gate", xd, 1, gd)      # eager work between replays, clobbers g
+        accel.sync()
+        accel.graph_launch(graph)
+        accel.sync()
+        assert np.array_equal(accel.d2h(np.empty(H, np.float32), yd), eager), f"replay {rep}"
+    accel.graph_destroy(graph)
+    for p in (xd, wd, gd, ud, yd):
+        accel.dev_free(p)
