@@ -101,6 +101,17 @@ def test_tuning_knobs_keep_results(accel, orc, synth, relerr, pkg):
         accel.tune("gemm_splitk", sk)
         assert relerr(accel.prefill_q8_gemm("t.tune", xs, 64, 256), ref) <= 1e-5
     accel.tune("gemm_splitk", 0)
+    # 256 x 128 tiles (8 waves per workgroup), both weight formats, ragged M and N
+    for ty, up in ((8, accel.upload_q8_0), (2, accel.upload_q4_0)):
+        raw = synth.make_weight(ty, 200, 1056, seed=13)
+        xs = synth.make_acts(300, 1056, seed=14)
+        assert up("t.tune8", raw, 1056, 200)
+        ref = orc.matmul_q8_from_f32(ty, raw, 1056, 200, xs)
+        for nw in (8, 4, 0):
+            accel.tune("gemm_nw", nw)
+            assert relerr(accel.prefill_q8_gemm("t.tune8", xs, 300, 200), ref) <= 1e-5, nw
+    with pytest.raises(pkg.SmxError):
+        accel.tune("gemm_nw", 3)
     with pytest.raises(pkg.SmxError):
         accel.tune("no_such_knob", 1)
     with pytest.raises(pkg.SmxError):
