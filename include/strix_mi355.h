@@ -171,6 +171,38 @@ void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
  * depend on them beyond fp32 summation order. */
 int smx_tune(smx_ctx* ctx, const char* knob, int value);
 
+/* ---- GGUF file -> resident weights: the loader side of the path, crates/strix-models/src/gguf.rs:104-238
+ *      (memory-mapped GGUF v2/v3: header, metadata, tensor index) and the upload loops of the models'
+ *      attach_accel (crates/strix-backend-cpu/src/mellum.rs:460-535, gemma.rs:415-470).  Host code;
+ *      smx_gguf_open / the accessors need no GPU.  Errors of smx_gguf_open go to err (may be NULL). ---- */
+typedef struct smx_gguf smx_gguf;
+int smx_gguf_open(const char* path, smx_gguf** out, char* err, size_t err_cap);
+void smx_gguf_close(smx_gguf* g);
+size_t smx_gguf_tensor_count(const smx_gguf* g);
+/* Tensor `index` in file order: name, ggml type number, dims in GGUF order (fastest first; at most
+ * dims_cap written), pointer to its bytes inside the mapping and their count (gguf.rs:217-238).
+ * Any out pointer may be NULL. */
+int smx_gguf_tensor(const smx_gguf* g, size_t index, const char** name, int* ggml_type, size_t* n_dims,
+                    size_t* dims, size_t dims_cap, const void** data, size_t* nbytes);
+int smx_gguf_find(const smx_gguf* g, const char* name, size_t* index);          /* 0: no such tensor */
+/* Metadata with the reference's widening rules (MetaValue::as_u64 / as_f32 / as_str, gguf.rs:43-72):
+ * 1 found, 0 no such key, <0 the value has another kind. */
+int smx_gguf_meta_u64(const smx_gguf* g, const char* key, uint64_t* value);
+int smx_gguf_meta_f32(const smx_gguf* g, const char* key, float* value);
+int smx_gguf_meta_str(const smx_gguf* g, const char* key, const char** value);
+/* attach_accel: every "*.weight" matrix (>= 2 dims; in_dim = dims[0], out_dim = the product of the
+ * rest) stored as Q4_0, Q8_0 or Q6_K is uploaded under its GGUF name; every layer whose
+ * blk.<il>.ffn_{gate,up,down}_exps.weight triple is Q8_0 or Q6_K becomes expert layer <il>.  Tensors in
+ * other encodings are left to the caller (see the host quantisers below).  Counts may be NULL. */
+int smx_gguf_attach(smx_ctx* ctx, const smx_gguf* g, size_t* n_weights, size_t* n_expert_layers);
+/* Host quantisers the reference uses to bring a tensor into a served format before upload
+ * (crates/strix-models/src/ggml_quant.rs:193-207 quantize_q8_0, :212-237 quantize_q4_0) and the
+ * dequantisers that feed them (:239-262, 401-430; ggml types 0 F32, 1 F16, 2 Q4_0, 8 Q8_0, 14 Q6_K).
+ * n elements, a multiple of the block size; out: n/32*34, n/32*18 bytes, n floats. */
+int smx_host_quantize_q8_0(const float* x, size_t n, void* out);
+int smx_host_quantize_q4_0(const float* x, size_t n, void* out);
+int smx_host_dequantize(int ggml_type, const void* bytes, size_t n, float* out);
+
 /* ---- per-kernel timing: the role of STRIX_PROF, decode.rs:25-69, 2190-2203,
  *      done with HIP events on the context's stream instead of host syncs ---- */
 int smx_prof_enable(smx_ctx* ctx, int on);   /* on: bracket each matmul kernel with an event pair */

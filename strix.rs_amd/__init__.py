@@ -32,7 +32,9 @@ EXPORTS = [
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
     "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused",
-    "smx_upload_moe_q6",
+    "smx_upload_moe_q6", "smx_gguf_open", "smx_gguf_close", "smx_gguf_tensor_count", "smx_gguf_tensor",
+    "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach",
+    "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -109,6 +111,21 @@ def load_library():
     L.smx_graph_launch.argtypes = [vp, vp]
     L.smx_graph_destroy.argtypes = [vp, vp]
     L.smx_graph_destroy.restype = None
+    L.smx_gguf_open.argtypes = [cp, C.POINTER(vp), cp, sz]
+    L.smx_gguf_close.argtypes = [vp]
+    L.smx_gguf_close.restype = None
+    L.smx_gguf_tensor_count.argtypes = [vp]
+    L.smx_gguf_tensor_count.restype = sz
+    L.smx_gguf_tensor.argtypes = [vp, sz, C.POINTER(cp), C.POINTER(i), C.POINTER(sz), C.POINTER(sz), sz, C.POINTER(vp),
+                                  C.POINTER(sz)]
+    L.smx_gguf_find.argtypes = [vp, cp, C.POINTER(sz)]
+    L.smx_gguf_meta_u64.argtypes = [vp, cp, C.POINTER(C.c_uint64)]
+    L.smx_gguf_meta_f32.argtypes = [vp, cp, C.POINTER(C.c_float)]
+    L.smx_gguf_meta_str.argtypes = [vp, cp, C.POINTER(cp)]
+    L.smx_gguf_attach.argtypes = [vp, vp, C.POINTER(sz), C.POINTER(sz)]
+    L.smx_host_quantize_q8_0.argtypes = [vp, sz, vp]
+    L.smx_host_quantize_q4_0.argtypes = [vp, sz, vp]
+    L.smx_host_dequantize.argtypes = [i, vp, sz, vp]
     _lib = L
     return L
 
@@ -119,6 +136,95 @@ def _p(a):
 
 def _c(a, dt):
     return np.ascontiguousarray(a, dtype=dt)
+
+
+class GgufFile:
+    """A memory-mapped GGUF file: metadata and tensor index (crates/strix-models/src/gguf.rs:104-238).
+    Needs no GPU."""
+
+    def __init__(self, path):
+        self._L = load_library()
+        h = C.c_void_p()
+        err = C.create_string_buffer(512)
+        rc = self._L.smx_gguf_open(str(path).encode(), C.byref(h), err, len(err))
+        if rc != SMX_OK:
+            raise SmxError(rc, err.value.decode())
+        self._h = h
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._L.smx_gguf_close(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()
+
+    def __len__(self):
+        return self._L.smx_gguf_tensor_count(self._h)
+
+    def tensor(self, index):
+        """(name, ggml_type, dims, bytes) of tensor `index`; bytes is a copy of its raw data."""
+        name, ty, nd, nb, data = C.c_char_p(), C.c_int(), C.c_size_t(), C.c_size_t(), C.c_void_p()
+        dims = (C.c_size_t * 8)()
+        rc = self._L.smx_gguf_tensor(self._h, index, C.byref(name), C.byref(ty), C.byref(nd), dims, 8, C.byref(data),
+                                     C.byref(nb))
+        if rc != SMX_OK:
+            raise IndexError(index)
+        raw = np.ctypeslib.as_array((C.c_uint8 * nb.value).from_address(data.value)).copy() if nb.value else np.empty(0, np.uint8)
+        return name.value.decode(), ty.value, [dims[d] for d in range(nd.value)], raw
+
+    def find(self, name):
+        idx = C.c_size_t()
+        return idx.value if self._L.smx_gguf_find(self._h, name.encode(), C.byref(idx)) == SMX_OK else None
+
+    def tensors(self):
+        return {t[0]: t for t in (self.tensor(i) for i in range(len(self)))}
+
+    def _meta(self, fn, key, out, what):
+        rc = fn(self._h, key.encode(), C.byref(out))
+        if rc == 0:
+            return None
+        if rc < 0:
+            raise TypeError(f"GGUF metadata {key!r} is not {what}")
+        return out.value
+
+    def meta_u64(self, key):
+        return self._meta(self._L.smx_gguf_meta_u64, key, C.c_uint64(), "an unsigned integer")
+
+    def meta_f32(self, key):
+        return self._meta(self._L.smx_gguf_meta_f32, key, C.c_float(), "a number")
+
+    def meta_str(self, key):
+        v = self._meta(self._L.smx_gguf_meta_str, key, C.c_char_p(), "a string")
+        return None if v is None else v.decode()
+
+
+def host_quantize_q8_0(x):
+    """f32 -> GGUF Q8_0 bytes (crates/strix-models/src/ggml_quant.rs:193-207)."""
+    x = _c(x, np.float32).reshape(-1)
+    out = np.empty(x.size // 32 * 34, np.uint8)
+    if load_library().smx_host_quantize_q8_0(_p(x), x.size, _p(out)) != SMX_OK:
+        raise ValueError("length must be a multiple of 32")
+    return out
+
+
+def host_quantize_q4_0(x):
+    """f32 -> GGUF Q4_0 bytes (ggml_quant.rs:212-237)."""
+    x = _c(x, np.float32).reshape(-1)
+    out = np.empty(x.size // 32 * 18, np.uint8)
+    if load_library().smx_host_quantize_q4_0(_p(x), x.size, _p(out)) != SMX_OK:
+        raise ValueError("length must be a multiple of 32")
+    return out
+
+
+def host_dequantize(ggml_type, raw, n):
+    """GGUF bytes -> f32 for F32, F16, Q4_0, Q8_0, Q6_K (ggml_quant.rs:239-262, 401-430)."""
+    raw = _c(raw, np.uint8)
+    out = np.empty(n, np.float32)
+    rc = load_library().smx_host_dequantize(int(ggml_type), _p(raw), n, _p(out))
+    if rc != SMX_OK:
+        raise ValueError(f"cannot dequantise ggml type {ggml_type} with {n} elements")
+    return out
 
 
 class Mi355WeightAccel:
@@ -188,6 +294,12 @@ class Mi355WeightAccel:
         gate, up, down = _c(gate, np.uint8), _c(up, np.uint8), _c(down, np.uint8)
         return self._check(self._L.smx_upload_moe_q6(self._h, layer, _p(gate), gate.size, _p(up), up.size,
                                                      _p(down), down.size, hidden, eff, ne))
+
+    def attach_gguf(self, gguf):
+        """The upload loop of the models' attach_accel (mellum.rs:460-535): returns (matrices, expert layers)."""
+        nw, nl = C.c_size_t(), C.c_size_t()
+        self._check(self._L.smx_gguf_attach(self._h, gguf._h, C.byref(nw), C.byref(nl)))
+        return nw.value, nl.value
 
     def evict(self, key):
         return self._check(self._L.smx_evict(self._h, key.encode()))

@@ -77,6 +77,19 @@ class Mi355WeightAccel final : public WeightAccel {
     bool upload_q8_0(const std::string& key, const uint8_t* b, size_t n, size_t in_dim, size_t out_dim) override {
         return ok(smx_upload_q8_0(ctx_, key.c_str(), b, n, in_dim, out_dim));
     }
+    // The upload loop of the models' attach_accel (mellum.rs:460-535) over a GGUF file: returns the
+    // number of adopted matrices plus expert layers.
+    size_t attach_gguf(const std::string& path) {
+        smx_gguf* g = nullptr;
+        char err[256] = {0};
+        const int rc = smx_gguf_open(path.c_str(), &g, err, sizeof err);
+        if (rc != SMX_OK) throw BackendError(rc, err);
+        size_t nw = 0, nl = 0;
+        const int ra = smx_gguf_attach(ctx_, g, &nw, &nl);
+        smx_gguf_close(g);
+        if (ra != SMX_OK) throw BackendError(ra, smx_last_error(ctx_));
+        return nw + nl;
+    }
     // accel.rs:185-196
     bool upload_moe_q6(size_t layer, const uint8_t* gate, size_t gate_n, const uint8_t* up, size_t up_n, const uint8_t* down,
                        size_t down_n, size_t hidden, size_t eff, size_t ne) {
