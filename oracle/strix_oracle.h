@@ -32,6 +32,16 @@
  *                The Q6_K x Q8 arithmetic is new (the reference's Q6_K kernels
  *                take f32 activations, kernels.rs:607-640): parity unpinned,
  *                pinned by the same brute-force checks.
+ *
+ *  Activation producers (rmsnorm, SwiGLU, GeGLU in front of a GEMV) and the
+ *  MoE chain follow crates/strix-backend-cpu/src/ops.rs:15-27, 74-87, 110-121
+ *  and mellum.rs:1623-1669.  Pinned by the reference's literal checks
+ *  (ops.rs:204-232, 260-276, 287-294) and float64 formulas.  Two deliberate
+ *  departures, both far inside the reference's own tolerances (1e-5 / 1e-3):
+ *  exp/tanh are fixed sequences of fp32 operations instead of libm calls, and
+ *  rmsnorm forms the mean of squares in double and rounds the scale once
+ *  (the reference sums in fp32 on the CPU and uses rsqrtf on the device), so
+ *  that the quantised int8 activations are reproducible bit for bit.
  */
 #ifndef STRIX_ORACLE_H
 #define STRIX_ORACLE_H
