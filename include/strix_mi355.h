@@ -154,6 +154,11 @@ int smx_gemv_fused(smx_ctx* ctx, const char* key, int act, const float* a, const
 
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                     const float* x_dev, float* y_dev);
+/* smx_moe_layer with the activations and the result on the device (y_dev: m x hidden floats); the
+ * routing tables still come from the host at every call, so it cannot be captured in a graph. */
+int smx_moe_layer_dev(smx_ctx* ctx, size_t layer, const float* xs_dev, size_t m, const size_t* plan,
+                      size_t nplan, const int32_t* slot_tok, const float* wslot, size_t slots,
+                      float* y_dev);
 
 /* ---- HIP graph capture of a sequence of `_dev` calls: the role of the reference's captured decode
  *      token (decode.rs:3053-3203), so a launch-bound chain of small GEMVs replays without per-launch

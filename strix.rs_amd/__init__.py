@@ -34,7 +34,7 @@ EXPORTS = [
     "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused",
     "smx_upload_moe_q6", "smx_gguf_open", "smx_gguf_close", "smx_gguf_tensor_count", "smx_gguf_tensor",
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach",
-    "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize",
+    "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -82,6 +82,7 @@ def load_library():
     L.smx_lm_head_argmax_rows.argtypes = [vp, cp, vp, sz, sz, vp]
     L.smx_moe_ffn.argtypes = [vp, sz, vp, vp, sz, vp, sz, C.c_float, vp, sz]
     L.smx_moe_layer.argtypes = [vp, sz, vp, sz, vp, sz, vp, vp, sz, vp, sz]
+    L.smx_moe_layer_dev.argtypes = [vp, sz, vp, sz, vp, sz, vp, vp, sz, vp]
     L.smx_dev_alloc.argtypes = [vp, sz, C.POINTER(vp)]
     L.smx_dev_free.argtypes = [vp, vp]
     L.smx_h2d.argtypes = [vp, vp, vp, sz]
@@ -373,6 +374,13 @@ class Mi355WeightAccel:
         ok = self._check(self._L.smx_moe_layer(self._h, layer, _p(xs), m, _p(plan), plan.shape[0],
                                                _p(slot_tok), _p(wslot), slot_tok.size, _p(y), y.size))
         return y if ok else None
+
+    def moe_layer_resident(self, layer, xs_dev, m, plan, slot_tok, wslot, y_dev):
+        """moe_layer_q8_dev with activations and result already on the device (enqueue only)."""
+        plan = _c(plan, np.uint64).reshape(-1, 3)
+        slot_tok, wslot = _c(slot_tok, np.int32), _c(wslot, np.float32)
+        return self._check(self._L.smx_moe_layer_dev(self._h, layer, xs_dev, m, _p(plan), plan.shape[0],
+                                                     _p(slot_tok), _p(wslot), slot_tok.size, y_dev))
 
     # -- parity instrumentation
     def quantize(self, x, k):

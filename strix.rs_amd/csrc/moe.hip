@@ -408,8 +408,10 @@ int smx_moe_ffn_dev(smx_ctx* c, size_t layer, const int32_t* ids, const float* w
     return moe_ffn_enqueue(c, it->second, ids, wexp, k, x_dev, y_dev, nullptr);
 }
 
-int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
-                  const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap) {
+// xs / y on the host (copied in and out, one sync) or, with on_device, device pointers (enqueue only).
+static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
+                          const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap,
+                          bool on_device) {
     if (!c) return SMX_ERR_ARG;
     if (!xs || !plan || !slot_tok || !wslot || !y) return fail(c, SMX_ERR_ARG, "moe_layer: null argument");
     auto it = c->moe.find(layer);
@@ -449,8 +451,12 @@ int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const siz
 
     SMX_HIP(c, hipSetDevice(c->device));
     int rc;
-    if ((rc = ensure(c, c->xf32, m * hidden * 4)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->yf32, m * hidden * 4)) != SMX_OK) return rc;
+    if (!on_device) {
+        if ((rc = ensure(c, c->xf32, m * hidden * 4)) != SMX_OK) return rc;
+        if ((rc = ensure(c, c->yf32, m * hidden * 4)) != SMX_OK) return rc;
+    }
+    const float* x_dev = on_device ? xs : (const float*)c->xf32.p;
+    float* y_dev = on_device ? y : (float*)c->yf32.p;
     if ((rc = ensure(c, c->xq, m * hidden)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->xd, m * nb * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->xs, m * nb * 4)) != SMX_OK) return rc;
@@ -467,7 +473,7 @@ int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const siz
     int8_t* aq = (int8_t*)(c->work.p + o_aq);
     float* ad = (float*)(c->work.p + o_ad);
     float* dy = (float*)(c->work.p + o_dy);
-    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
+    if (!on_device) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_st, slot_tok, slots * 4, hipMemcpyHostToDevice, c->stream));
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ws, wslot, slots * 4, hipMemcpyHostToDevice, c->stream));
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_tp, tok_ptr.data(), (m + 1) * 4, hipMemcpyHostToDevice, c->stream));
@@ -475,7 +481,7 @@ int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const siz
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t1, tiles_gu.data(), tiles_gu.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t2, tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
     // the host vectors above are pageable: the copies have completed when hipMemcpyAsync returns
-    rc = launch_actquant(c, (const float*)c->xf32.p, m, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+    rc = launch_actquant(c, x_dev, m, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
     if (rc != SMX_OK) return rc;
     {
         GemmArgs p = {};
@@ -514,12 +520,26 @@ int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const siz
         ProfScope ps(c, "moe_combine");
         hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((hidden + 255) / 256), (unsigned)m), dim3(256), 0, c->stream,
                            dy, (const int*)(c->tab.p + o_tp), (const int*)(c->tab.p + o_ts),
-                           (const float*)(c->tab.p + o_ws), (float*)c->yf32.p, (int)hidden);
+                           (const float*)(c->tab.p + o_ws), y_dev, (int)hidden);
         SMX_HIP(c, hipGetLastError());
     }
-    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, m * hidden * 4, hipMemcpyDeviceToHost, c->stream));
-    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    if (!on_device) {
+        SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, m * hidden * 4, hipMemcpyDeviceToHost, c->stream));
+        SMX_HIP(c, hipStreamSynchronize(c->stream));
+    }
     return SMX_OK;
+}
+
+int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
+                  const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap) {
+    return moe_layer_impl(c, layer, xs, m, plan, nplan, slot_tok, wslot, slots, y, y_cap, false);
+}
+
+int smx_moe_layer_dev(smx_ctx* c, size_t layer, const float* xs_dev, size_t m, const size_t* plan, size_t nplan,
+                      const int32_t* slot_tok, const float* wslot, size_t slots, float* y_dev) {
+    if (c && c->capturing)
+        return fail(c, SMX_ERR_ARG, "moe_layer_dev: the routing tables are copied from the host at every call and cannot be captured");
+    return moe_layer_impl(c, layer, xs_dev, m, plan, nplan, slot_tok, wslot, slots, y_dev, SIZE_MAX, true);
 }
 
 }  // extern "C"

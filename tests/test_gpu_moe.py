@@ -101,6 +101,26 @@ def test_moe_layer_matches_decode_path(accel, orc, synth, relerr, ne, hidden, ef
         assert relerr(y[t], yt) <= 2e-2
 
 
+def test_moe_layer_resident_equals_host_call(accel, synth, pkg):
+    ne, hidden, eff, k, m = 8, 256, 96, 3, 70
+    _layer(accel, synth, 9, ne, hidden, eff, seed=33)
+    ids, w = synth.zipf_routing(m, ne, k, seed=34)
+    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
+    xs = synth.make_acts(m, hidden, seed=35)
+    want = accel.moe_layer_q8_dev(9, xs, m, plan, slot_tok, wslot)
+    xd, yd = accel.dev_alloc(xs.nbytes), accel.dev_alloc(xs.nbytes)
+    accel.h2d(xd, xs)
+    assert accel.moe_layer_resident(9, xd, m, plan, slot_tok, wslot, yd)
+    assert np.array_equal(accel.d2h(np.empty_like(xs), yd), want)
+    accel.graph_begin()
+    with pytest.raises(pkg.SmxError):
+        accel.moe_layer_resident(9, xd, m, plan, slot_tok, wslot, yd)   # host tables: not capturable
+    accel.graph_destroy(accel.graph_end())
+    assert accel.moe_layer_resident(99, xd, m, plan, slot_tok, wslot, yd) is False
+    accel.dev_free(xd)
+    accel.dev_free(yd)
+
+
 def test_moe_layer_rejects_bad_plan(accel, synth, pkg):
     _layer(accel, synth, 8, 4, 64, 32, seed=2)
     xs = synth.make_acts(2, 64, seed=1)
