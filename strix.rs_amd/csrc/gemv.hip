@@ -29,12 +29,12 @@ struct GemvJobs {
     GemvJob job[SMX_GEMV_GROUP_MAX];
 };
 
-template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool FUSEQ, bool DUMP, int NT>
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT>
 __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, int m, int* __restrict__ dump,
                                                   int dump_per_row) {
     const int nw = NT / 64;
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FUSEQ, DUMP>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
+    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
@@ -42,22 +42,31 @@ namespace {
 
 // Launch geometry: slots per wave, pipeline depth, K-split, lanes per row, threads per workgroup.
 struct Geom {
+    bool prod = false;  // an activation producer runs in the staging
     int rpw, pre, ks, lpr, nt;
     unsigned grid;
     size_t lds;
 };
 
-template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool DUMP, int NT>
-int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump,
-               int dump_per_row) {
-    // one activation row: quantiser fused into the staging; several rows: staged from rows quantised once
-    auto k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, MT == 1, DUMP, NT>;
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT>
+int launch_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump, int dump_per_row) {
+    auto k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP, NT>;
     static size_t lds_set = 0;
     int rc = set_dyn_lds(c, k, g.lds, &lds_set);
     if (rc != SMX_OK) return rc;
     hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(NT), g.lds, c->stream, J, nblk, m, dump, dump_per_row);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
+}
+
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool DUMP, int NT>
+int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump,
+               int dump_per_row) {
+    // one activation row: quantiser fused into the staging (FQ 1), behind an activation producer if the
+    // caller asked for one (FQ 2: its own variant, so that the plain GEMV carries none of its code);
+    // several rows: staged from rows quantised once (FQ 0)
+    if (MT == 1 && !DUMP && g.prod) return launch_fq<Ops, MT, RPW, PRE, KS, LPR, (MT == 1 && !DUMP) ? 2 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
+    return launch_fq<Ops, MT, RPW, PRE, KS, LPR, MT == 1 ? 1 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
 }
 
 // The compiled variants (RPW, PRE, KS, LPR):
@@ -241,6 +250,7 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
     }
     const Weight& w0 = *ws[0];
     Geom g = pick_geom(c, w0.type, maxN, w0.nblk, 1, false, n);
+    g.prod = prod && prod->kind != SMX_ACT_NONE;
     if (g.lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "gemv: activation of %zu needs %zu bytes of LDS", w0.K, g.lds);
     return launch_jobs(c, w0.type, g, J, n, (int)w0.nblk, 1, 1, nullptr, 0, name);
 }

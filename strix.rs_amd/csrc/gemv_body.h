@@ -328,13 +328,15 @@ __device__ __forceinline__ float rms_scale(char* scratch, const float* x, int n,
 // Stage one activation row into LDS.  8 lanes per 32-block, one float4 / one packed dword each;
 // reductions inside the 8 lanes go over DPP.  With the quantiser fused, an activation producer
 // (X.prod: rmsnorm(x)*x2, silu(x)*x2, gelu_tanh(x)*x2; kernels.rs:101-226) runs on the values first.
-template <class Ops, bool FUSEQ>
+// FQ: 0 the row is pre-quantised, 1 fp32 row quantised here, 2 the same behind an activation producer.
+template <class Ops, int FQ>
 __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X, int t, bool zero) {
     const int nb32 = Ops::nb32(nblk);
     const int items = nb32 * 8;
     constexpr int SB = 2;  // items per thread requested before any is consumed
     float rs = 1.f;
-    if (FUSEQ && X.prod == SMX_ACT_RMSNORM) rs = rms_scale(tok, X.x + (size_t)t * nb32 * 32, nb32 * 32, X.eps);
+    constexpr bool FUSEQ = FQ != 0;
+    if (FQ == 2 && X.prod == SMX_ACT_RMSNORM) rs = rms_scale(tok, X.x + (size_t)t * nb32 * 32, nb32 * 32, X.eps);
     for (int i0 = threadIdx.x; i0 < items; i0 += blockDim.x * SB) {
         float4 v[SB], v2[SB];
         int pk[SB];
@@ -348,7 +350,7 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
                 v2[j] = make_float4(1.f, 1.f, 1.f, 1.f);
                 if (live) {
                     v[j] = ((const float4*)(X.x + (size_t)t * nb32 * 32))[i];
-                    if (X.x2) v2[j] = ((const float4*)(X.x2 + (size_t)t * nb32 * 32))[i];
+                    if (FQ == 2 && X.x2) v2[j] = ((const float4*)(X.x2 + (size_t)t * nb32 * 32))[i];
                 }
             } else {
                 if (live) pk[j] = ((const int*)(X.xq + (size_t)t * nb32 * 32))[i];
@@ -364,7 +366,7 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
             float d = 0.f;
             if (FUSEQ) {
                 float4 w = v[j];
-                if (X.prod != SMX_ACT_NONE) {
+                if (FQ == 2 && X.prod != SMX_ACT_NONE) {
 #pragma clang fp contract(off)
                     const float4 g = v2[j];
                     if (X.prod == SMX_ACT_RMSNORM) {
@@ -455,7 +457,7 @@ __device__ __forceinline__ void stage_prequant_all(char* smem, int tokb, int nbl
 // KS adjacent waves (same workgroup) form a group that shares each chunk: wave j of the group takes
 // passes j, j+KS, ...; with KS > 1 every group owns at most one chunk (the launcher guarantees
 // nchunks <= n_waves / KS) and the KS partial sums meet in LDS behind the staged activation.
-template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, bool FUSEQ, bool DUMP>
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP>
 __device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* __restrict__ y, int ldy, int nblk, int N,
                                           int m, int* __restrict__ dump, int dump_per_row, int wave_id, int n_waves) {
     extern __shared__ __align__(16) char smem[];
@@ -494,8 +496,8 @@ __device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* _
         if (l_chunk < nchunks) issue(k);
     SMX_STAMP(1);
 
-    if (FUSEQ) {
-        for (int t = 0; t < MT; t++) stage_token<Ops, true>(smem + t * tokb, nblk, X, t, t >= m);
+    if (FQ != 0) {
+        for (int t = 0; t < MT; t++) stage_token<Ops, FQ>(smem + t * tokb, nblk, X, t, t >= m);
     } else {
         stage_prequant_all<Ops, MT>(smem, tokb, nblk, X, m);
     }
