@@ -86,11 +86,20 @@ int matmul_host(smx_ctx* c, const char* key, const float* xs, size_t m, size_t i
     int rc;
     if ((rc = ensure(c, c->xf32, m * w->K * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
-    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
+    // small transfers go through pinned staging: a pageable hipMemcpyAsync costs ~10 us each way
+    const size_t xb = m * w->K * 4, yb = m * w->N * 4;
+    const bool pinned = xb + yb <= (size_t(8) << 20);
+    if (pinned) {
+        if ((rc = ensure_host(c, c->hx, xb)) != SMX_OK) return rc;
+        if ((rc = ensure_host(c, c->hy, yb)) != SMX_OK) return rc;
+        memcpy(c->hx.p, xs, xb);
+    }
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, pinned ? (const void*)c->hx.p : (const void*)xs, xb, hipMemcpyHostToDevice, c->stream));
     rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, force_gemm, nullptr);
     if (rc != SMX_OK) return rc;
-    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, m * w->N * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(pinned ? (void*)c->hy.p : (void*)y, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
+    if (pinned) memcpy(y, c->hy.p, yb);
     return SMX_OK;
 }
 
@@ -145,6 +154,12 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
     if ((rc = ensure(c, c->xf32, xbytes)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->yf32, ybytes)) != SMX_OK) return rc;
     (void)qbytes; (void)dbytes;
+    // small batches travel as ONE pinned transfer each way instead of two pageable copies per item
+    const bool pinned = xbytes + ybytes <= (size_t(8) << 20);
+    if (pinned) {
+        if ((rc = ensure_host(c, c->hx, xbytes)) != SMX_OK) return rc;
+        if ((rc = ensure_host(c, c->hy, ybytes)) != SMX_OK) return rc;
+    }
     size_t xo = 0, yo = 0;
     std::vector<size_t> yoff(n, 0);
     std::vector<float*> xdev(n, nullptr), ydev(n, nullptr);
@@ -154,10 +169,12 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
         xdev[i] = (float*)(c->xf32.p + xo);
         ydev[i] = (float*)(c->yf32.p + yo);
         yoff[i] = yo;
-        SMX_HIP(c, hipMemcpyAsync(xdev[i], xs[i], w->K * 4, hipMemcpyHostToDevice, c->stream));
+        if (pinned) memcpy(c->hx.p + xo, xs[i], w->K * 4);
+        else SMX_HIP(c, hipMemcpyAsync(xdev[i], xs[i], w->K * 4, hipMemcpyHostToDevice, c->stream));
         xo += (w->K * 4 + 255) & ~size_t(255);
         yo += (w->N * 4 + 255) & ~size_t(255);
     }
+    if (pinned && xo) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, c->hx.p, xo, hipMemcpyHostToDevice, c->stream));
     // consecutive items of one format and row length share a launch (up to 8 per launch)
     for (size_t i = 0; i < n;) {
         if (!ws[i]) { i++; continue; }
@@ -175,10 +192,17 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
         for (int k = 0; k < g; k++) status[idx[k]] = rc;
         i = j;
     }
-    for (size_t i = 0; i < n; i++)
-        if (ws[i] && status[i] == SMX_OK)
-            SMX_HIP(c, hipMemcpyAsync(ys[i], c->yf32.p + yoff[i], ws[i]->N * 4, hipMemcpyDeviceToHost, c->stream));
+    if (pinned) {
+        if (yo) SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yo, hipMemcpyDeviceToHost, c->stream));
+    } else {
+        for (size_t i = 0; i < n; i++)
+            if (ws[i] && status[i] == SMX_OK)
+                SMX_HIP(c, hipMemcpyAsync(ys[i], c->yf32.p + yoff[i], ws[i]->N * 4, hipMemcpyDeviceToHost, c->stream));
+    }
     SMX_HIP(c, hipStreamSynchronize(c->stream));  // the batch's single sync (decode.rs:3247)
+    if (pinned)
+        for (size_t i = 0; i < n; i++)
+            if (ws[i] && status[i] == SMX_OK) memcpy(ys[i], c->hy.p + yoff[i], ws[i]->N * 4);
     return SMX_OK;
 }
 
@@ -283,14 +307,19 @@ int smx_gemv_fused(smx_ctx* c, const char* key, int act, const float* a, const f
     if ((rc = ensure(c, c->yf32, w->N * 4)) != SMX_OK) return rc;
     float* a_dev = (float*)c->xf32.p;
     float* b_dev = b ? a_dev + w->K : nullptr;
-    SMX_HIP(c, hipMemcpyAsync(a_dev, a, w->K * 4, hipMemcpyHostToDevice, c->stream));
-    if (b) SMX_HIP(c, hipMemcpyAsync(b_dev, b, w->K * 4, hipMemcpyHostToDevice, c->stream));
+    const size_t xb = (b ? 2 : 1) * w->K * 4, yb = w->N * 4;
+    if ((rc = ensure_host(c, c->hx, xb)) != SMX_OK) return rc;
+    if ((rc = ensure_host(c, c->hy, yb)) != SMX_OK) return rc;
+    memcpy(c->hx.p, a, w->K * 4);
+    if (b) memcpy(c->hx.p + w->K * 4, b, w->K * 4);
+    SMX_HIP(c, hipMemcpyAsync(a_dev, c->hx.p, xb, hipMemcpyHostToDevice, c->stream));
     const float* xs[1] = {a_dev};
     float* ys[1] = {(float*)c->yf32.p};
     const ActProd prod = {act, b_dev, eps};
     if ((rc = launch_gemv_group(c, &w, xs, ys, 1, nullptr, &prod)) != SMX_OK) return rc;
-    SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, w->N * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
+    memcpy(y, c->hy.p, yb);
     return SMX_OK;
 }
 

@@ -44,6 +44,25 @@ int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
     return SMX_OK;
 }
 
+int ensure_host(smx_ctx* c, DevBuf& b, size_t bytes) {
+    if (bytes <= b.cap) return SMX_OK;
+    if (b.p) {
+        SMX_HIP(c, hipStreamSynchronize(c->stream));
+        SMX_HIP(c, hipHostFree(b.p));
+        b.p = nullptr;
+        b.cap = 0;
+    }
+    const size_t cap = (bytes + (size_t(1) << 16) - 1) & ~((size_t(1) << 16) - 1);
+    hipError_t e = hipHostMalloc((void**)&b.p, cap, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        b.p = nullptr;
+        return fail(c, SMX_ERR_NOMEM, "pinned host allocation of %zu bytes failed: %s", cap, hipGetErrorString(e));
+    }
+    b.cap = cap;
+    return SMX_OK;
+}
+
 ProfScope::ProfScope(smx_ctx* c_, const char* name) : c(c_) {
     if (!c->prof_on || c->capturing) return;
     hipEvent_t e0, e1;
@@ -218,6 +237,8 @@ void smx_destroy(smx_ctx* c) {
     }
     for (DevBuf* b : {&c->xf32, &c->xq, &c->xd, &c->xs, &c->yf32, &c->work, &c->work2, &c->tab})
         if (b->p) (void)hipFree(b->p);
+    for (DevBuf* b : {&c->hx, &c->hy})
+        if (b->p) (void)hipHostFree(b->p);
     for (auto& r : c->prof) {
         (void)hipEventDestroy(r.e0);
         (void)hipEventDestroy(r.e1);

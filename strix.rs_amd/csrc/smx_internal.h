@@ -71,6 +71,7 @@ struct smx_ctx {
     smx::DevBuf work;   // split-K partials, MoE intermediates, dumps
     smx::DevBuf work2;
     smx::DevBuf tab;    // small tables (ids, weights, tile tables)
+    smx::DevBuf hx, hy; // pinned HOST staging of the host-pointer calls' activations and results
 
     // tuning overrides (0 = automatic)
     int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
@@ -98,6 +99,8 @@ int hip_fail(smx_ctx* c, hipError_t e, const char* what);
     } while (0)
 
 int ensure(smx_ctx* c, DevBuf& b, size_t bytes);
+// the same for a pinned host buffer (hipHostMalloc)
+int ensure_host(smx_ctx* c, DevBuf& b, size_t bytes);
 
 // Raises a kernel's dynamic-LDS limit when it asks for more than the 48 KB default (remembered per
 // kernel so that replays and captured launches do not repeat the call).
