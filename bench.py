@@ -261,7 +261,7 @@ class Bench:
             acc.gemm_dev(name, xd, M, yd)
 
         ms, wall_ms = self._timed(step, steps, warmup)
-        kname = "gemm_i8_q4_0" if ty == Q4_0 else "gemm_i8_q8_0"
+        kname = {Q4_0: "gemm_i8_q4_0", Q8_0: "gemm_i8_q8_0", Q6_K: "gemm_i8_q6_k"}[ty]
         kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
         names = self.last_names
         acc.evict(name)
@@ -414,6 +414,8 @@ def main():
         ("gemm_q4_0_ffn_up", lambda: b.gemm("gemm_q4_0_ffn_up", Q4_0, 2048, 15360, 3840)),
         ("gemm_q8_0_ffn_down", lambda: b.gemm("gemm_q8_0_ffn_down", Q8_0, 2048, 3840, 15360)),
         ("gemm_q4_0_ffn_down", lambda: b.gemm("gemm_q4_0_ffn_down", Q4_0, 2048, 3840, 15360)),
+        ("gemm_q6_k_ffn_up", lambda: b.gemm("gemm_q6_k_ffn_up", Q6_K, 2048, 15360, 3840)),
+        ("gemm_q6_k_ffn_down", lambda: b.gemm("gemm_q6_k_ffn_down", Q6_K, 2048, 3840, 15360)),
         ("moe_decode", lambda: b.moe("moe_decode", 64, 2048, 768, 8, 1, layers=4)),
         ("moe_prefill_m512", lambda: b.moe("moe_prefill_m512", 64, 2048, 768, 8, 512, layers=1)),
     ]

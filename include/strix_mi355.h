@@ -69,8 +69,9 @@ int smx_upload_moe_q8(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_
                       const void* up, size_t up_nbytes, const void* down, size_t down_nbytes,
                       size_t hidden, size_t eff, size_t ne);
 /* WeightAccel::upload_moe_q6, accel.rs:185-196; decode.rs:2793-2831: the same tensors as Q6_K
- * superblocks (hidden and eff multiples of 256).  Such a layer is served by smx_moe_ffn (one token);
- * smx_moe_layer returns an error for it. */
+ * superblocks (hidden and eff multiples of 256).  Served by smx_moe_ffn (one token) and by
+ * smx_moe_layer[_dev] (grouped prefill; stands in for q6_gemm_moe, kernels.rs:1688-1735, and
+ * moe_layer_ffn, decode.rs:3552-3629). */
 int smx_upload_moe_q6(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_nbytes,
                       const void* up, size_t up_nbytes, const void* down, size_t down_nbytes,
                       size_t hidden, size_t eff, size_t ne);
@@ -95,8 +96,8 @@ int smx_gemv_batch(smx_ctx* ctx, size_t n, const char* const* keys, const float*
 
 /* ---- prefill GEMM ---- */
 /* WeightAccel::prefill_q8_gemm, accel.rs:213; decode.rs:3257-3297 (and the
- * Q4_0 GEMMs kernels.rs:481-601).  xs[m][in_dim] -> y[m][out_dim], any
- * resident Q4_0/Q8_0 weight, any m; split-K is chosen internally. */
+ * Q4_0 GEMMs kernels.rs:481-601, the Q6_K GEMM :1688-1735).  xs[m][in_dim] -> y[m][out_dim], any
+ * resident Q4_0/Q8_0/Q6_K weight, any m; split-K is chosen internally. */
 int smx_gemm(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim, float* y,
              size_t y_cap);
 /* WeightAccel::lm_head_argmax_rows, accel.rs:217; decode.rs:3631-3690.

@@ -63,8 +63,6 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restric
 int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm,
                    int32_t* dump) {
     if (m <= SMX_GEMV_MAX_M && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump);  // quantiser fused
-    if (w.type == kQ6_K)
-        return fail(c, SMX_ERR_LIMIT, "Q6_K weights are served by the GEMV path only (at most %d rows per call)", SMX_GEMV_MAX_M);
     int rc = ensure_act(c, m, w.K);
     if (rc != SMX_OK) return rc;
     rc = launch_actquant(c, xs_dev, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
@@ -220,7 +218,8 @@ int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t
     if ((rc = ensure(c, c->tab, m * 4)) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
     if (w->type == kQ6_K && m > SMX_GEMV_MAX_M) {
-        // Q6_K has no GEMM on this path: heads with more rows go through in GEMV-sized groups
+        // a Q6_K head is HBM-bound at these row counts: GEMV-sized groups re-read the weights once per
+        // 8 rows, which costs less than a GEMM whose 128-token tiles would be mostly empty
         rc = SMX_OK;
         for (size_t t = 0; t < m && rc == SMX_OK; t += SMX_GEMV_MAX_M) {
             const size_t mm = std::min<size_t>(SMX_GEMV_MAX_M, m - t);

@@ -13,6 +13,10 @@
 //     0x4B400000 so its i32 result, read as a float, is 12582912 + I exactly; one FMA with the
 //     exactly representable -dw*12582912 (dw is an f16 value) gives fl(dw*I) with no int->float
 //     conversion, a second FMA applies dx and accumulates: two VALU operations per output per block;
+//   * Q6_K weights (kernels.rs:1688-1735 q6_gemm_moe keeps them in their 210-byte form too): the 6-bit
+//     quants are widened to signed int8 (q - 32) while being staged, and because the format scales
+//     16-element sub-blocks each 32-block takes two v_mfma_i32_32x32x16_i8, one exact i32 per
+//     sub-block, each rescaled by its own d * sc (four VALU operations per output per 32-block);
 //   * split-K: grid.z slices of whole stages write fp32 partials that a second kernel sums in slice
 //     order (deterministic, unlike the reference's atomicAdd, kernels.rs:597).
 // Bound: dense int8 MFMA, 2*M*N*K operations.
@@ -34,12 +38,16 @@ constexpr int B_BYTES = 16 * GRP;           // 128 weight rows
 // per CU; NW = 4: 128 x 128, two per CU).  The larger tile reads 25 % fewer operand bytes per
 // operation through L2, which is what bounds the kernel after the epilogue FMAs.
 constexpr int a_bytes(int NW) { return 4 * NW * GRP; }
-constexpr int stage_bytes(int NW) { return a_bytes(NW) + B_BYTES + KB * 128 * 4 + KB * 32 * NW * 4; }
+constexpr int stage_bytes(int NW, bool q6 = false) { return a_bytes(NW) + B_BYTES + (q6 ? 2 : 1) * KB * 128 * 4 + KB * 32 * NW * 4; }
 constexpr float MAGIC_F = 12582912.f;       // 1.5 * 2^23
 constexpr int MAGIC_I = 0x4B400000;
 
 __device__ __forceinline__ float h2f_(uint16_t h) { return __half2float(__ushort_as_half(h)); }
 __device__ __forceinline__ unsigned sub8(unsigned x) { return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
+// four 6-bit quants (low nibbles in lo4, the two high bits in hi2) -> four signed bytes q - 32
+__device__ __forceinline__ unsigned q6_bytes(unsigned lo4, unsigned hi2) {
+    return (((lo4 & 0x0f0f0f0fu) | ((hi2 & 0x03030303u) << 4) | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+}
 
 // 64 lanes x 16 bytes from global memory straight into LDS (no register round trip): lane i's
 // bytes land at LDS byte address lds_base + 16 * i; lds_base is wave-uniform (M0).  Completion is
@@ -56,16 +64,24 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) {
     return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
 }
 
+// Operand fragments of one 32-block.  SUB = 1: one K = 32 MFMA per row tile, a lane holds 16 k of
+// its row; SUB = 2 (Q6_K): two K = 16 MFMAs, a lane holds 8 k of each 16-element sub-block.
+template <int SUB>
 struct GemmFrag {
-    v4i a;         // this wave's 32 tokens x 32 k
-    v4i b[4];      // 4 x (32 weight rows x 32 k)
-    float4 dx[4];  // activation scales of the 16 tokens this lane accumulates
-    float dw[4];   // weight scale of this lane's row in each of the 4 row tiles
+    v4i a;           // this wave's 32 tokens x 32 k
+    v4i b[4];        // 4 x (32 weight rows x 32 k)
+    float4 dx[4];    // activation scales of the 16 tokens this lane accumulates
+    float dw[4][SUB];  // weight scale of this lane's row in each of the 4 row tiles (per sub-block)
 };
 
-template <bool Q4, bool DUMP, int NW>
+constexpr int FMT_Q8 = 0, FMT_Q4 = 1, FMT_Q6 = 2;
+
+template <int FMT, bool DUMP, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmArgs p) {
-    constexpr int BM = 32 * NW, A_BYTES = a_bytes(NW), STAGE_BYTES = stage_bytes(NW);
+    constexpr bool Q4 = FMT == FMT_Q4, Q6 = FMT == FMT_Q6;
+    static_assert(!Q6 || NW == 4, "the Q6_K staging map is written for 256 threads");
+    constexpr int SUB = Q6 ? 2 : 1;  // scaled sub-blocks per 32-block
+    constexpr int BM = 32 * NW, A_BYTES = a_bytes(NW), STAGE_BYTES = stage_bytes(NW, Q6);
     constexpr int BG = 16 / NW;  // 8-row groups of B each wave stages
     constexpr int WS = 8 / NW;   // weight scales per thread per stage
     extern __shared__ __align__(16) char smem[];
@@ -102,13 +118,18 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     const int g_rowlo = lane >> 3, g_chunk = ((lane & 7) - g_rowlo) & 7;
     const int q_bi = lane & 3, q_rowlo = lane >> 2;   // Q4_0 B: lane = [row:4][block:2], 64 contiguous bytes per row
     constexpr int QG = Q4 ? 8 / NW : 1;  // Q4_0 B: 16-byte blocks per thread per stage
+    // Q6_K B: thread = [row:7][p:1]; per stage (one half of a superblock) it reads ql[16p..], ql[32 + 16p..]
+    // and qh[16p..] of that half and makes the four 16-byte chunks 2j + p, j = 0..3 (ggml_quant.rs:417-426)
+    const int q6_row = tid >> 1, q6_p = tid & 1;
     unsigned a_off[4], b_off[Q4 ? QG : BG];  // element offsets; the launcher keeps M*K and N*K below 2^31
 #pragma unroll
     for (int ps = 0; ps < 4; ps++) {
         const int ti = min(tok0 + (ps * NW + wave) * 8 + g_rowlo, M_end - 1);
         a_off[ps] = (unsigned)(p.a_rowmap ? p.a_rowmap[ti] : ti) * (unsigned)K;
     }
-    if (!Q4) {
+    if (Q6) {
+        b_off[0] = (unsigned)min(row0 + q6_row, N_end - 1) * (unsigned)(p.nb >> 3);  // first superblock of the row
+    } else if (!Q4) {
 #pragma unroll
         for (int ps = 0; ps < BG; ps++)
             b_off[ps] = (unsigned)min(row0 + (ps * NW + wave) * 8 + g_rowlo, N_end - 1) * (unsigned)K;
@@ -122,14 +143,15 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     const int sr = tid & (BM - 1), sh = tid / BM;
     const int wr = tid & 127, wh = tid >> 7;
     const bool w_valid = row0 + wr < N_end, x_valid = tok0 + sr < M_end;
-    const size_t scw_base = (size_t)min(row0 + wr, N_end - 1) * p.nb;
+    const size_t scw_base = (size_t)min(row0 + wr, N_end - 1) * (Q6 ? p.nb >> 3 : p.nb);
     size_t scx_base;
     {
         const int ti = min(tok0 + sr, M_end - 1);
         scx_base = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * p.nb;
     }
-    uint4 rb[QG];       // Q4_0 only
-    uint16_t rsw[WS];   // raw weight scales (f16), row wr
+    uint4 rb[Q6 ? 3 : QG];  // Q4_0 / Q6_K quants on their way through registers
+    uint16_t rsw[WS];   // raw weight scales (f16), row wr (Q6_K: rsw[0] = d of the superblock)
+    unsigned rsc = 0;   // Q6_K: the four sub-block scales 4 * wh .. 4 * wh + 3 of the stage, row wr
     float rsx0, rsx1;   // activation scales of blocks 2*sh, 2*sh+1, token sr
 
     // issue every global read of stage s; the register-staged parts are written by finish_stage
@@ -141,7 +163,13 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
 #pragma unroll
         for (int ps = 0; ps < 4; ps++) load_to_lds16(p.xq + a_off[ps] + koff, sA + ps * NW * GRP);
-        if (!Q4) {
+        if (Q6) {
+            const size_t sbi = (size_t)b_off[0] + (s >> 1);
+            const char* ql = (const char*)op.wquants + sbi * 128 + (s & 1) * 64 + q6_p * 16;
+            rb[0] = *(const uint4*)ql;
+            rb[1] = *(const uint4*)(ql + 32);
+            rb[2] = *(const uint4*)((const char*)op.wqh + sbi * 64 + (s & 1) * 32 + q6_p * 16);
+        } else if (!Q4) {
 #pragma unroll
             for (int ps = 0; ps < BG; ps++)
                 load_to_lds16((const int8_t*)op.wquants + b_off[ps] + koff, sB + ps * NW * GRP);
@@ -151,8 +179,13 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
             for (int ps = 0; ps < QG; ps++) rb[ps] = ((const uint4*)op.wquants)[b_off[ps] + bq];
         }
         // branch-free and unconverted, so that nothing here waits for a load before the MFMA work
+        if (Q6) {
+            rsw[0] = op.wscales[scw_base + (s >> 1)];
+            rsc = *(const unsigned*)(op.wsc + (scw_base + (s >> 1)) * 16 + (s & 1) * 8 + wh * 4);
+        } else {
 #pragma unroll
-        for (int j = 0; j < WS; j++) rsw[j] = op.wscales[scw_base + min(blk0 + wh * WS + j, p.nb - 1)];
+            for (int j = 0; j < WS; j++) rsw[j] = op.wscales[scw_base + min(blk0 + wh * WS + j, p.nb - 1)];
+        }
         rsx0 = p.xd[scx_base + min(blk0 + 2 * sh, p.nb - 1)];
         rsx1 = p.xd[scx_base + min(blk0 + 2 * sh + 1, p.nb - 1)];
     };
@@ -160,8 +193,27 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     auto finish_stage = [&](int buf, int s) {
         char* sB = smem + buf * STAGE_BYTES + A_BYTES;
         float* sdw = (float*)(sB + B_BYTES);
-        float* sdx = sdw + KB * 128;
+        float* sdx = sdw + SUB * KB * 128;
         const int blk0 = s * KB;
+        if (Q6) {
+            const int r = q6_row;
+            const int off = (r >> 3) * GRP + (r & 7) * 128;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint4 q = rb[j & 1], h = rb[2];
+                const int ls = (j >> 1) * 4, hs = 2 * j;
+                uint4 o;
+                o.x = q6_bytes(q.x >> ls, h.x >> hs);
+                o.y = q6_bytes(q.y >> ls, h.y >> hs);
+                o.z = q6_bytes(q.z >> ls, h.z >> hs);
+                o.w = q6_bytes(q.w >> ls, h.w >> hs);
+                *(uint4*)(sB + off + ((2 * j + q6_p + r) & 7) * 16) = o;  // elements 32j + 16p .. + 15 of the stage
+            }
+            const float d = w_valid ? h2f_(rsw[0]) : 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++)  // d * sc is exact in fp32 (11 x 8 significant bits)
+                sdw[(wh * 4 + j) * 128 + wr] = d * (float)(int)(signed char)(rsc >> (8 * j));
+        }
         if (Q4) {
 #pragma unroll
             for (int ps = 0; ps < QG; ps++) {
@@ -177,9 +229,11 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
                 *(uint4*)(sB + off + ((2 * q_bi + 1 + r) & 7) * 16) = hi;  // elements 16..31
             }
         }
+        if (!Q6) {
 #pragma unroll
-        for (int j = 0; j < WS; j++)
-            sdw[(wh * WS + j) * 128 + wr] = (w_valid && blk0 + wh * WS + j < p.nb) ? h2f_(rsw[j]) : 0.f;
+            for (int j = 0; j < WS; j++)
+                sdw[(wh * WS + j) * 128 + wr] = (w_valid && blk0 + wh * WS + j < p.nb) ? h2f_(rsw[j]) : 0.f;
+        }
         sdx[(2 * sh) * BM + sr] = (x_valid && blk0 + 2 * sh < p.nb) ? rsx0 : 0.f;
         sdx[(2 * sh + 1) * BM + sr] = (x_valid && blk0 + 2 * sh + 1 < p.nb) ? rsx1 : 0.f;
     };
@@ -199,19 +253,35 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     int frag_lane[KB];
 #pragma unroll
     for (int bi = 0; bi < KB; bi++) frag_lane[bi] = (col >> 3) * GRP + (col & 7) * 128 + ((2 * bi + half + col) & 7) * 16;
+    // Q6_K: a lane takes bytes 8 * half .. + 7 of BOTH 16-byte chunks of the block (the order of k
+    // inside an MFMA does not matter as long as both operands use the same one)
+    const int frag6 = (col >> 3) * GRP + (col & 7) * 128 + half * 8;
 
-    auto read_frag = [&](GemmFrag& f, int buf, int bi) {
+    auto read_frag = [&](GemmFrag<SUB>& f, int buf, int bi) {
         const char* sA = smem + buf * STAGE_BYTES;
         const char* sB = sA + A_BYTES;
         const float* sdw = (const float*)(sB + B_BYTES);
-        const float* sdx = sdw + KB * 128;
-        f.a = *(const v4i*)(sA + wave * 4 * GRP + frag_lane[bi]);
+        const float* sdx = sdw + SUB * KB * 128;
 #pragma unroll
         for (int g = 0; g < 4; g++) f.dx[g] = *(const float4*)(sdx + bi * BM + wave * 32 + g * 8 + half * 4);
+        if (Q6) {
+            const int o0 = frag6 + ((2 * bi + col) & 7) * 16, o1 = frag6 + ((2 * bi + 1 + col) & 7) * 16;
+            const int2 a0 = *(const int2*)(sA + wave * 4 * GRP + o0), a1 = *(const int2*)(sA + wave * 4 * GRP + o1);
+            f.a = v4i{a0.x, a0.y, a1.x, a1.y};
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-            f.b[nt] = *(const v4i*)(sB + nt * 4 * GRP + frag_lane[bi]);
-            f.dw[nt] = sdw[bi * 128 + nt * 32 + col];
+            for (int nt = 0; nt < 4; nt++) {
+                const int2 b0 = *(const int2*)(sB + nt * 4 * GRP + o0), b1 = *(const int2*)(sB + nt * 4 * GRP + o1);
+                f.b[nt] = v4i{b0.x, b0.y, b1.x, b1.y};
+#pragma unroll
+                for (int jj = 0; jj < SUB; jj++) f.dw[nt][jj] = sdw[(2 * bi + jj) * 128 + nt * 32 + col];
+            }
+        } else {
+            f.a = *(const v4i*)(sA + wave * 4 * GRP + frag_lane[bi]);
+#pragma unroll
+            for (int nt = 0; nt < 4; nt++) {
+                f.b[nt] = *(const v4i*)(sB + nt * 4 * GRP + frag_lane[bi]);
+                f.dw[nt][0] = sdw[bi * 128 + nt * 32 + col];
+            }
         }
     };
 
@@ -219,20 +289,31 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     // FMAs of nt so that the matrix pipe and the vector ALU overlap within the wave.  The empty asm
     // statements pin the order: without them the FMAs of a whole stage sink below its 16 MFMAs,
     // whose results (256 registers) then spill.
-    auto compute = [&](const GemmFrag& f, int blk) {
+    // unit u = row tile u / SUB, sub-block u % SUB
+    auto mfma_unit = [&](const GemmFrag<SUB>& f, int u) -> v16i {
+        if (Q6) {
+            const int nt = u >> 1, jj = u & 1;
+            const long a = ((long)(unsigned)f.a[2 * jj]) | ((long)f.a[2 * jj + 1] << 32);
+            const long b = ((long)(unsigned)f.b[nt][2 * jj]) | ((long)f.b[nt][2 * jj + 1] << 32);
+            return __builtin_amdgcn_mfma_i32_32x32x16_i8(a, b, cmagic, 0, 0, 0);
+        }
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a, f.b[u], cmagic, 0, 0, 0);
+    };
+    auto compute = [&](const GemmFrag<SUB>& f, int blk) {
         const float dxr[16] = {f.dx[0].x, f.dx[0].y, f.dx[0].z, f.dx[0].w, f.dx[1].x, f.dx[1].y, f.dx[1].z, f.dx[1].w,
                                f.dx[2].x, f.dx[2].y, f.dx[2].z, f.dx[2].w, f.dx[3].x, f.dx[3].y, f.dx[3].z, f.dx[3].w};
         v16i d[2];
-        d[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a, f.b[0], cmagic, 0, 0, 0);
+        d[0] = mfma_unit(f, 0);
 #pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-            if (nt + 1 < 4) {
-                d[(nt + 1) & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.a, f.b[nt + 1], cmagic, 0, 0, 0);
-                asm volatile("" : "+v"(d[(nt + 1) & 1]));
+        for (int u = 0; u < 4 * SUB; u++) {
+            const int nt = u / SUB, jj = u % SUB;
+            if (u + 1 < 4 * SUB) {
+                d[(u + 1) & 1] = mfma_unit(f, u + 1);
+                asm volatile("" : "+v"(d[(u + 1) & 1]));
             }
-            const v16i dn = d[nt & 1];
-            const float dw = f.dw[nt];
-            const float ndw = -dw * MAGIC_F;  // exact: dw has an 11-bit significand
+            const v16i dn = d[u & 1];
+            const float dw = f.dw[nt][jj];
+            const float ndw = -dw * MAGIC_F;  // exact: dw has at most 18 significant bits (f16, or f16 x int8)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[nt][i] = fmaf(dxr[i], fmaf(dw, __int_as_float(dn[i]), ndw), acc[nt][i]);
             asm volatile("" : "+v"(acc[nt][0]), "+v"(acc[nt][1]), "+v"(acc[nt][2]), "+v"(acc[nt][3]), "+v"(acc[nt][4]),
@@ -245,7 +326,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
                 for (int i = 0; i < 16; i++) {
                     const int tok = tok0 + wave * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
                     if (tok < M_end && row < N_end && blk < p.nb)
-                        p.dump[((size_t)tok * p.N + row) * p.nb + blk] = dn[i] - MAGIC_I;
+                        p.dump[((size_t)tok * p.N + row) * (SUB * p.nb) + SUB * blk + jj] = dn[i] - MAGIC_I;
                 }
             }
         }
@@ -264,7 +345,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const int buf = (s - s_begin) & 1;
         if (s + 1 < s_end) issue_stage(buf ^ 1, s + 1);
         if (wave_live) {
-        GemmFrag f0, f1;
+        GemmFrag<SUB> f0, f1;
         read_frag(f0, buf, 0);
         read_frag(f1, buf, 1);
         __builtin_amdgcn_sched_barrier(0);
@@ -320,11 +401,11 @@ static int pick_splitk(int slots, int tiles, int nstages) {
     return std::max(1, std::min(z, 16));
 }
 
-template <bool Q4, bool DUMP, int NW>
+template <int FMT, bool DUMP, int NW>
 static int launch_gemm_variant(smx_ctx* c, const GemmArgs& p, dim3 grid) {
-    auto k = gemm_i8_kernel<Q4, DUMP, NW>;
+    auto k = gemm_i8_kernel<FMT, DUMP, NW>;
     static size_t lds_set = 0;
-    const size_t lds = 2 * stage_bytes(NW);
+    const size_t lds = 2 * stage_bytes(NW, FMT == FMT_Q6);
     int rc = set_dyn_lds(c, k, lds, &lds_set);
     if (rc != SMX_OK) return rc;
     hipLaunchKernelGGL(k, grid, dim3(64 * NW), lds, c->stream, p);
@@ -332,14 +413,23 @@ static int launch_gemm_variant(smx_ctx* c, const GemmArgs& p, dim3 grid) {
     return SMX_OK;
 }
 
+GemmOperand gemm_operand(const Weight& w, float* out) {
+    GemmOperand o = {};
+    o.wscales = w.scales;
+    o.wquants = w.quants;
+    o.out = out;
+    o.wqh = w.qh;
+    o.wsc = w.sc;
+    return o;
+}
+
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y, int32_t* dump) {
-    if (w.type != kQ4_0 && w.type != kQ8_0) return fail(c, SMX_ERR_ARG, "gemm: weight type %d not supported", (int)w.type);
+    if (w.type != kQ4_0 && w.type != kQ8_0 && w.type != kQ6_K) return fail(c, SMX_ERR_ARG, "gemm: weight type %d not supported", (int)w.type);
     if (m > (size_t(1) << 24) || w.N > (size_t(1) << 24) || w.K > (size_t(1) << 20) || m * w.K >= (size_t(1) << 31) ||
         w.N * w.K >= (size_t(1) << 31))
         return fail(c, SMX_ERR_LIMIT, "gemm: shape m=%zu N=%zu K=%zu exceeds the kernel's index range", m, w.N, w.K);
     GemmArgs p = {};
-    p.op[0].wscales = w.scales;
-    p.op[0].wquants = w.quants;
+    p.op[0] = gemm_operand(w, y);
     p.xq = xq;
     p.xd = xd;
     p.a_rowmap = nullptr;
@@ -348,10 +438,10 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     p.M = (int)m;
     p.N = (int)w.N;
     p.ldo = (int)w.N;
-    p.nb = (int)w.nblk;
+    p.nb = (int)(w.K / 32);
     // 128 x 128 tiles, two workgroups per CU; 256 x 128 (one 8-wave workgroup per CU) measures slower
     int nw = 4;
-    if (c->tune_gemm_nw == 4 || c->tune_gemm_nw == 8) nw = c->tune_gemm_nw;
+    if (w.type != kQ6_K && (c->tune_gemm_nw == 4 || c->tune_gemm_nw == 8)) nw = c->tune_gemm_nw;
     const int bm = 32 * nw;
     p.tiles_m = (p.M + bm - 1) / bm;
     p.tiles_n = (p.N + BN - 1) / BN;
@@ -370,14 +460,16 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     }
     const dim3 grid((unsigned)T, 1, (unsigned)Z);
     {
-        ProfScope ps(c, w.type == kQ4_0 ? "gemm_i8_q4_0" : "gemm_i8_q8_0");
+        ProfScope ps(c, w.type == kQ4_0 ? "gemm_i8_q4_0" : w.type == kQ6_K ? "gemm_i8_q6_k" : "gemm_i8_q8_0");
         int rc;
-        if (w.type == kQ4_0) {
-            if (dump) rc = nw == 8 ? launch_gemm_variant<true, true, 8>(c, p, grid) : launch_gemm_variant<true, true, 4>(c, p, grid);
-            else rc = nw == 8 ? launch_gemm_variant<true, false, 8>(c, p, grid) : launch_gemm_variant<true, false, 4>(c, p, grid);
+        if (w.type == kQ6_K) {
+            rc = dump ? launch_gemm_variant<FMT_Q6, true, 4>(c, p, grid) : launch_gemm_variant<FMT_Q6, false, 4>(c, p, grid);
+        } else if (w.type == kQ4_0) {
+            if (dump) rc = nw == 8 ? launch_gemm_variant<FMT_Q4, true, 8>(c, p, grid) : launch_gemm_variant<FMT_Q4, true, 4>(c, p, grid);
+            else rc = nw == 8 ? launch_gemm_variant<FMT_Q4, false, 8>(c, p, grid) : launch_gemm_variant<FMT_Q4, false, 4>(c, p, grid);
         } else {
-            if (dump) rc = nw == 8 ? launch_gemm_variant<false, true, 8>(c, p, grid) : launch_gemm_variant<false, true, 4>(c, p, grid);
-            else rc = nw == 8 ? launch_gemm_variant<false, false, 8>(c, p, grid) : launch_gemm_variant<false, false, 4>(c, p, grid);
+            if (dump) rc = nw == 8 ? launch_gemm_variant<FMT_Q8, true, 8>(c, p, grid) : launch_gemm_variant<FMT_Q8, true, 4>(c, p, grid);
+            else rc = nw == 8 ? launch_gemm_variant<FMT_Q8, false, 8>(c, p, grid) : launch_gemm_variant<FMT_Q8, false, 4>(c, p, grid);
         }
         if (rc != SMX_OK) return rc;
     }
@@ -393,10 +485,13 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
 
 // Grouped GEMM over a tile table (MoE prefill): one launch covers every expert; grid.y selects
 // one of `nops` weight/output pairs that share the activation rows (gate and up).
-int launch_gemm_grouped(smx_ctx* c, const GemmArgs& args, int ntiles, int nops, const char* name) {
+int launch_gemm_grouped(smx_ctx* c, QType type, const GemmArgs& args, int ntiles, int nops, const char* name) {
     if (ntiles <= 0) return SMX_OK;
     ProfScope ps(c, name);
-    return launch_gemm_variant<false, false, 4>(c, args, dim3((unsigned)ntiles, (unsigned)nops, 1));
+    const dim3 grid((unsigned)ntiles, (unsigned)nops, 1);
+    if (type == kQ6_K) return launch_gemm_variant<FMT_Q6, false, 4>(c, args, grid);
+    if (type == kQ8_0) return launch_gemm_variant<FMT_Q8, false, 4>(c, args, grid);
+    return fail(c, SMX_ERR_ARG, "grouped gemm: weight type %d not supported", (int)type);
 }
 
 }  // namespace smx

@@ -418,8 +418,6 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
     if (it == c->moe.end()) return SMX_NOT_RESIDENT;
     const MoeLayer& L = it->second;
     const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
-    if (L.type != kQ8_0)
-        return fail(c, SMX_ERR_LIMIT, "moe_layer: layer %zu holds Q6_K experts, which only the one-token path (moe_ffn) serves", layer);
     if (m == 0 || slots == 0) return fail(c, SMX_ERR_ARG, "moe_layer: m %zu, slots %zu", m, slots);  // decode.rs:1622
     if (y_cap < m * hidden) return fail(c, SMX_ERR_ARG, "moe_layer: output capacity %zu < %zu", y_cap, m * hidden);
     if (slots > (size_t(1) << 24) || m > 65535 || m * hidden >= (size_t(1) << 31) || slots * eff >= (size_t(1) << 31) ||
@@ -485,8 +483,8 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
     if (rc != SMX_OK) return rc;
     {
         GemmArgs p = {};
-        p.op[0] = {L.gate.scales, L.gate.quants, g};
-        p.op[1] = {L.up.scales, L.up.quants, u};
+        p.op[0] = gemm_operand(L.gate, g);
+        p.op[1] = gemm_operand(L.up, u);
         p.xq = (const int8_t*)c->xq.p;
         p.xd = (const float*)c->xd.p;
         p.a_rowmap = (const int*)(c->tab.p + o_st);  // slot -> token: the gather of kernels.rs:1162-1171
@@ -496,14 +494,14 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
         p.nb = (int)nb;
         p.ldo = (int)eff;
         p.stages_per_slice = (int)((nb + 3) / 4);
-        rc = launch_gemm_grouped(c, p, (int)tiles_gu.size(), 2, "moe_gemm_gate_up");
+        rc = launch_gemm_grouped(c, L.type, p, (int)tiles_gu.size(), 2, "moe_gemm_gate_up");
         if (rc != SMX_OK) return rc;
     }
     rc = silu_mul_quant(c, g, u, eff, slots, eff, aq, ad);
     if (rc != SMX_OK) return rc;
     {
         GemmArgs p = {};
-        p.op[0] = {L.down.scales, L.down.quants, dy};
+        p.op[0] = gemm_operand(L.down, dy);
         p.op[1] = p.op[0];
         p.xq = aq;
         p.xd = ad;
@@ -513,7 +511,7 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
         p.nb = (int)enb;
         p.ldo = (int)hidden;
         p.stages_per_slice = (int)((enb + 3) / 4);
-        rc = launch_gemm_grouped(c, p, (int)tiles_dn.size(), 1, "moe_gemm_down");
+        rc = launch_gemm_grouped(c, L.type, p, (int)tiles_dn.size(), 1, "moe_gemm_down");
         if (rc != SMX_OK) return rc;
     }
     {

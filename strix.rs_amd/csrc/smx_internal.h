@@ -123,9 +123,11 @@ struct ProfScope {
 
 // One weight/output pair of a GEMM launch.
 struct GemmOperand {
-    const uint16_t* wscales;  // f16 [rows][nb]
-    const void* wquants;      // Q8_0: i8 [rows][K];  Q4_0: 16 B [rows][nb]
+    const uint16_t* wscales;  // f16 [rows][nb]; Q6_K: the superblock scale d, [rows][nb / 8]
+    const void* wquants;      // Q8_0: i8 [rows][K];  Q4_0: 16 B [rows][nb];  Q6_K: ql, 128 B [rows][nb / 8]
     float* out;               // [M][ldo] (split-K: Z such planes)
+    const void* wqh;          // Q6_K: qh, 64 B [rows][nb / 8]
+    const int8_t* wsc;        // Q6_K: sub-block scales, 16 per superblock
 };
 // One 128 x 128 output tile of a grouped GEMM.
 struct GemmTile {
@@ -139,7 +141,7 @@ struct GemmArgs {
     const float* xd;        // [*][nb]
     const int* a_rowmap;    // optional: activation row index per logical row (MoE gather)
     const GemmTile* tiles;  // optional tile table; dense tiling when null
-    int* dump;              // optional [M][N][nb]
+    int* dump;              // optional [M][N][nb] (Q6_K: [M][N][2 * nb], one per 16-element sub-block)
     int M, N, nb, ldo;
     int tiles_m, tiles_n;
     int stages_per_slice;   // stages (of 4 blocks) each grid.z slice covers
@@ -166,6 +168,8 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);
 
-int launch_gemm_grouped(smx_ctx* c, const GemmArgs& args, int ntiles, int nops, const char* name);
+int launch_gemm_grouped(smx_ctx* c, QType type, const GemmArgs& args, int ntiles, int nops, const char* name);
+// the weight planes of w as a GEMM operand writing to out
+GemmOperand gemm_operand(const Weight& w, float* out);
 
 }  // namespace smx

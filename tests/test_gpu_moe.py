@@ -53,10 +53,6 @@ def test_moe_ffn_q6k_experts_stagewise(accel, orc, synth, relerr, pkg, ne, hidde
     assert relerr(y, ry2) <= TOL
     assert relerr(y, ry) <= 2e-2
     assert np.array_equal(accel.moe_ffn(7, ids[0], w[0], x), y)
-    # the grouped prefill entry point does not take Q6_K layers
-    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
-    with pytest.raises(pkg.SmxError):
-        accel.moe_layer_q8_dev(7, x[None, :], 1, plan, slot_tok, wslot)
     with pytest.raises(pkg.SmxError):
         accel.upload_moe_q6(8, gate[:-1], up, down, hidden, eff, ne)
 
@@ -73,13 +69,13 @@ def test_moe_ffn_declines_and_errors(accel, synth, pkg):
         accel.moe_ffn(4, [0], [1.0], x, sgate=0.5)
 
 
-def _moe_layer_oracle(orc, gate, up, down, hidden, eff, ne, xs, ids, w, dev_aq=None):
+def _moe_layer_oracle(orc, gate, up, down, hidden, eff, ne, xs, ids, w, ty=8):
     """Per token: the decode oracle with experts in ascending slot (= ascending expert) order."""
     m = xs.shape[0]
     out = np.zeros((m, hidden), np.float32)
     for t in range(m):
         order = np.argsort(ids[t], kind="stable")
-        out[t], _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[t][order], w[t][order], xs[t])
+        out[t], _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[t][order], w[t][order], xs[t], ty=ty)
     return out
 
 
@@ -98,6 +94,25 @@ def test_moe_layer_matches_decode_path(accel, orc, synth, relerr, ne, hidden, ef
     for t in (0, m // 2, m - 1):
         order = np.argsort(ids[t], kind="stable")
         yt = accel.moe_ffn(7, ids[t][order], w[t][order], xs[t])
+        assert relerr(y[t], yt) <= 2e-2
+
+
+@pytest.mark.parametrize("ne,hidden,eff,k,m", [(4, 256, 256, 2, 5), (8, 512, 256, 3, 37), (16, 512, 768, 4, 300)])
+def test_moe_layer_q6k_experts(accel, orc, synth, relerr, ne, hidden, eff, k, m):
+    """Grouped prefill over Q6_K expert layers (q6_gemm_moe, kernels.rs:1688-1735; moe_layer_ffn,
+    decode.rs:3552-3629): the table-driven GEMM with Q6_K sub-block scales."""
+    gate, up, down = synth.make_moe_q6(ne, hidden, eff, seed=hidden + m)
+    assert accel.upload_moe_q6(17, gate, up, down, hidden, eff, ne)
+    ids, w = synth.zipf_routing(m, ne, k, seed=19)
+    xs = synth.make_acts(m, hidden, seed=20)
+    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
+    y = accel.moe_layer_q8_dev(17, xs, m, plan, slot_tok, wslot)
+    assert y.shape == (m, hidden)
+    ref = _moe_layer_oracle(orc, gate, up, down, hidden, eff, ne, xs, ids, w, ty=14)
+    assert relerr(y, ref) <= 2e-2     # re-quantised intermediate, as for Q8_0 experts above
+    for t in (0, m // 2, m - 1):
+        order = np.argsort(ids[t], kind="stable")
+        yt = accel.moe_ffn(17, ids[t][order], w[t][order], xs[t])
         assert relerr(y[t], yt) <= 2e-2
 
 
