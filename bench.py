@@ -279,14 +279,14 @@ class Bench:
         }
 
     # ------------------------------------------------------------------ MoE
-    def moe(self, name, ne, hidden, eff, k, m, layers, steps=None, warmup=None):
+    def moe(self, name, ne, hidden, eff, k, m, layers, steps=None, warmup=None, ty=Q8_0):
         """Decode (m == 1): rotate over `layers` resident layers (320 MB each) so expert reads are
         cache-cold.  Prefill (m > 1): one layer, m tokens grouped by expert."""
         acc, sy = self.acc, self.synth
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
-        gate, up, down = sy.make_moe_q8(ne, hidden, eff, seed=3000)
+        gate, up, down = (sy.make_moe_q6 if ty == Q6_K else sy.make_moe_q8)(ne, hidden, eff, seed=3000)
         for l in range(layers):
-            assert acc.upload_moe_q8(l, gate, up, down, hidden, eff, ne)
+            assert (acc.upload_moe_q6 if ty == Q6_K else acc.upload_moe_q8)(l, gate, up, down, hidden, eff, ne)
         del gate, up, down
         out = {"workload": name, "shape": {"experts": ne, "hidden": hidden, "eff": eff, "top_k": k, "M": m}}
         if m == 1:
@@ -303,7 +303,7 @@ class Bench:
             kus, nk = self._kernel_avg_us(step, steps, warmup, "moe_gemv")
             acc.dev_free(xd)
             acc.dev_free(yd)
-            wbytes = k * 3 * eff * (hidden // 32) * 34
+            wbytes = k * 3 * eff * (hidden // 256 * 210 if ty == Q6_K else hidden // 32 * 34)
             gbs = wbytes * steps / (ms * 1e-3) / 1e9
             out.update({"expert_weight_bytes": wbytes, "layers_rotated": layers, "steps": steps,
                         "ms_per_step": ms / steps, "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
@@ -418,6 +418,8 @@ def main():
         ("gemm_q6_k_ffn_down", lambda: b.gemm("gemm_q6_k_ffn_down", Q6_K, 2048, 3840, 15360)),
         ("moe_decode", lambda: b.moe("moe_decode", 64, 2048, 768, 8, 1, layers=4)),
         ("moe_prefill_m512", lambda: b.moe("moe_prefill_m512", 64, 2048, 768, 8, 512, layers=1)),
+        ("moe_decode_q6_k", lambda: b.moe("moe_decode_q6_k", 64, 2048, 768, 8, 1, layers=4, ty=Q6_K)),
+        ("moe_prefill_m512_q6_k", lambda: b.moe("moe_prefill_m512_q6_k", 64, 2048, 768, 8, 512, layers=1, ty=Q6_K)),
     ]
     for name, fn in plans:
         if want(name):
