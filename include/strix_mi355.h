@@ -201,9 +201,15 @@ int smx_gguf_meta_str(const smx_gguf* g, const char* key, const char** value);
  * blk.<il>.ffn_{gate,up,down}_exps.weight triple is Q8_0 or Q6_K becomes expert layer <il>.  Tensors in
  * other encodings are left to the caller (see the host quantisers below).  Counts may be NULL. */
 int smx_gguf_attach(smx_ctx* ctx, const smx_gguf* g, size_t* n_weights, size_t* n_expert_layers);
+/* One matrix re-encoded on the host as Q8_0 (target_type 8) or Q4_0 (2) and uploaded under `key`
+ * (NULL: its own name): the reference's repacks of tensors in an encoding the device path does not
+ * serve (gemma3n.rs:455-470, a Q4_K token_embd becomes the Q8_0 lm_head) or that should be lighter
+ * (qwen35.rs:741-760, Q8_0 -> Q4_0).  0: no such tensor. */
+int smx_gguf_upload_as(smx_ctx* ctx, const smx_gguf* g, const char* tensor, const char* key, int target_type);
 /* Host quantisers the reference uses to bring a tensor into a served format before upload
  * (crates/strix-models/src/ggml_quant.rs:193-207 quantize_q8_0, :212-237 quantize_q4_0) and the
- * dequantisers that feed them (:239-262, 401-430; ggml types 0 F32, 1 F16, 2 Q4_0, 8 Q8_0, 14 Q6_K).
+ * dequantisers that feed them (:128-430; ggml types 0 F32, 1 F16, 2 Q4_0, 3 Q4_1, 6 Q5_0, 7 Q5_1,
+ * 8 Q8_0, 12 Q4_K, 13 Q5_K, 14 Q6_K; others return SMX_ERR_LIMIT, as the reference's dequantize errs).
  * n elements, a multiple of the block size; out: n/32*34, n/32*18 bytes, n floats. */
 int smx_host_quantize_q8_0(const float* x, size_t n, void* out);
 int smx_host_quantize_q4_0(const float* x, size_t n, void* out);

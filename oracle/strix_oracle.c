@@ -69,8 +69,8 @@ uint16_t orc_f32_to_f16(float f) {
 
 int orc_block_elems(int type) {
     switch (type) {
-        case ORC_Q4_0: case ORC_Q8_0: return 32;
-        case ORC_Q6_K: return 256;
+        case ORC_Q4_0: case ORC_Q8_0: case ORC_Q4_1: case ORC_Q5_0: case ORC_Q5_1: return 32;
+        case ORC_Q6_K: case ORC_Q4_K: case ORC_Q5_K: return 256;
         default: return 0;
     }
 }
@@ -80,6 +80,11 @@ int orc_block_bytes(int type) {
         case ORC_Q4_0: return 18;  /* ggml_quant.rs:111 */
         case ORC_Q8_0: return 34;  /* :115 */
         case ORC_Q6_K: return 210; /* :121 */
+        case ORC_Q4_1: return 20;  /* :112 */
+        case ORC_Q5_0: return 22;  /* :113 */
+        case ORC_Q5_1: return 24;  /* :114 */
+        case ORC_Q4_K: return 144; /* :119 */
+        case ORC_Q5_K: return 176; /* :120 */
         default: return 0;
     }
 }
@@ -141,6 +146,97 @@ static void dequant_q6_k(const uint8_t* bytes, float* out, size_t nblocks) {
     }
 }
 
+/* ggml_quant.rs:265-275 */
+static void dequant_q4_1(const uint8_t* bytes, float* out, size_t nblocks) {
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t* blk = bytes + b * 20;
+        float d = rd_f16(blk), m = rd_f16(blk + 2);
+        const uint8_t* qs = blk + 4;
+        for (int j = 0; j < 16; j++) {
+            out[b * 32 + j] = d * (float)(qs[j] & 0x0F) + m;
+            out[b * 32 + j + 16] = d * (float)(qs[j] >> 4) + m;
+        }
+    }
+}
+
+/* the fifth bits of values j and j + 16 of a Q5 block, ggml_quant.rs:284-285 */
+static inline void q5_high_bits(uint32_t qh, int j, int* h0, int* h1) {
+    *h0 = (int)(((qh >> j) << 4) & 0x10);
+    *h1 = (int)((qh >> (j + 12)) & 0x10);
+}
+
+/* ggml_quant.rs:278-292 */
+static void dequant_q5_0(const uint8_t* bytes, float* out, size_t nblocks) {
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t* blk = bytes + b * 22;
+        float d = rd_f16(blk);
+        uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+        const uint8_t* qs = blk + 6;
+        for (int j = 0; j < 16; j++) {
+            int h0, h1;
+            q5_high_bits(qh, j, &h0, &h1);
+            out[b * 32 + j] = (float)((int)((qs[j] & 0x0F) | h0) - 16) * d;
+            out[b * 32 + j + 16] = (float)((int)((qs[j] >> 4) | h1) - 16) * d;
+        }
+    }
+}
+
+/* ggml_quant.rs:295-311 */
+static void dequant_q5_1(const uint8_t* bytes, float* out, size_t nblocks) {
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t* blk = bytes + b * 24;
+        float d = rd_f16(blk), m = rd_f16(blk + 2);
+        uint32_t qh = (uint32_t)blk[4] | ((uint32_t)blk[5] << 8) | ((uint32_t)blk[6] << 16) | ((uint32_t)blk[7] << 24);
+        const uint8_t* qs = blk + 8;
+        for (int j = 0; j < 16; j++) {
+            int h0, h1;
+            q5_high_bits(qh, j, &h0, &h1);
+            out[b * 32 + j] = (float)((qs[j] & 0x0F) | h0) * d + m;
+            out[b * 32 + j + 16] = (float)((qs[j] >> 4) | h1) * d + m;
+        }
+    }
+}
+
+/* 6-bit scale and min of sub-block j out of the 12 packed bytes, ggml_quant.rs:316-324 */
+static inline void scale_min_k4(int j, const uint8_t* q, int* sc, int* mn) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *mn = q[j + 4] & 63;
+    } else {
+        *sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
+        *mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+    }
+}
+
+/* ggml_quant.rs:328-359 (fifth = 0) and :365-400 (fifth = 1: Q5_K, 32 more bytes of high bits) */
+static void dequant_q45_k(const uint8_t* bytes, float* out, size_t nblocks, int fifth) {
+    const size_t bb = fifth ? 176 : 144;
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t* blk = bytes + b * bb;
+        float d = rd_f16(blk), dmin = rd_f16(blk + 2);
+        const uint8_t* scales = blk + 4;
+        const uint8_t* qh = blk + 16;
+        const uint8_t* qs = blk + (fifth ? 48 : 16);
+        float* ob = out + b * 256;
+        for (int chunk = 0; chunk < 4; chunk++) {
+            int sc1, m1, sc2, m2;
+            scale_min_k4(2 * chunk, scales, &sc1, &m1);
+            scale_min_k4(2 * chunk + 1, scales, &sc2, &m2);
+            float d1 = d * (float)sc1, min1 = dmin * (float)m1, d2 = d * (float)sc2, min2 = dmin * (float)m2;
+            const uint8_t* q = qs + chunk * 32;
+            for (int l = 0; l < 32; l++) {
+                float lo = (float)(q[l] & 0x0F), hi = (float)(q[l] >> 4);
+                if (fifth) {
+                    if (qh[l] & (1u << (2 * chunk))) lo += 16.0f;
+                    if (qh[l] & (2u << (2 * chunk))) hi += 16.0f;
+                }
+                ob[chunk * 64 + l] = d1 * lo - min1;
+                ob[chunk * 64 + 32 + l] = d2 * hi - min2;
+            }
+        }
+    }
+}
+
 int orc_dequantize(int type, const uint8_t* bytes, size_t nbytes, float* out, size_t n) {
     int be = orc_block_elems(type);
     if (be == 0 || n % (size_t)be != 0) return -1; /* ggml_quant.rs:142-146 */
@@ -150,6 +246,11 @@ int orc_dequantize(int type, const uint8_t* bytes, size_t nbytes, float* out, si
         case ORC_Q8_0: dequant_q8_0(bytes, out, nblocks); break;
         case ORC_Q4_0: dequant_q4_0(bytes, out, nblocks); break;
         case ORC_Q6_K: dequant_q6_k(bytes, out, nblocks); break;
+        case ORC_Q4_1: dequant_q4_1(bytes, out, nblocks); break;
+        case ORC_Q5_0: dequant_q5_0(bytes, out, nblocks); break;
+        case ORC_Q5_1: dequant_q5_1(bytes, out, nblocks); break;
+        case ORC_Q4_K: dequant_q45_k(bytes, out, nblocks, 0); break;
+        case ORC_Q5_K: dequant_q45_k(bytes, out, nblocks, 1); break;
         default: return -1;
     }
     return 0;

@@ -33,6 +33,13 @@
  *                take f32 activations, kernels.rs:607-640): parity unpinned,
  *                pinned by the same brute-force checks.
  *
+ *  Requantisation sources — Q4_1, Q5_0, Q5_1, Q4_K, Q5_K decode
+ *                (ggml_quant.rs:265-400), host-side only.  Q4_K and Q5_K are
+ *                pinned by the literal blocks of ggml_quant.rs:472-494, 525-541;
+ *                Q4_1, Q5_0, Q5_1 have no reference test: PARITY UNPINNED BY THE
+ *                REFERENCE, pinned bit for bit against a vectorised numpy decoder
+ *                written from the published block layouts.
+ *
  *  Activation producers (rmsnorm, SwiGLU, GeGLU in front of a GEMV) and the
  *  MoE chain follow crates/strix-backend-cpu/src/ops.rs:15-27, 74-87, 110-121
  *  and mellum.rs:1623-1669.  Pinned by the reference's literal checks
@@ -52,7 +59,8 @@
 extern "C" {
 #endif
 
-enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q6_K = 14 }; /* GGML type ids, ggml_quant.rs:569-572 */
+enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q6_K = 14, /* GGML type ids, ggml_quant.rs:43-58 */
+       ORC_Q4_1 = 3, ORC_Q5_0 = 6, ORC_Q5_1 = 7, ORC_Q4_K = 12, ORC_Q5_K = 13 }; /* dequantised only (requantisation sources) */
 
 /* ---- half precision (exact conversions; `half` crate semantics) ---- */
 float orc_f16_to_f32(uint16_t h);

@@ -33,7 +33,7 @@ EXPORTS = [
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
     "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused",
     "smx_upload_moe_q6", "smx_gguf_open", "smx_gguf_close", "smx_gguf_tensor_count", "smx_gguf_tensor",
-    "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach",
+    "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
@@ -127,6 +127,7 @@ def load_library():
     L.smx_host_quantize_q8_0.argtypes = [vp, sz, vp]
     L.smx_host_quantize_q4_0.argtypes = [vp, sz, vp]
     L.smx_host_dequantize.argtypes = [i, vp, sz, vp]
+    L.smx_gguf_upload_as.argtypes = [vp, vp, C.c_char_p, C.c_char_p, i]
     _lib = L
     return L
 
@@ -301,6 +302,12 @@ class Mi355WeightAccel:
         nw, nl = C.c_size_t(), C.c_size_t()
         self._check(self._L.smx_gguf_attach(self._h, gguf._h, C.byref(nw), C.byref(nl)))
         return nw.value, nl.value
+
+    def upload_as(self, gguf, tensor, target_type, key=None):
+        """One matrix of the file re-encoded as Q8_0 (8) or Q4_0 (2) on the host and uploaded
+        (gemma3n.rs:455-470, qwen35.rs:741-760)."""
+        return self._check(self._L.smx_gguf_upload_as(self._h, gguf._h, tensor.encode(),
+                                                      key.encode() if key else None, int(target_type)))
 
     def evict(self, key):
         return self._check(self._L.smx_evict(self._h, key.encode()))

@@ -386,6 +386,46 @@ int smx_gguf_attach(smx_ctx* c, const smx_gguf* g, size_t* n_weights, size_t* n_
     return SMX_OK;
 }
 
+// One tensor re-encoded on the host and uploaded: the reference's repacks of a tensor whose encoding
+// the device path does not serve (gemma3n.rs:455-470: a Q4_K token_embd becomes a Q8_0 lm_head) or
+// that the caller wants lighter (qwen35.rs:741-760: Q8_0 -> Q4_0).  Rows are converted in slabs so
+// that the fp32 form of a large tensor never exists as a whole.
+int smx_gguf_upload_as(smx_ctx* c, const smx_gguf* g, const char* tensor, const char* key, int target_type) {
+    if (!c) return SMX_ERR_ARG;
+    if (!g || !tensor) return smx::fail(c, SMX_ERR_ARG, "gguf_upload_as: null argument");
+    if (target_type != 2 && target_type != 8)
+        return smx::fail(c, SMX_ERR_ARG, "gguf_upload_as: target type %d (2 = Q4_0 or 8 = Q8_0)", target_type);
+    auto it = g->index.find(tensor);
+    if (it == g->index.end()) return SMX_NOT_RESIDENT;
+    const smx_gguf::Tensor& t = g->tensors[it->second];
+    if (t.dims.size() < 2) return smx::fail(c, SMX_ERR_ARG, "gguf_upload_as: %s is not a matrix", tensor);
+    const BlockFormat* f = format_of(t.type);
+    const size_t in_dim = (size_t)t.dims[0];
+    size_t out_dim = 1;
+    for (size_t d = 1; d < t.dims.size(); d++) out_dim *= (size_t)t.dims[d];
+    if (!f || in_dim % f->elems != 0 || in_dim % 32 != 0)
+        return smx::fail(c, SMX_ERR_ARG, "gguf_upload_as: %s has row length %zu in encoding %u", tensor, in_dim, t.type);
+    const uint8_t* src = g->map + g->data_offset + t.offset;
+    const char* name = key ? key : tensor;
+    if ((int)t.type == target_type)
+        return target_type == 2 ? smx_upload_q4_0(c, name, src, t.nbytes, in_dim, out_dim)
+                                : smx_upload_q8_0(c, name, src, t.nbytes, in_dim, out_dim);
+    const size_t row_src = in_dim / f->elems * f->bytes, row_dst = in_dim / 32 * (target_type == 2 ? 18 : 34);
+    const size_t slab = std::max<size_t>(1, (size_t(8) << 20) / in_dim);  // rows per slab: 32 MB of floats
+    std::vector<float> tmp(std::min(slab, out_dim) * in_dim);
+    std::vector<uint8_t> enc(out_dim * row_dst);
+    for (size_t r0 = 0; r0 < out_dim; r0 += slab) {
+        const size_t rows = std::min(slab, out_dim - r0);
+        int rc = smx_host_dequantize((int)t.type, src + r0 * row_src, rows * in_dim, tmp.data());
+        if (rc != SMX_OK) return smx::fail(c, rc, "gguf_upload_as: encoding %u of %s has no dequantiser", t.type, tensor);
+        rc = target_type == 2 ? smx_host_quantize_q4_0(tmp.data(), rows * in_dim, enc.data() + r0 * row_dst)
+                              : smx_host_quantize_q8_0(tmp.data(), rows * in_dim, enc.data() + r0 * row_dst);
+        if (rc != SMX_OK) return smx::fail(c, rc, "gguf_upload_as: quantiser failed on %s", tensor);
+    }
+    return target_type == 2 ? smx_upload_q4_0(c, name, enc.data(), enc.size(), in_dim, out_dim)
+                            : smx_upload_q8_0(c, name, enc.data(), enc.size(), in_dim, out_dim);
+}
+
 // ---- host quantisers / dequantisers (n a multiple of the block size) ----
 
 // ggml_quant.rs:193-207
@@ -481,6 +521,55 @@ int smx_host_dequantize(int ggml_type, const void* bytes, size_t n, float* out) 
                 ql += 64;
                 qh += 32;
                 sc += 8;
+            }
+        }
+    } else if (ggml_type == 3 || ggml_type == 6 || ggml_type == 7) {
+        // Q4_1 (d, m, nibbles), Q5_0 (d, 32 fifth bits, nibbles), Q5_1 (d, m, fifth bits, nibbles):
+        // ggml_quant.rs:265-311.  Value i of the block: nibble i % 16 of byte i % 16's low (i < 16) or high half.
+        if (n % 32) return SMX_ERR_ARG;
+        const bool has_m = ggml_type != 6, has_h = ggml_type != 3;
+        const size_t bb = 2 + (has_m ? 2 : 0) + (has_h ? 4 : 0) + 16;
+        for (size_t b = 0; b < n / 32; b++, p += bb) {
+            const uint8_t* q = p + 2;
+            const float d = f16_to_f32((uint16_t)(p[0] | (p[1] << 8)));
+            float m = 0.f;
+            uint32_t hbits = 0;
+            if (has_m) { m = f16_to_f32((uint16_t)(q[0] | (q[1] << 8))); q += 2; }
+            if (has_h) { hbits = (uint32_t)q[0] | ((uint32_t)q[1] << 8) | ((uint32_t)q[2] << 16) | ((uint32_t)q[3] << 24); q += 4; }
+            for (int i = 0; i < 32; i++) {
+                const int nib = i < 16 ? (q[i] & 0x0f) : (q[i - 16] >> 4);
+                const int v = nib | (int)(((hbits >> i) & 1u) << 4);
+                if (ggml_type == 6) out[b * 32 + i] = (float)(v - 16) * d;   // symmetric: no min
+                else out[b * 32 + i] = (ggml_type == 3 ? d * (float)v : (float)v * d) + m;
+            }
+        }
+    } else if (ggml_type == 12 || ggml_type == 13) {
+        // Q4_K / Q5_K superblocks (ggml_quant.rs:328-400): d, dmin, 12 bytes holding eight 6-bit
+        // (scale, min) pairs, [Q5_K: 32 bytes of fifth bits,] 128 nibble bytes.  Sub-block s (32 values)
+        // takes the low (s even) or high (s odd) nibbles of bytes 32 * (s / 2) .. + 31, bit s of the
+        // fifth-bit byte l, and y = (d * sc_s) * q - dmin * m_s.
+        if (n % 256) return SMX_ERR_ARG;
+        const bool k5 = ggml_type == 13;
+        for (size_t b = 0; b < n / 256; b++, p += k5 ? 176 : 144) {
+            const float d = f16_to_f32((uint16_t)(p[0] | (p[1] << 8))), dmin = f16_to_f32((uint16_t)(p[2] | (p[3] << 8)));
+            const uint8_t *pk = p + 4, *hb = p + 16, *qs = p + (k5 ? 48 : 16);
+            for (int s = 0; s < 8; s++) {
+                int sc, mn;
+                if (s < 4) {
+                    sc = pk[s] & 63;
+                    mn = pk[s + 4] & 63;
+                } else {  // low four bits in bytes 8..11, the upper two in the top bits of bytes 0..7
+                    sc = (pk[s + 4] & 0x0f) | ((pk[s - 4] >> 6) << 4);
+                    mn = (pk[s + 4] >> 4) | ((pk[s] >> 6) << 4);
+                }
+                const float ds = d * (float)sc, ms = dmin * (float)mn;
+                const uint8_t* q = qs + 32 * (s >> 1);
+                float* y = out + b * 256 + s * 32;
+                for (int l = 0; l < 32; l++) {
+                    float v = (float)((s & 1) ? (q[l] >> 4) : (q[l] & 0x0f));
+                    if (k5 && ((hb[l] >> s) & 1)) v += 16.0f;
+                    y[l] = ds * v - ms;
+                }
             }
         }
     } else {

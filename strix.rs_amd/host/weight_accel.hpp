@@ -90,6 +90,17 @@ class Mi355WeightAccel final : public WeightAccel {
         if (ra != SMX_OK) throw BackendError(ra, smx_last_error(ctx_));
         return nw + nl;
     }
+    // One matrix of a GGUF file re-encoded on the host as Q8_0 (8) or Q4_0 (2) and uploaded under
+    // `key`: the repacks of gemma3n.rs:455-470 (Q4_K token_embd -> Q8_0 lm_head) and qwen35.rs:741-760.
+    bool upload_as(const std::string& path, const std::string& tensor, const std::string& key, int target_type) {
+        smx_gguf* g = nullptr;
+        char err[256] = {0};
+        const int rc = smx_gguf_open(path.c_str(), &g, err, sizeof err);
+        if (rc != SMX_OK) throw BackendError(rc, err);
+        const int ru = smx_gguf_upload_as(ctx_, g, tensor.c_str(), key.c_str(), target_type);
+        smx_gguf_close(g);
+        return ok(ru);
+    }
     // accel.rs:185-196
     bool upload_moe_q6(size_t layer, const uint8_t* gate, size_t gate_n, const uint8_t* up, size_t up_n, const uint8_t* down,
                        size_t down_n, size_t hidden, size_t eff, size_t ne) {

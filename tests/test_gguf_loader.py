@@ -89,8 +89,16 @@ def test_host_quantisers_match_the_oracle(pkg, orc, synth):
     h = np.arange(65536, dtype=np.uint16)
     f = pkg.host_dequantize(1, h.view(np.uint8), 65536)
     assert np.array_equal(f.view(np.uint32), h.view(np.float16).astype(np.float32).view(np.uint32))
+    # the encodings that only feed the requantisers (Q4_1, Q5_0, Q5_1, Q4_K, Q5_K), random bytes with sane scales
+    for ty, be, bb in ((3, 32, 20), (6, 32, 22), (7, 32, 24), (12, 256, 144), (13, 256, 176)):
+        raw = rng.integers(0, 256, (64, bb), dtype=np.uint8)
+        raw[:, 0:2] = rng.uniform(-0.1, 0.1, (64, 1)).astype(np.float16).view(np.uint8)
+        if ty != 6:
+            raw[:, 2:4] = rng.uniform(-0.1, 0.1, (64, 1)).astype(np.float16).view(np.uint8)
+        got, want = pkg.host_dequantize(ty, raw, 64 * be), orc.dequantize(ty, raw, 64 * be)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), ty
     with pytest.raises(ValueError):
-        pkg.host_dequantize(12, np.zeros(144, np.uint8), 256)   # Q4_K is not served
+        pkg.host_dequantize(10, np.zeros(84, np.uint8), 256)    # Q2_K has no dequantiser (ggml_quant.rs:517-521)
     with pytest.raises(ValueError):
         pkg.host_quantize_q8_0(np.zeros(33, np.float32))
 
@@ -153,3 +161,33 @@ def test_attach_uploads_matrices_and_expert_layers(accel, pkg, orc, synth, reler
     f = pkg.host_dequantize(14, o, 96 * H)
     assert accel.upload_q8_0("output.q8", pkg.host_quantize_q8_0(f), H, 96)
     assert relerr(accel.gemv("output.q8", x, 96), orc.matmul_q8_from_f32(8, orc.quantize_q8_0(f), H, 96, x)[0]) <= 1e-5
+
+
+@pytest.mark.gpu
+def test_upload_as_requantises_unserved_encodings(accel, pkg, orc, synth, relerr, tmp_path):
+    """gemma3n.rs:455-470 (Q4_K token_embd -> Q8_0 lm_head) and qwen35.rs:741-760 (Q8_0 -> Q4_0) in one call."""
+    H, V = 512, 300
+    rng = np.random.default_rng(3)
+    k4 = rng.integers(0, 256, (V * H // 256, 144), dtype=np.uint8)
+    k4[:, 0:2] = rng.uniform(0.001, 0.02, (k4.shape[0], 1)).astype(np.float16).view(np.uint8)
+    k4[:, 2:4] = rng.uniform(0.001, 0.02, (k4.shape[0], 1)).astype(np.float16).view(np.uint8)
+    k4 = k4.reshape(-1)
+    d8 = synth.make_weight(8, 64, H, seed=3)
+    p = gw.write_gguf(tmp_path / "m.gguf", [], [("token_embd.weight", 12, [H, V], k4), ("blk.0.attn_q.weight", 8, [H, 64], d8),
+                                                 ("blk.0.attn_norm.weight", 0, [H], np.ones(H, np.float32).view(np.uint8))])
+    g = pkg.GgufFile(p)
+    x = synth.make_acts(1, H, seed=4)[0]
+    assert accel.upload_as(g, "token_embd.weight", 8, key="lm_head.q8")
+    want8 = orc.quantize_q8_0(orc.dequantize(12, k4, V * H))
+    assert relerr(accel.gemv("lm_head.q8", x, V), orc.matmul_q8_from_f32(8, want8, H, V, x)[0]) <= 1e-5
+    assert accel.upload_as(g, "blk.0.attn_q.weight", 2)                 # under its own name, lighter
+    want4 = orc.quantize_q4_0(orc.dequantize(8, d8, 64 * H))
+    assert relerr(accel.gemv("blk.0.attn_q.weight", x, 64), orc.matmul_q8_from_f32(2, want4, H, 64, x)[0]) <= 1e-5
+    assert accel.upload_as(g, "blk.0.attn_q.weight", 8, key="q.same")   # already in the target encoding: plain upload
+    assert relerr(accel.gemv("q.same", x, 64), orc.matmul_q8_from_f32(8, d8, H, 64, x)[0]) <= 1e-5
+    assert accel.upload_as(g, "no.such.tensor", 8) is False
+    with pytest.raises(pkg.SmxError):
+        accel.upload_as(g, "blk.0.attn_norm.weight", 8)                 # not a matrix
+    with pytest.raises(pkg.SmxError):
+        accel.upload_as(g, "token_embd.weight", 14)                     # no host quantiser for Q6_K
+    g.close()

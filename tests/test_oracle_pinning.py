@@ -64,6 +64,30 @@ def test_q6_k_decodes_known_values(orc):     # ggml_quant.rs:497-514
     assert y[0] == -11.0 and y[1] == -32.0 and y[32] == -32.0 and y.size == 256
 
 
+def test_q4_k_with_zero_min_decodes_to_scaled_nibbles(orc):   # ggml_quant.rs:472-494
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = f16_bytes(orc, 1.0)
+    blk[4] = 1                                   # sub-block 0: scale 1
+    blk[16:48] = np.arange(32) % 16              # low nibbles of the first 32 quant bytes
+    y = orc.dequantize(12, blk, 256)
+    assert y.size == 256 and np.abs(y[:32] - np.arange(32) % 16).max() < 1e-4
+
+
+def test_q5_k_first_value_uses_high_bit(orc):                 # ggml_quant.rs:525-541
+    blk = np.zeros(176, np.uint8)
+    blk[0:2] = f16_bytes(orc, 1.0)
+    blk[4] = 1
+    blk[16] = 0b00000001
+    blk[48] = 0x0F
+    y = orc.dequantize(13, blk, 256)
+    assert y.size == 256 and abs(y[0] - 31.0) < 1e-3 and y[32] == 0.0
+
+
+def test_unimplemented_quant_errors(orc):                     # ggml_quant.rs:517-521
+    with pytest.raises(ValueError):
+        orc.dequantize(10, np.zeros(84, np.uint8), 256)
+
+
 def test_rejects_bad_sizes(orc):             # ggml_quant.rs:562-565
     with pytest.raises(ValueError):
         orc.dequantize(Q8_0, np.zeros(34, np.uint8), 16)
@@ -102,6 +126,73 @@ def test_dequant_matches_independent_numpy(orc, synth, ty):
     d, q = (np_q4_ints if ty == Q4_0 else np_q8_ints)(raw, N, K)
     want = (d[:, :, None].astype(np.float32) * q.astype(np.float32)).reshape(N, K)
     assert np.array_equal(orc.dequantize(ty, raw, N * K).reshape(N, K), want)
+
+
+def _f16(b):
+    return np.ascontiguousarray(b).view(np.float16).astype(np.float32)[..., 0]
+
+
+def _np_q4_1_q5(ty, raw, n):
+    """Q4_1 / Q5_0 / Q5_1 as the published GGML block layouts describe them (vectorised, no loops):
+    value i = nibble (low halves first) | bit i of the 32-bit field << 4."""
+    bb = {3: 20, 6: 22, 7: 24}[ty]
+    b = raw.reshape(-1, bb)
+    d = _f16(b[:, 0:2])
+    pos = 2
+    m = np.zeros_like(d)
+    if ty in (3, 7):
+        m = _f16(b[:, 2:4])
+        pos = 4
+    hi = np.zeros((b.shape[0], 32), np.int64)
+    if ty in (6, 7):
+        bits = b[:, pos:pos + 4].copy().view("<u4")[:, 0].astype(np.int64)
+        hi = (bits[:, None] >> np.arange(32)[None, :]) & 1
+        pos += 4
+    qs = b[:, pos:pos + 16].astype(np.int64)
+    q = np.concatenate([qs & 15, qs >> 4], axis=1) | (hi << 4)
+    if ty == 6:
+        return ((q - 16).astype(np.float32) * d[:, None]).reshape(-1)[:n]
+    return (q.astype(np.float32) * d[:, None] + m[:, None]).reshape(-1)[:n]
+
+
+def _np_q45_k(ty, raw, n):
+    """Q4_K / Q5_K: scales and mins are 6-bit fields packed in 12 bytes (llama.cpp get_scale_min_k4)."""
+    bb = 144 if ty == 12 else 176
+    b = raw.reshape(-1, bb)
+    nb = b.shape[0]
+    d, dmin = _f16(b[:, 0:2]), _f16(b[:, 2:4])
+    p = b[:, 4:16].astype(np.int64)
+    sc = np.empty((nb, 8), np.int64)
+    mn = np.empty((nb, 8), np.int64)
+    sc[:, :4], mn[:, :4] = p[:, 0:4] & 63, p[:, 4:8] & 63
+    sc[:, 4:] = (p[:, 8:12] & 15) | ((p[:, 0:4] >> 6) << 4)
+    mn[:, 4:] = (p[:, 8:12] >> 4) | ((p[:, 4:8] >> 6) << 4)
+    qs = b[:, bb - 128:].astype(np.int64).reshape(nb, 4, 32)
+    q = np.stack([qs & 15, qs >> 4], axis=2).reshape(nb, 8, 32)          # sub-block 2c: low, 2c+1: high
+    if ty == 13:
+        hb = b[:, 16:48].astype(np.int64)
+        q = q + (((hb[:, None, :] >> np.arange(8)[None, :, None]) & 1) << 4)
+    ds = d[:, None] * sc.astype(np.float32)
+    ms = dmin[:, None] * mn.astype(np.float32)
+    return (ds[:, :, None] * q.astype(np.float32) - ms[:, :, None]).reshape(-1)[:n]
+
+
+@pytest.mark.parametrize("ty", [3, 6, 7, 12, 13])
+def test_requantisation_sources_match_independent_numpy(orc, ty):
+    """Q4_1, Q5_0, Q5_1, Q4_K, Q5_K (ggml_quant.rs:265-400) only ever feed the host requantisers; the
+    reference tests pin one literal block of Q4_K and Q5_K (above), the rest is pinned here against a
+    vectorised decoder written from the format description."""
+    be, bb = {3: (32, 20), 6: (32, 22), 7: (32, 24), 12: (256, 144), 13: (256, 176)}[ty]
+    rng = np.random.default_rng(ty)
+    raw = rng.integers(0, 256, (40, bb), dtype=np.uint8)
+    sc = rng.uniform(-0.1, 0.1, (40, 2)).astype(np.float16)
+    raw[:, 0:2] = sc[:, 0:1].view(np.uint8)
+    if ty != 6:
+        raw[:, 2:4] = sc[:, 1:2].view(np.uint8)      # m / dmin; for Q5_0 these bytes belong to the bit field
+    raw = raw.reshape(-1)
+    want = (_np_q4_1_q5 if ty in (3, 6, 7) else _np_q45_k)(ty, raw, 40 * be)
+    got = orc.dequantize(ty, raw, 40 * be)
+    assert np.array_equal(got, want)
 
 
 def test_f32_oracle_on_reference_seeded_data(orc):
