@@ -70,11 +70,33 @@ template <int SUB>
 struct GemmFrag {
     v4i a;           // this wave's 32 tokens x 32 k
     v4i b[4];        // 4 x (32 weight rows x 32 k)
-    float4 dx[4];    // activation scales of the 16 tokens this lane accumulates
+    float4 dx[4];    // SUB = 1: activation scales of the 16 tokens this lane accumulates
+    float dxv;       // SUB = 2: one scale per lane: lane n of each 16-lane row holds the scale of the token of accumulator n
     float dw[4][SUB];  // weight scale of this lane's row in each of the 4 row tiles (per sub-block)
 };
 
 constexpr int FMT_Q8 = 0, FMT_Q4 = 1, FMT_Q6 = 2;
+
+// acc[I] += dx(token of accumulator I) * t[I].  The 16 activation scales a lane needs differ between
+// the two lane halves (MFMA 32x32 output: accumulator i of lane half h is token (i/4)*8 + h*4 + i%4),
+// so the Q6_K variant keeps them ONE per lane -- lane n of every 16-lane row holds the scale of
+// accumulator n for that row's half -- and the multiply-add reads it through a row broadcast (DPP
+// row_newbcast:n): one LDS dword and one register per lane and block instead of 16.  Measured: the
+// Q6_K kernel gains 9 % (its 16 spilled registers are gone); the Q8_0 / Q4_0 kernels, which fit
+// their registers either way, lose 4 % to the broadcast form and keep the 16 scales in registers.
+#define SMX_FMAC_BC(I)                                                                      \
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I " row_mask:0xf bank_mask:0xf"        \
+        : "+v"(accv[I])                                                                     \
+        : "v"(dxv), "v"(t[I]))
+__device__ __forceinline__ void scale_accumulate(float (&accv)[16], const v16i& dn, float dw, float ndw, float dxv) {
+    float t[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) t[i] = fmaf(dw, __int_as_float(dn[i]), ndw);
+    SMX_FMAC_BC(0); SMX_FMAC_BC(1); SMX_FMAC_BC(2); SMX_FMAC_BC(3); SMX_FMAC_BC(4); SMX_FMAC_BC(5); SMX_FMAC_BC(6);
+    SMX_FMAC_BC(7); SMX_FMAC_BC(8); SMX_FMAC_BC(9); SMX_FMAC_BC(10); SMX_FMAC_BC(11); SMX_FMAC_BC(12);
+    SMX_FMAC_BC(13); SMX_FMAC_BC(14); SMX_FMAC_BC(15);
+}
+#undef SMX_FMAC_BC
 
 template <int FMT, bool DUMP, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmArgs p) {
@@ -255,6 +277,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     for (int bi = 0; bi < KB; bi++) frag_lane[bi] = (col >> 3) * GRP + (col & 7) * 128 + ((2 * bi + half + col) & 7) * 16;
     // Q6_K: a lane takes bytes 8 * half .. + 7 of BOTH 16-byte chunks of the block (the order of k
     // inside an MFMA does not matter as long as both operands use the same one)
+    const int dx_tok = ((lane & 15) >> 2) * 8 + half * 4 + (lane & 3);  // token of accumulator lane % 16 in this lane's half
     const int frag6 = (col >> 3) * GRP + (col & 7) * 128 + half * 8;
 
     auto read_frag = [&](GemmFrag<SUB>& f, int buf, int bi) {
@@ -262,8 +285,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const char* sB = sA + A_BYTES;
         const float* sdw = (const float*)(sB + B_BYTES);
         const float* sdx = sdw + SUB * KB * 128;
+        if (Q6) {
+            f.dxv = sdx[bi * BM + wave * 32 + dx_tok];
+        } else {
 #pragma unroll
-        for (int g = 0; g < 4; g++) f.dx[g] = *(const float4*)(sdx + bi * BM + wave * 32 + g * 8 + half * 4);
+            for (int g = 0; g < 4; g++) f.dx[g] = *(const float4*)(sdx + bi * BM + wave * 32 + g * 8 + half * 4);
+        }
         if (Q6) {
             const int o0 = frag6 + ((2 * bi + col) & 7) * 16, o1 = frag6 + ((2 * bi + 1 + col) & 7) * 16;
             const int2 a0 = *(const int2*)(sA + wave * 4 * GRP + o0), a1 = *(const int2*)(sA + wave * 4 * GRP + o1);
@@ -314,8 +341,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
             const v16i dn = d[u & 1];
             const float dw = f.dw[nt][jj];
             const float ndw = -dw * MAGIC_F;  // exact: dw has at most 18 significant bits (f16, or f16 x int8)
+            if (Q6) {
+                scale_accumulate(acc[nt], dn, dw, ndw, f.dxv);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 16; i++) acc[nt][i] = fmaf(dxr[i], fmaf(dw, __int_as_float(dn[i]), ndw), acc[nt][i]);
+                for (int i = 0; i < 16; i++) acc[nt][i] = fmaf(dxr[i], fmaf(dw, __int_as_float(dn[i]), ndw), acc[nt][i]);
+            }
             asm volatile("" : "+v"(acc[nt][0]), "+v"(acc[nt][1]), "+v"(acc[nt][2]), "+v"(acc[nt][3]), "+v"(acc[nt][4]),
                               "+v"(acc[nt][5]), "+v"(acc[nt][6]), "+v"(acc[nt][7]), "+v"(acc[nt][8]), "+v"(acc[nt][9]),
                               "+v"(acc[nt][10]), "+v"(acc[nt][11]), "+v"(acc[nt][12]), "+v"(acc[nt][13]),
@@ -341,9 +372,15 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     // a wave whose 32 tokens all lie past the tile's end (ragged expert groups, M tails) only helps
     // with the staging: its SIMD time goes to the other workgroup on the CU
     const bool wave_live = tok0 + wave * 32 < M_end;
+    // The waves of a workgroup leave the barrier together, and 8 KB of loads per wave queue up in the
+    // CU's one address unit (20 cycles per 1 KB load alone, 64 behind three other waves): even waves
+    // issue the next stage's loads before block 0, odd waves after it (measured +4 %; spreading them
+    // over all four blocks leaves the last ones too little time to land: +1 %).
+    const int my_slot = wave & 1;
     for (int s = s_begin; s < s_end; s++) {
         const int buf = (s - s_begin) & 1;
-        if (s + 1 < s_end) issue_stage(buf ^ 1, s + 1);
+        const bool more = s + 1 < s_end;
+        if (more && (my_slot == 0 || !wave_live)) issue_stage(buf ^ 1, s + 1);
         if (wave_live) {
         GemmFrag<SUB> f0, f1;
         read_frag(f0, buf, 0);
@@ -351,6 +388,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         __builtin_amdgcn_sched_barrier(0);
         compute(f0, s * KB + 0);
         __builtin_amdgcn_sched_barrier(0);
+        if (more && my_slot == 1) issue_stage(buf ^ 1, s + 1);
         read_frag(f0, buf, 2);
         __builtin_amdgcn_sched_barrier(0);
         compute(f1, s * KB + 1);
@@ -362,7 +400,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         compute(f1, s * KB + 3);
         __builtin_amdgcn_sched_barrier(0);
         }
-        if (s + 1 < s_end) finish_stage(buf ^ 1, s + 1);
+        if (more) finish_stage(buf ^ 1, s + 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
