@@ -105,7 +105,6 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     constexpr int SUB = Q6 ? 2 : 1;  // scaled sub-blocks per 32-block
     constexpr int BM = 32 * NW, A_BYTES = a_bytes(NW), STAGE_BYTES = stage_bytes(NW, Q6);
     constexpr int BG = 16 / NW;  // 8-row groups of B each wave stages
-    constexpr int WS = 8 / NW;   // weight scales per thread per stage
     extern __shared__ __align__(16) char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int K = p.nb * 32;
@@ -160,21 +159,25 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         for (int ps = 0; ps < QG; ps++)
             b_off[ps] = (unsigned)min(row0 + (ps * NW + wave) * 16 + q_rowlo, N_end - 1) * (unsigned)p.nb;
     }
-    // scales: thread (sr, sh) carries blocks 2*sh, 2*sh+1 of the stage for token sr, and thread
-    // (wr, wh) blocks wh*WS .. wh*WS+WS-1 for weight row wr
-    const int sr = tid & (BM - 1), sh = tid / BM;
+    // scales of a stage (4 blocks): threads 0..127 carry the four f16 scales of weight row tid (8
+    // contiguous bytes), threads 128..128+BM-1 the four fp32 scales of token tid - 128 (16 contiguous
+    // bytes): one load per thread when rows are 4-block aligned (nb % 4 == 0), four clamped loads otherwise.
+    // Q6_K weight scales: thread (wr, wh) carries d and the sub-block scales 4*wh .. 4*wh+3 of row wr.
+    const bool role_w = tid < 128, role_x = !role_w && tid - 128 < BM;   // wave-uniform
+    const int role_r = role_w ? tid : tid - 128;
+    const bool vec_sc = (p.nb & 3) == 0;
     const int wr = tid & 127, wh = tid >> 7;
-    const bool w_valid = row0 + wr < N_end, x_valid = tok0 + sr < M_end;
+    const bool w_valid = row0 + wr < N_end, x_valid = tok0 + role_r < M_end;
     const size_t scw_base = (size_t)min(row0 + wr, N_end - 1) * (Q6 ? p.nb >> 3 : p.nb);
     size_t scx_base;
     {
-        const int ti = min(tok0 + sr, M_end - 1);
+        const int ti = min(tok0 + role_r, M_end - 1);
         scx_base = (size_t)(p.a_rowmap ? p.a_rowmap[ti] : ti) * p.nb;
     }
     uint4 rb[Q6 ? 3 : QG];  // Q4_0 / Q6_K quants on their way through registers
-    uint16_t rsw[WS];   // raw weight scales (f16), row wr (Q6_K: rsw[0] = d of the superblock)
+    uint4 rsv = {0, 0, 0, 0};  // the thread's four raw scales: f16 pairs in .x .y (weights) or four fp32 (activations)
+    uint16_t rsd = 0;   // Q6_K: d of the superblock, row wr
     unsigned rsc = 0;   // Q6_K: the four sub-block scales 4 * wh .. 4 * wh + 3 of the stage, row wr
-    float rsx0, rsx1;   // activation scales of blocks 2*sh, 2*sh+1, token sr
 
     // issue every global read of stage s; the register-staged parts are written by finish_stage
     // all global reads of stage s (issuing them piecemeal between the blocks measures slower)
@@ -202,14 +205,29 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         }
         // branch-free and unconverted, so that nothing here waits for a load before the MFMA work
         if (Q6) {
-            rsw[0] = op.wscales[scw_base + (s >> 1)];
+            rsd = op.wscales[scw_base + (s >> 1)];
             rsc = *(const unsigned*)(op.wsc + (scw_base + (s >> 1)) * 16 + (s & 1) * 8 + wh * 4);
-        } else {
-#pragma unroll
-            for (int j = 0; j < WS; j++) rsw[j] = op.wscales[scw_base + min(blk0 + wh * WS + j, p.nb - 1)];
+        } else if (role_w) {
+            const uint16_t* ws = op.wscales + scw_base;
+            if (vec_sc) {
+                const uint2 v = *(const uint2*)(ws + blk0);
+                rsv.x = v.x; rsv.y = v.y;
+            } else {
+                const int last = p.nb - 1;
+                rsv.x = (unsigned)ws[min(blk0, last)] | ((unsigned)ws[min(blk0 + 1, last)] << 16);
+                rsv.y = (unsigned)ws[min(blk0 + 2, last)] | ((unsigned)ws[min(blk0 + 3, last)] << 16);
+            }
         }
-        rsx0 = p.xd[scx_base + min(blk0 + 2 * sh, p.nb - 1)];
-        rsx1 = p.xd[scx_base + min(blk0 + 2 * sh + 1, p.nb - 1)];
+        if (role_x) {
+            const unsigned* xs = (const unsigned*)p.xd + scx_base;
+            if (vec_sc) {
+                rsv = *(const uint4*)(xs + blk0);
+            } else {
+                const int last = p.nb - 1;
+                rsv.x = xs[min(blk0, last)]; rsv.y = xs[min(blk0 + 1, last)];
+                rsv.z = xs[min(blk0 + 2, last)]; rsv.w = xs[min(blk0 + 3, last)];
+            }
+        }
     };
 
     auto finish_stage = [&](int buf, int s) {
@@ -231,7 +249,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
                 o.w = q6_bytes(q.w >> ls, h.w >> hs);
                 *(uint4*)(sB + off + ((2 * j + q6_p + r) & 7) * 16) = o;  // elements 32j + 16p .. + 15 of the stage
             }
-            const float d = w_valid ? h2f_(rsw[0]) : 0.f;
+            const float d = w_valid ? h2f_(rsd) : 0.f;
 #pragma unroll
             for (int j = 0; j < 4; j++)  // d * sc is exact in fp32 (11 x 8 significant bits)
                 sdw[(wh * 4 + j) * 128 + wr] = d * (float)(int)(signed char)(rsc >> (8 * j));
@@ -251,13 +269,16 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
                 *(uint4*)(sB + off + ((2 * q_bi + 1 + r) & 7) * 16) = hi;  // elements 16..31
             }
         }
-        if (!Q6) {
+        if (!Q6 && role_w) {
+            const unsigned h[4] = {rsv.x & 0xffffu, rsv.x >> 16, rsv.y & 0xffffu, rsv.y >> 16};
 #pragma unroll
-            for (int j = 0; j < WS; j++)
-                sdw[(wh * WS + j) * 128 + wr] = (w_valid && blk0 + wh * WS + j < p.nb) ? h2f_(rsw[j]) : 0.f;
+            for (int j = 0; j < KB; j++) sdw[j * 128 + wr] = (w_valid && blk0 + j < p.nb) ? h2f_((uint16_t)h[j]) : 0.f;
         }
-        sdx[(2 * sh) * BM + sr] = (x_valid && blk0 + 2 * sh < p.nb) ? rsx0 : 0.f;
-        sdx[(2 * sh + 1) * BM + sr] = (x_valid && blk0 + 2 * sh + 1 < p.nb) ? rsx1 : 0.f;
+        if (role_x) {
+            const unsigned v[4] = {rsv.x, rsv.y, rsv.z, rsv.w};
+#pragma unroll
+            for (int j = 0; j < KB; j++) sdx[j * BM + role_r] = (x_valid && blk0 + j < p.nb) ? __uint_as_float(v[j]) : 0.f;
+        }
     };
 
     float acc[4][16];
