@@ -44,7 +44,8 @@ def test_lm_head_q6k_sampled(accel, orc, synth, relerr):
     accel.evict("t.head")
 
 
-@pytest.mark.parametrize("ty,M,N,K", [(8, 2048, 15360, 3840), (2, 2048, 15360, 3840), (8, 2048, 3840, 15360), (2, 2048, 3840, 15360)])
+@pytest.mark.parametrize("ty,M,N,K", [(8, 2048, 15360, 3840), (2, 2048, 15360, 3840), (8, 2048, 3840, 15360), (2, 2048, 3840, 15360),
+                                      (14, 2048, 15360, 3840), (14, 1000, 3840, 15360)])
 def test_prefill_gemm_full_size_sampled(accel, orc, synth, relerr, ty, M, N, K):
     raw = synth.make_weight(ty, N, K, seed=10 + ty)
     xs = synth.make_acts(M, K, seed=20 + ty)
@@ -65,10 +66,11 @@ def test_prefill_gemm_full_size_sampled(accel, orc, synth, relerr, ty, M, N, K):
     accel.evict("t.fg")
 
 
-def test_moe_full_size_decode_and_prefill(accel, orc, synth, relerr):
+@pytest.mark.parametrize("ty", [8, 14])
+def test_moe_full_size_decode_and_prefill(accel, orc, synth, relerr, ty):
     ne, hidden, eff, k, m = 64, 2048, 768, 8, 512
-    gate, up, down = synth.make_moe_q8(ne, hidden, eff, seed=30)
-    assert accel.upload_moe_q8(21, gate, up, down, hidden, eff, ne)
+    gate, up, down = (synth.make_moe_q8 if ty == 8 else synth.make_moe_q6)(ne, hidden, eff, seed=30)
+    assert (accel.upload_moe_q8 if ty == 8 else accel.upload_moe_q6)(21, gate, up, down, hidden, eff, ne)
     ids, w = synth.zipf_routing(m, ne, k, seed=31)
     xs = synth.make_acts(m, hidden, seed=32)
     plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
@@ -78,6 +80,6 @@ def test_moe_full_size_decode_and_prefill(accel, orc, synth, relerr):
     for t in (0, 255, 511):
         order = np.argsort(ids[t], kind="stable")
         yd, gu, aq, ad = accel.moe_ffn_stages(21, ids[t][order], w[t][order], xs[t], eff)
-        ref, _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[t][order], w[t][order], xs[t], aq_in=aq, ad_in=ad)
+        ref, _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[t][order], w[t][order], xs[t], aq_in=aq, ad_in=ad, ty=ty)
         assert relerr(yd, ref) <= TOL
         assert relerr(y[t], yd) <= 2e-2      # prefill and decode chains differ only at quantiser rounding boundaries
