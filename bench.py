@@ -192,7 +192,7 @@ class Bench:
                 "frac_hbm_peak": gbs / HBM_PEAK_GBS, "kernel": KERNEL[ty], "kernel_avg_us": ms / steps * 1e3,
                 "kernel_GBps": gbs, "kernel_frac_hbm_peak": gbs / HBM_PEAK_GBS}
 
-    # ------------------------------------------------------------------ dense FFN decode step (2 launches)
+    # ------------------------------------------------------------------ dense FFN decode step (2 calls, 3 launches)
     def ffn_block(self, name, ty, H, F, min_total_bytes, steps=None, warmup=None):
         """One token through a dense FFN: launch 1 = rmsnorm + quantiser + gate and up GEMVs, launch 2 =
         SwiGLU + quantiser + down GEMV; rotating through >= 1 GB of (gate, up, down) sets."""
@@ -225,7 +225,7 @@ class Bench:
             acc.dev_free(p)
         algo = 2 * a1 + a2
         gbs = algo * steps / (ms * 1e-3) / 1e9
-        return {"workload": name, "shape": {"hidden": H, "ffn": F, "M": 1, "launches_per_step": 2}, "weight_sets": nsets,
+        return {"workload": name, "shape": {"hidden": H, "ffn": F, "M": 1, "calls_per_step": 2, "launches_per_step": 3}, "weight_sets": nsets,
                 "algorithmic_bytes": algo, "steps": steps, "ms_per_step": ms / steps, "GBps": gbs,
                 "frac_hbm_peak": gbs / HBM_PEAK_GBS}
 

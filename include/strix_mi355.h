@@ -164,7 +164,10 @@ int smx_moe_layer_dev(smx_ctx* ctx, size_t layer, const float* xs_dev, size_t m,
 /* ---- HIP graph capture of a sequence of `_dev` calls: the role of the reference's captured decode
  *      token (decode.rs:3053-3203), so a launch-bound chain of small GEMVs replays without per-launch
  *      host cost.  Between begin and end only `_dev` entry points may be called, with shapes already
- *      seen once outside capture (no scratch growth while capturing); per-kernel timing is off. ---- */
+ *      seen once outside capture (no scratch growth while capturing); per-kernel timing is off.
+ *      A graph stays valid when later calls grow the context's scratch (the buffers it captured are
+ *      kept until the context closes); it does NOT survive smx_evict of a weight it uses, nor the
+ *      caller freeing the activation buffers it was captured with. ---- */
 typedef struct smx_graph smx_graph;
 int smx_graph_begin(smx_ctx* ctx);
 int smx_graph_end(smx_ctx* ctx, smx_graph** out);

@@ -7,9 +7,77 @@
 // 16-wide sub-blocks of Q6_K.
 #include <algorithm>
 
+#include "detmath.h"
 #include "smx_internal.h"
 
 namespace smx {
+
+// Up to SMX_GEMV_GROUP_MAX rows, each the product of an activation function of one operand and a
+// second operand (SwiGLU: silu(a) * b, GeGLU: gelu_tanh(a) * b; kernels.rs:151-226), quantised like
+// actquant_kernel below.  Row j goes to xq + j*K, xd / xs + j*K/32.  The arithmetic is the one the
+// GEMV staging performs when it runs the producer itself, operation for operation.
+struct ProdRows {
+    const float4* a[SMX_GEMV_GROUP_MAX];
+    const float4* b[SMX_GEMV_GROUP_MAX];
+};
+__global__ __launch_bounds__(256) void actprod_quant_kernel(const ProdRows R, int kind, int* __restrict__ xq4,
+                                                            float* __restrict__ xd, int* __restrict__ xs, int nb32) {
+#pragma clang fp contract(off)
+    const int j = blockIdx.y;
+    const int gid = blockIdx.x * 256 + threadIdx.x;
+    const int blk = gid >> 3;
+    const bool live = blk < nb32;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f), g = v;
+    if (live) {
+        v = R.a[j][gid];
+        g = R.b[j][gid];
+    }
+    float4 w;
+    if (kind == SMX_ACT_SILU_MUL) {
+        w.x = det_silu(v.x) * g.x; w.y = det_silu(v.y) * g.y; w.z = det_silu(v.z) * g.z; w.w = det_silu(v.w) * g.w;
+    } else {
+        w.x = det_gelu_tanh(v.x) * g.x; w.y = det_gelu_tanh(v.y) * g.y;
+        w.z = det_gelu_tanh(v.z) * g.z; w.w = det_gelu_tanh(v.w) * g.w;
+    }
+    float a = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
+    a = fmaxf(a, __shfl_xor(a, 1));
+    a = fmaxf(a, __shfl_xor(a, 2));
+    a = fmaxf(a, __shfl_xor(a, 4));
+    const float d = a / 127.f;
+    const float inv = d > 0.f ? 1.f / d : 0.f;
+    const int q0 = max(-127, min(127, (int)rintf(w.x * inv)));
+    const int q1 = max(-127, min(127, (int)rintf(w.y * inv)));
+    const int q2 = max(-127, min(127, (int)rintf(w.z * inv)));
+    const int q3 = max(-127, min(127, (int)rintf(w.w * inv)));
+    int s = q0 + q1 + q2 + q3;
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    const int other = __shfl_xor(s, 4);
+    if (live) {
+        xq4[(size_t)j * nb32 * 8 + gid] = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+        if ((gid & 7) == 0) {
+            xd[(size_t)j * nb32 + blk] = d;
+            xs[(size_t)j * nb32 + blk] = (s & 0xffff) | (other << 16);
+        }
+    }
+}
+
+int launch_actprod_quant(smx_ctx* c, int kind, const float* const* as, const float* const* bs, int n, size_t K,
+                         int8_t* xq, float* xd, int32_t* xs) {
+    if (K % 32 != 0 || n < 1 || n > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "producer quantiser: %d rows of %zu", n, K);
+    if (kind != SMX_ACT_SILU_MUL && kind != SMX_ACT_GEGLU) return fail(c, SMX_ERR_ARG, "producer quantiser: kind %d", kind);
+    ProdRows R = {};
+    for (int j = 0; j < n; j++) {
+        R.a[j] = (const float4*)as[j];
+        R.b[j] = (const float4*)bs[j];
+    }
+    const int nb32 = (int)(K / 32);
+    ProfScope ps(c, "actprod_quant");
+    hipLaunchKernelGGL(actprod_quant_kernel, dim3((unsigned)((nb32 * 8 + 255) / 256), (unsigned)n), dim3(256), 0, c->stream, R,
+                       kind, (int*)xq, xd, (int*)xs, nb32);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
 
 // 8 lanes per 32-block, one float4 each: 128-bit loads, 32-bit packed stores.
 __global__ __launch_bounds__(256) void actquant_kernel(const float4* __restrict__ x, int* __restrict__ xq4,

@@ -29,7 +29,8 @@ int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
         return fail(c, SMX_ERR_ARG, "scratch would grow to %zu bytes during graph capture: run the call once outside capture first", bytes);
     if (b.p) {
         SMX_HIP(c, hipStreamSynchronize(c->stream));
-        SMX_HIP(c, hipFree(b.p));
+        if (c->live_graphs > 0) c->retired.push_back(b.p);  // a graph may still name this buffer
+        else SMX_HIP(c, hipFree(b.p));
         b.p = nullptr;
         b.cap = 0;
     }
@@ -237,6 +238,7 @@ void smx_destroy(smx_ctx* c) {
     }
     for (DevBuf* b : {&c->xf32, &c->xq, &c->xd, &c->xs, &c->yf32, &c->work, &c->work2, &c->tab})
         if (b->p) (void)hipFree(b->p);
+    for (char* p : c->retired) (void)hipFree(p);
     for (DevBuf* b : {&c->hx, &c->hy})
         if (b->p) (void)hipHostFree(b->p);
     for (auto& r : c->prof) {
@@ -403,6 +405,7 @@ int smx_graph_end(smx_ctx* c, smx_graph** out) {
         delete g;
         return hip_fail(c, e, "hipStreamEndCapture/hipGraphInstantiate");
     }
+    c->live_graphs++;
     *out = g;
     return SMX_OK;
 }
@@ -418,6 +421,7 @@ void smx_graph_destroy(smx_ctx* c, smx_graph* g) {
     if (c) (void)hipStreamSynchronize(c->stream);
     if (g->exec) (void)hipGraphExecDestroy(g->exec);
     if (g->graph) (void)hipGraphDestroy(g->graph);
+    if (c && c->live_graphs > 0) c->live_graphs--;
     delete g;
 }
 

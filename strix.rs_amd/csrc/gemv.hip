@@ -40,9 +40,13 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, in
 
 namespace {
 
+// Row length from which silu / gelu producers run in their own launch (measured on 2560 <- 9728).
+constexpr size_t kProducerSplitK = 4096;
+
 // Launch geometry: slots per wave, pipeline depth, K-split, lanes per row, threads per workgroup.
 struct Geom {
     bool prod = false;  // an activation producer runs in the staging
+    bool preq = false;  // the (single) activation row arrives quantised
     int rpw, pre, ks, lpr, nt;
     unsigned grid;
     size_t lds;
@@ -65,6 +69,7 @@ int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk
     // one activation row: quantiser fused into the staging (FQ 1), behind an activation producer if the
     // caller asked for one (FQ 2: its own variant, so that the plain GEMV carries none of its code);
     // several rows: staged from rows quantised once (FQ 0)
+    if (MT == 1 && !DUMP && g.preq) return launch_fq<Ops, MT, RPW, PRE, KS, LPR, 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
     if (MT == 1 && !DUMP && g.prod) return launch_fq<Ops, MT, RPW, PRE, KS, LPR, (MT == 1 && !DUMP) ? 2 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
     return launch_fq<Ops, MT, RPW, PRE, KS, LPR, MT == 1 ? 1 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
 }
@@ -251,6 +256,25 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
     const Weight& w0 = *ws[0];
     Geom g = pick_geom(c, w0.type, maxN, w0.nblk, 1, false, n);
     g.prod = prod && prod->kind != SMX_ACT_NONE;
+    // Every workgroup runs the producer over the whole row.  For the exp-based ones on a long row
+    // (an FFN's down projection) that repeated work outweighs a launch: they run once, in a
+    // quantiser kernel of their own, and the GEMV stages the quantised row.
+    if (g.prod && (prod->kind == SMX_ACT_SILU_MUL || prod->kind == SMX_ACT_GEGLU) && w0.K >= kProducerSplitK) {
+        const float* bs[SMX_GEMV_GROUP_MAX];
+        for (int i = 0; i < n; i++) bs[i] = J.job[i].X.x2;
+        const size_t nb = w0.K / 32;
+        int rc;
+        if ((rc = ensure(c, c->xq, (size_t)n * w0.K)) != SMX_OK) return rc;
+        if ((rc = ensure(c, c->xd, (size_t)n * nb * 4)) != SMX_OK) return rc;
+        if ((rc = ensure(c, c->xs, (size_t)n * nb * 4)) != SMX_OK) return rc;
+        rc = launch_actprod_quant(c, prod->kind, xs, bs, n, w0.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+        if (rc != SMX_OK) return rc;
+        for (int i = 0; i < n; i++)
+            J.job[i].X = {nullptr, (const int8_t*)c->xq.p + (size_t)i * w0.K, (const float*)c->xd.p + (size_t)i * nb,
+                          (const int*)c->xs.p + (size_t)i * nb};
+        g.prod = false;
+        g.preq = true;
+    }
     if (g.lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "gemv: activation of %zu needs %zu bytes of LDS", w0.K, g.lds);
     return launch_jobs(c, w0.type, g, J, n, (int)w0.nblk, 1, 1, nullptr, 0, name);
 }

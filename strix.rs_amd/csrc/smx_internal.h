@@ -77,6 +77,11 @@ struct smx_ctx {
     int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
 
     bool capturing = false;  // between smx_graph_begin and smx_graph_end
+    // A captured graph holds the addresses of the scratch buffers its kernels used.  While any graph
+    // of this context is alive, a scratch buffer that has to grow is retired (kept until the context
+    // closes) instead of freed, so that replays keep reading and writing valid memory.
+    int live_graphs = 0;
+    std::vector<char*> retired;
 
     // profiling
     bool prof_on = false;
@@ -151,6 +156,9 @@ struct GemmArgs {
 // ---- launchers (all enqueue on c->stream; return SMX_OK or an error) ----
 // Activation quantiser: x[m][K] f32 -> xq[m][K], xd[m][K/32], xs[m][K/32] (two i16 sums per block).
 int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, float* xd, int32_t* xs);
+// n rows act(as[j]) * bs[j] (SMX_ACT_SILU_MUL or SMX_ACT_GEGLU), quantised: row j at xq + j*K, xd/xs + j*K/32.
+int launch_actprod_quant(smx_ctx* c, int kind, const float* const* as, const float* const* bs, int n, size_t K,
+                         int8_t* xq, float* xd, int32_t* xs);
 // GEMV with the activation quantiser fused into its LDS staging: x fp32 [m][K] -> y[m][N],
 // m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);

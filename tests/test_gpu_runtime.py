@@ -65,6 +65,37 @@ def test_graph_replays_equal_eager(accel, synth):
         accel.dev_free(p)
 
 
+def test_graph_survives_later_scratch_growth(pkg, synth):
+    """A graph captured with small scratch buffers must keep working after a larger eager call made
+    the context reallocate them (the captured buffers are retired, not freed)."""
+    acc = pkg.Mi355WeightAccel(0)                    # a fresh context: its scratch starts at the minimum size
+    N, K, m = 256, 4096, 48
+    raw = synth.make_weight(8, N, K, seed=41)
+    assert acc.upload_q8_0("t.sg", raw, K, N)
+    xs = synth.make_acts(m, K, seed=42)
+    xd, yd = acc.dev_alloc(xs.nbytes), acc.dev_alloc(m * N * 4)
+    acc.h2d(xd, xs)
+    acc.gemm_dev("t.sg", xd, m, yd)                  # quantiser scratch + split-K partials
+    want = acc.d2h(np.empty((m, N), np.float32), yd)
+    acc.graph_begin()
+    acc.gemm_dev("t.sg", xd, m, yd)
+    g = acc.graph_end()
+    big = synth.make_acts(3000, K, seed=43)          # 12 MB of int8 rows, 3 MB of partials: every scratch buffer grows
+    bd, by = acc.dev_alloc(big.nbytes), acc.dev_alloc(3000 * N * 4)
+    acc.h2d(bd, big)
+    acc.gemm_dev("t.sg", bd, 3000, by)
+    acc.sync()
+    for rep in range(3):
+        acc.h2d(yd, np.zeros((m, N), np.float32))
+        acc.graph_launch(g)
+        acc.sync()
+        assert np.array_equal(acc.d2h(np.empty((m, N), np.float32), yd), want), f"replay {rep}"
+    acc.graph_destroy(g)
+    for p in (xd, yd, bd, by):
+        acc.dev_free(p)
+    acc.close()
+
+
 def test_capture_refuses_scratch_growth(accel, synth, pkg):
     raw = synth.make_weight(8, 128, 4096, seed=8)
     assert accel.upload_q8_0("t.grow", raw, 4096, 128)
