@@ -108,7 +108,9 @@ int smx_lm_head_argmax_rows(smx_ctx* ctx, const char* key, const float* xs, size
 /* ---- MoE ---- */
 /* WeightAccel::moe_ffn, accel.rs:201-210; decode.rs:2833-2870, 1923-2128.
  * y[hidden] = sum_k wexp[k] * down_k( silu(gate_k x) * (up_k x) ), k routed
- * experts accumulated in routed order.  sgate must be 0 (no shared expert). */
+ * experts accumulated in routed order.  sgate != 0 adds sgate * shared_expert(x), the dense FFN
+ * blk.<layer>.ffn_{gate,up,down}_shexp.weight (decode.rs:1820-1855 queue_shexp); as in the
+ * reference the call declines (0) when those three weights are not resident. */
 int smx_moe_ffn(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                 const float* x, size_t x_len, float sgate, float* y, size_t y_cap);
 /* WeightAccel::moe_layer_q8_dev, accel.rs:311-321; decode.rs:1608-1739.
@@ -153,6 +155,9 @@ int smx_gemv_fused_dev(smx_ctx* ctx, size_t n, const char* const* keys, int act,
 int smx_gemv_fused(smx_ctx* ctx, const char* key, int act, const float* a, const float* b, size_t in_len,
                    float eps, float* y, size_t out_cap);
 
+/* y_dev += sgate * shared_expert(x_dev) for layer `layer` (the second half of moe_ffn with a shared
+ * expert, decode.rs:1820-1855), to follow smx_moe_ffn_dev on device-resident activations. */
+int smx_moe_shexp_dev(smx_ctx* ctx, size_t layer, float sgate, const float* x_dev, float* y_dev);
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                     const float* x_dev, float* y_dev);
 /* smx_moe_layer with the activations and the result on the device (y_dev: m x hidden floats); the

@@ -27,7 +27,7 @@ EXPORTS = [
     "smx_resident_bytes", "smx_upload_q4_0", "smx_upload_q8_0", "smx_upload_q6_k",
     "smx_upload_moe_q8", "smx_evict", "smx_gemv", "smx_gemv_rows", "smx_gemv_batch", "smx_gemm",
     "smx_lm_head_argmax_rows", "smx_moe_ffn", "smx_moe_layer", "smx_dev_alloc", "smx_dev_free",
-    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev",
+    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev", "smx_moe_shexp_dev",
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
@@ -95,6 +95,7 @@ def load_library():
     L.smx_gemv_fused_dev.argtypes = [vp, sz, vp, i, vp, vp, C.c_float, vp]
     L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
+    L.smx_moe_shexp_dev.argtypes = [vp, sz, C.c_float, vp, vp]
     L.smx_prof_enable.argtypes = [vp, i]
     L.smx_prof_reset.argtypes = [vp]
     L.smx_prof_read.argtypes = [vp, cp, C.POINTER(C.c_double), C.POINTER(sz)]
@@ -467,6 +468,10 @@ class Mi355WeightAccel:
     def moe_ffn_dev(self, layer, ids, wexp, x_dev, y_dev):
         ids, wexp = _c(ids, np.int32), _c(wexp, np.float32)
         return self._check(self._L.smx_moe_ffn_dev(self._h, layer, _p(ids), _p(wexp), ids.size, x_dev, y_dev))
+
+    def moe_shexp_dev(self, layer, sgate, x_dev, y_dev):
+        """y_dev += sgate * shared_expert(x_dev) (decode.rs:1820-1855)."""
+        return self._check(self._L.smx_moe_shexp_dev(self._h, layer, float(sgate), x_dev, y_dev))
 
     def graph_begin(self):
         self._check(self._L.smx_graph_begin(self._h))

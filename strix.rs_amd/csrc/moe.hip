@@ -333,6 +333,56 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     return SMX_OK;
 }
 
+// out[i] += sd[i] * sgate (kernels.rs:1747-1751 shexp_add)
+__global__ __launch_bounds__(256) void shexp_add_kernel(float* __restrict__ out, const float* __restrict__ sd, float sgate, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] += sd[i] * sgate;
+}
+
+// The layer's shared expert, added onto y (decode.rs:1820-1855 queue_shexp): the dense FFN
+// blk.<layer>.ffn_{gate,up,down}_shexp.weight over the same activation, scaled by the caller's gate.
+// Gate and up share one grouped GEMV launch; silu(g)*u is quantised inside the down GEMV's staging
+// (or in a launch of its own on long rows).  Declines when the three weights are not resident.
+static int shexp_enqueue(smx_ctx* c, size_t layer, size_t hidden, float sgate, const float* x_dev, float* y_dev) {
+    const std::string base = "blk." + std::to_string(layer) + ".ffn_";
+    const Weight* w[3];
+    const char* part[3] = {"gate", "up", "down"};
+    for (int i = 0; i < 3; i++) {
+        auto it = c->weights.find(base + part[i] + "_shexp.weight");
+        if (it == c->weights.end()) return SMX_NOT_RESIDENT;
+        w[i] = &it->second;
+    }
+    const size_t sff = w[0]->N;
+    if (w[0]->K != hidden || w[1]->K != hidden || w[1]->N != sff || w[1]->type != w[0]->type || w[2]->K != sff ||
+        w[2]->N != hidden)
+        return fail(c, SMX_ERR_ARG, "moe_ffn: shared expert of layer %zu has shapes %zux%zu, %zux%zu, %zux%zu for hidden %zu",
+                    layer, w[0]->N, w[0]->K, w[1]->N, w[1]->K, w[2]->N, w[2]->K, hidden);
+    Carver cv;
+    const size_t o_g = cv.take(sff * 4), o_u = cv.take(sff * 4), o_d = cv.take(hidden * 4);
+    int rc = ensure(c, c->work2, cv.off);
+    if (rc != SMX_OK) return rc;
+    float* g = (float*)(c->work2.p + o_g);
+    float* u = (float*)(c->work2.p + o_u);
+    float* sd = (float*)(c->work2.p + o_d);
+    {
+        const Weight* ws[2] = {w[0], w[1]};
+        const float* xs[2] = {x_dev, x_dev};
+        float* ys[2] = {g, u};
+        if ((rc = launch_gemv_group(c, ws, xs, ys, 2, "shexp_gate_up")) != SMX_OK) return rc;
+    }
+    {
+        const ActProd prod = {SMX_ACT_SILU_MUL, u, 0.f};
+        const float* xs[1] = {g};
+        float* ys[1] = {sd};
+        if ((rc = launch_gemv_group(c, &w[2], xs, ys, 1, "shexp_down", &prod)) != SMX_OK) return rc;
+    }
+    ProfScope ps(c, "shexp_add");
+    hipLaunchKernelGGL(shexp_add_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, c->stream, y_dev, sd, sgate,
+                       (int)hidden);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
 static int moe_ffn_host(smx_ctx* c, size_t layer, const int32_t* ids, const float* wexp, size_t k, const float* x,
                         size_t x_len, float sgate, float* y, size_t y_cap, float* gu, int8_t* aq, float* ad) {
     if (!c) return SMX_ERR_ARG;
@@ -342,8 +392,6 @@ static int moe_ffn_host(smx_ctx* c, size_t layer, const int32_t* ids, const floa
     const MoeLayer& L = it->second;
     if (x_len != L.hidden) return fail(c, SMX_ERR_ARG, "moe_ffn: activation length %zu, hidden %zu", x_len, L.hidden);
     if (y_cap < L.hidden) return fail(c, SMX_ERR_ARG, "moe_ffn: output capacity %zu < %zu", y_cap, L.hidden);
-    if (sgate != 0.0f)
-        return fail(c, SMX_ERR_ARG, "moe_ffn: shared-expert gate %g: the shared expert is outside this path", (double)sgate);
     SMX_HIP(c, hipSetDevice(c->device));
     int rc;
     if ((rc = ensure(c, c->xf32, L.hidden * 4)) != SMX_OK) return rc;
@@ -352,6 +400,13 @@ static int moe_ffn_host(smx_ctx* c, size_t layer, const int32_t* ids, const floa
     MoeScratch s;
     rc = moe_ffn_enqueue(c, L, ids, wexp, k, (const float*)c->xf32.p, (float*)c->yf32.p, &s);
     if (rc != SMX_OK) return rc;
+    if (sgate != 0.0f) {  // decode.rs:2850, 2865: no shared expert resident -> the whole call declines
+        rc = shexp_enqueue(c, layer, L.hidden, sgate, (const float*)c->xf32.p, (float*)c->yf32.p);
+        if (rc != SMX_OK) {
+            (void)hipStreamSynchronize(c->stream);
+            return rc;
+        }
+    }
     SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, L.hidden * 4, hipMemcpyDeviceToHost, c->stream));
     if (gu) {
         for (size_t kk = 0; kk < k; kk++) {
@@ -406,6 +461,14 @@ int smx_moe_ffn_dev(smx_ctx* c, size_t layer, const int32_t* ids, const float* w
     auto it = c->moe.find(layer);
     if (it == c->moe.end()) return SMX_NOT_RESIDENT;
     return moe_ffn_enqueue(c, it->second, ids, wexp, k, x_dev, y_dev, nullptr);
+}
+
+int smx_moe_shexp_dev(smx_ctx* c, size_t layer, float sgate, const float* x_dev, float* y_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!x_dev || !y_dev) return fail(c, SMX_ERR_ARG, "moe_shexp_dev: null argument");
+    auto it = c->moe.find(layer);
+    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+    return shexp_enqueue(c, layer, it->second.hidden, sgate, x_dev, y_dev);
 }
 
 // xs / y on the host (copied in and out, one sync) or, with on_device, device pointers (enqueue only).

@@ -65,8 +65,39 @@ def test_moe_ffn_declines_and_errors(accel, synth, pkg):
         accel.moe_ffn(4, [7], [1.0], x)          # expert id out of range
     with pytest.raises(pkg.SmxError):
         accel.moe_ffn(4, [0], [1.0], x[:32])     # wrong hidden
-    with pytest.raises(pkg.SmxError):
-        accel.moe_ffn(4, [0], [1.0], x, sgate=0.5)
+    assert accel.moe_ffn(4, [0], [1.0], x, sgate=0.5) is None   # no shared expert resident: declines (decode.rs:2865)
+
+
+@pytest.mark.parametrize("ty,hidden,sff", [(8, 256, 512), (2, 256, 4608), (14, 512, 256)])
+def test_moe_ffn_shared_expert(accel, orc, synth, relerr, ty, hidden, sff):
+    """moe_ffn with a shared-expert gate (decode.rs:1820-1855 queue_shexp, kernels.rs:1747-1751):
+    y = routed + sgate * down_s(silu(gate_s x) * (up_s x)), checked stage by stage on the device's own g, u."""
+    ne, eff, k, layer, sgate = 4, 256, 2, 23, 0.37
+    gate, up, down = synth.make_moe_q8(ne, hidden, eff, seed=50)
+    assert accel.upload_moe_q8(layer, gate, up, down, hidden, eff, ne)
+    upl = {2: accel.upload_q4_0, 8: accel.upload_q8_0, 14: accel.upload_q6_k}[ty]
+    sg, su, sd = synth.make_weight(ty, sff, hidden, seed=51), synth.make_weight(ty, sff, hidden, seed=52), synth.make_weight(ty, hidden, sff, seed=53)
+    names = [f"blk.{layer}.ffn_{p}_shexp.weight" for p in ("gate", "up", "down")]
+    assert upl(names[0], sg, hidden, sff) and upl(names[1], su, hidden, sff)
+    ids, w = synth.zipf_routing(1, ne, k, seed=54)
+    x = synth.make_acts(1, hidden, seed=55)[0]
+    assert accel.moe_ffn(layer, ids[0], w[0], x, sgate=sgate) is None      # down weight still missing
+    assert upl(names[2], sd, sff, hidden)
+    routed = accel.moe_ffn(layer, ids[0], w[0], x)
+    y = accel.moe_ffn(layer, ids[0], w[0], x, sgate=sgate)
+    g, u = accel.gemv(names[0], x, sff), accel.gemv(names[1], x, sff)
+    assert relerr(g, orc.matmul_q8_from_f32(ty, sg, hidden, sff, x)[0]) <= TOL
+    shared = orc.matmul_q8_from_f32(ty, sd, sff, hidden, orc.act_produce(2, g, u))[0]
+    assert relerr(y, routed + np.float32(sgate) * shared) <= TOL
+    # device-resident form: routed part, then the shared expert on top
+    xd, yd = accel.dev_alloc(x.nbytes), accel.dev_alloc(x.nbytes)
+    accel.h2d(xd, x)
+    assert accel.moe_ffn_dev(layer, ids[0], w[0], xd, yd) and accel.moe_shexp_dev(layer, sgate, xd, yd)
+    assert np.array_equal(accel.d2h(np.empty(hidden, np.float32), yd), y)
+    accel.dev_free(xd)
+    accel.dev_free(yd)
+    for n in names:
+        accel.evict(n)
 
 
 def _moe_layer_oracle(orc, gate, up, down, hidden, eff, ne, xs, ids, w, ty=8):
