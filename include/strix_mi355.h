@@ -117,6 +117,15 @@ int smx_moe_ffn(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wex
  * xs[m][hidden]; plan[nplan][3] = (expert, slot_off, count); slot_tok[slots],
  * wslot[slots]; y[m][hidden] = sum over the token's slots (ascending slot
  * index) of wslot * expert_ffn(xs[token]). */
+/* WeightAccel::moe_layer_ffn, accel.rs:238-246; decode.rs:3552-3629 (and the per-expert forms
+ * moe_expert_ffn / moe_expert_queue + flush, accel.rs:220-262, which are this call with one group).
+ * xs[rows][hidden] holds the rows of every expert group back to back (gathered by the caller),
+ * plan[nplan][2] = (expert, rows of the group); dy[rows][hidden] = the unweighted expert outputs,
+ * for the caller's weighted scatter.  Q8_0 and Q6_K expert layers. */
+int smx_moe_layer_ffn(smx_ctx* ctx, size_t layer, const int32_t* plan, size_t nplan, const float* xs,
+                      size_t rows, float* dy, size_t dy_cap);
+int smx_moe_expert_ffn(smx_ctx* ctx, size_t layer, size_t expert, const float* xs, size_t m, float* y,
+                       size_t y_cap);
 int smx_moe_layer(smx_ctx* ctx, size_t layer, const float* xs, size_t m, const size_t* plan,
                   size_t nplan, const int32_t* slot_tok, const float* wslot, size_t slots,
                   float* y, size_t y_cap);

@@ -27,7 +27,7 @@ EXPORTS = [
     "smx_resident_bytes", "smx_upload_q4_0", "smx_upload_q8_0", "smx_upload_q6_k",
     "smx_upload_moe_q8", "smx_evict", "smx_gemv", "smx_gemv_rows", "smx_gemv_batch", "smx_gemm",
     "smx_lm_head_argmax_rows", "smx_moe_ffn", "smx_moe_layer", "smx_dev_alloc", "smx_dev_free",
-    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev", "smx_moe_shexp_dev",
+    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev", "smx_moe_shexp_dev", "smx_moe_layer_ffn", "smx_moe_expert_ffn",
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
@@ -96,6 +96,8 @@ def load_library():
     L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_moe_shexp_dev.argtypes = [vp, sz, C.c_float, vp, vp]
+    L.smx_moe_layer_ffn.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz]
+    L.smx_moe_expert_ffn.argtypes = [vp, sz, sz, vp, sz, vp, sz]
     L.smx_prof_enable.argtypes = [vp, i]
     L.smx_prof_reset.argtypes = [vp]
     L.smx_prof_read.argtypes = [vp, cp, C.POINTER(C.c_double), C.POINTER(sz)]
@@ -381,6 +383,20 @@ class Mi355WeightAccel:
         y = np.empty_like(xs)
         ok = self._check(self._L.smx_moe_layer(self._h, layer, _p(xs), m, _p(plan), plan.shape[0],
                                                _p(slot_tok), _p(wslot), slot_tok.size, _p(y), y.size))
+        return y if ok else None
+
+    def moe_layer_ffn(self, layer, plan, xs, rows):
+        """plan: (expert, rows) pairs; xs[rows][hidden] expert-major; returns dy[rows][hidden] (accel.rs:238-246)."""
+        plan = _c(plan, np.int32).reshape(-1, 2)
+        xs = _c(xs, np.float32).reshape(rows, -1)
+        dy = np.empty_like(xs)
+        ok = self._check(self._L.smx_moe_layer_ffn(self._h, layer, _p(plan), plan.shape[0], _p(xs), rows, _p(dy), dy.size))
+        return dy if ok else None
+
+    def moe_expert_ffn(self, layer, expert, xs, m):
+        xs = _c(xs, np.float32).reshape(m, -1)
+        y = np.empty_like(xs)
+        ok = self._check(self._L.smx_moe_expert_ffn(self._h, layer, expert, _p(xs), m, _p(y), y.size))
         return y if ok else None
 
     def moe_layer_resident(self, layer, xs_dev, m, plan, slot_tok, wslot, y_dev):

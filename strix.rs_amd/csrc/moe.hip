@@ -471,53 +471,17 @@ int smx_moe_shexp_dev(smx_ctx* c, size_t layer, float sgate, const float* x_dev,
     return shexp_enqueue(c, layer, it->second.hidden, sgate, x_dev, y_dev);
 }
 
-// xs / y on the host (copied in and out, one sync) or, with on_device, device pointers (enqueue only).
-static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
-                          const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap,
-                          bool on_device) {
-    if (!c) return SMX_ERR_ARG;
-    if (!xs || !plan || !slot_tok || !wslot || !y) return fail(c, SMX_ERR_ARG, "moe_layer: null argument");
-    auto it = c->moe.find(layer);
-    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
-    const MoeLayer& L = it->second;
+// The grouped expert FFN over a slot table: quantise the m activation rows, gate and up of every
+// expert group in one GEMM launch (slot s reads activation row rowmap[s], or row s when rowmap is
+// null), silu(g)*u re-quantised, down in a second GEMM launch.  dy[slots][hidden] is left in c->work.
+// plan3 = (expert, slot_off, count) entries tiling [0, slots); tiles go to c->tab at tab_off.
+static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const size_t* plan3, size_t nplan, const float* x_dev, size_t m,
+                             const int* rowmap_dev, size_t slots, size_t tab_off, float** dy_out) {
     const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
-    if (m == 0 || slots == 0) return fail(c, SMX_ERR_ARG, "moe_layer: m %zu, slots %zu", m, slots);  // decode.rs:1622
-    if (y_cap < m * hidden) return fail(c, SMX_ERR_ARG, "moe_layer: output capacity %zu < %zu", y_cap, m * hidden);
-    if (slots > (size_t(1) << 24) || m > 65535 || m * hidden >= (size_t(1) << 31) || slots * eff >= (size_t(1) << 31) ||
-        L.ne * eff * hidden >= (size_t(1) << 31))
-        return fail(c, SMX_ERR_LIMIT, "moe_layer: m %zu / slots %zu exceed the launch limits", m, slots);
-    // the plan must tile [0, slots) with in-range experts; every slot's token must exist
-    size_t covered = 0;
-    for (size_t i = 0; i < nplan; i++) {
-        const size_t e = plan[i * 3], off = plan[i * 3 + 1], cnt = plan[i * 3 + 2];
-        if (e >= L.ne || cnt == 0 || off != covered || off + cnt > slots)
-            return fail(c, SMX_ERR_ARG, "moe_layer: plan entry %zu (expert %zu, off %zu, count %zu) is inconsistent", i, e, off, cnt);
-        covered += cnt;
-    }
-    if (covered != slots) return fail(c, SMX_ERR_ARG, "moe_layer: plan covers %zu of %zu slots", covered, slots);
-    std::vector<int> tok_ptr(m + 1, 0), tok_slots(slots);
-    for (size_t s = 0; s < slots; s++) {
-        if (slot_tok[s] < 0 || (size_t)slot_tok[s] >= m)
-            return fail(c, SMX_ERR_ARG, "moe_layer: slot %zu names token %d of %zu", s, slot_tok[s], m);
-        tok_ptr[slot_tok[s] + 1]++;
-    }
-    for (size_t t = 0; t < m; t++) tok_ptr[t + 1] += tok_ptr[t];
-    {
-        std::vector<int> fill(tok_ptr.begin(), tok_ptr.end() - 1);
-        for (size_t s = 0; s < slots; s++) tok_slots[fill[slot_tok[s]]++] = (int)s;  // ascending slot order per token
-    }
     std::vector<GemmTile> tiles_gu, tiles_dn;
-    build_tiles(plan, nplan, eff, &tiles_gu);
-    build_tiles(plan, nplan, hidden, &tiles_dn);
-
-    SMX_HIP(c, hipSetDevice(c->device));
+    build_tiles(plan3, nplan, eff, &tiles_gu);
+    build_tiles(plan3, nplan, hidden, &tiles_dn);
     int rc;
-    if (!on_device) {
-        if ((rc = ensure(c, c->xf32, m * hidden * 4)) != SMX_OK) return rc;
-        if ((rc = ensure(c, c->yf32, m * hidden * 4)) != SMX_OK) return rc;
-    }
-    const float* x_dev = on_device ? xs : (const float*)c->xf32.p;
-    float* y_dev = on_device ? y : (float*)c->yf32.p;
     if ((rc = ensure(c, c->xq, m * hidden)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->xd, m * nb * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->xs, m * nb * 4)) != SMX_OK) return rc;
@@ -526,22 +490,17 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
                  o_ad = cv.take(slots * enb * 4), o_dy = cv.take(slots * hidden * 4);
     if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
     Carver ct;
-    const size_t o_st = ct.take(slots * 4), o_ws = ct.take(slots * 4), o_tp = ct.take((m + 1) * 4), o_ts = ct.take(slots * 4),
-                 o_t1 = ct.take(tiles_gu.size() * sizeof(GemmTile)), o_t2 = ct.take(tiles_dn.size() * sizeof(GemmTile));
-    if ((rc = ensure(c, c->tab, ct.off)) != SMX_OK) return rc;
+    ct.off = tab_off;
+    const size_t o_t1 = ct.take(tiles_gu.size() * sizeof(GemmTile)), o_t2 = ct.take(tiles_dn.size() * sizeof(GemmTile));
+    if (c->tab.cap < ct.off) return fail(c, SMX_ERR_ARG, "moe: table scratch of %zu bytes was not reserved", ct.off);
     float* g = (float*)(c->work.p + o_g);
     float* u = (float*)(c->work.p + o_u);
     int8_t* aq = (int8_t*)(c->work.p + o_aq);
     float* ad = (float*)(c->work.p + o_ad);
     float* dy = (float*)(c->work.p + o_dy);
-    if (!on_device) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_st, slot_tok, slots * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ws, wslot, slots * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_tp, tok_ptr.data(), (m + 1) * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ts, tok_slots.data(), slots * 4, hipMemcpyHostToDevice, c->stream));
+    // the host vectors are pageable: the copies have completed when hipMemcpyAsync returns
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t1, tiles_gu.data(), tiles_gu.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
     SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t2, tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
-    // the host vectors above are pageable: the copies have completed when hipMemcpyAsync returns
     rc = launch_actquant(c, x_dev, m, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
     if (rc != SMX_OK) return rc;
     {
@@ -550,7 +509,7 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
         p.op[1] = gemm_operand(L.up, u);
         p.xq = (const int8_t*)c->xq.p;
         p.xd = (const float*)c->xd.p;
-        p.a_rowmap = (const int*)(c->tab.p + o_st);  // slot -> token: the gather of kernels.rs:1162-1171
+        p.a_rowmap = rowmap_dev;  // slot -> token: the gather of kernels.rs:1162-1171
         p.tiles = (const GemmTile*)(c->tab.p + o_t1);
         p.M = (int)slots;
         p.N = (int)eff;
@@ -577,6 +536,80 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
         rc = launch_gemm_grouped(c, L.type, p, (int)tiles_dn.size(), 1, "moe_gemm_down");
         if (rc != SMX_OK) return rc;
     }
+    *dy_out = dy;
+    return SMX_OK;
+}
+
+// bytes of c->tab the two tile tables of a plan need
+static size_t tile_table_bytes(const size_t* plan3, size_t nplan, size_t eff, size_t hidden) {
+    size_t n = 0;
+    for (size_t i = 0; i < nplan; i++) {
+        const size_t tm = (plan3[i * 3 + 2] + 127) / 128;
+        n += tm * ((eff + 127) / 128) + tm * ((hidden + 127) / 128);
+    }
+    return n * sizeof(GemmTile) + 512;
+}
+
+static int moe_check_shape(smx_ctx* c, const MoeLayer& L, size_t m, size_t slots) {
+    if (slots > (size_t(1) << 24) || m > (size_t(1) << 24) || m * L.hidden >= (size_t(1) << 31) || slots * L.eff >= (size_t(1) << 31) ||
+        slots * L.hidden >= (size_t(1) << 31) || L.ne * L.eff * L.hidden >= (size_t(1) << 31))
+        return fail(c, SMX_ERR_LIMIT, "moe: m %zu / slots %zu exceed the launch limits", m, slots);
+    return SMX_OK;
+}
+
+// xs / y on the host (copied in and out, one sync) or, with on_device, device pointers (enqueue only).
+static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
+                          const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap,
+                          bool on_device) {
+    if (!c) return SMX_ERR_ARG;
+    if (!xs || !plan || !slot_tok || !wslot || !y) return fail(c, SMX_ERR_ARG, "moe_layer: null argument");
+    auto it = c->moe.find(layer);
+    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+    const MoeLayer& L = it->second;
+    const size_t hidden = L.hidden;
+    if (m == 0 || slots == 0) return fail(c, SMX_ERR_ARG, "moe_layer: m %zu, slots %zu", m, slots);  // decode.rs:1622
+    if (y_cap < m * hidden) return fail(c, SMX_ERR_ARG, "moe_layer: output capacity %zu < %zu", y_cap, m * hidden);
+    int rc = moe_check_shape(c, L, m, slots);
+    if (rc != SMX_OK) return rc;
+    if (m > 65535) return fail(c, SMX_ERR_LIMIT, "moe_layer: %zu tokens (the combine launch takes 65535)", m);
+    // the plan must tile [0, slots) with in-range experts; every slot's token must exist
+    size_t covered = 0;
+    for (size_t i = 0; i < nplan; i++) {
+        const size_t e = plan[i * 3], off = plan[i * 3 + 1], cnt = plan[i * 3 + 2];
+        if (e >= L.ne || cnt == 0 || off != covered || off + cnt > slots)
+            return fail(c, SMX_ERR_ARG, "moe_layer: plan entry %zu (expert %zu, off %zu, count %zu) is inconsistent", i, e, off, cnt);
+        covered += cnt;
+    }
+    if (covered != slots) return fail(c, SMX_ERR_ARG, "moe_layer: plan covers %zu of %zu slots", covered, slots);
+    std::vector<int> tok_ptr(m + 1, 0), tok_slots(slots);
+    for (size_t s = 0; s < slots; s++) {
+        if (slot_tok[s] < 0 || (size_t)slot_tok[s] >= m)
+            return fail(c, SMX_ERR_ARG, "moe_layer: slot %zu names token %d of %zu", s, slot_tok[s], m);
+        tok_ptr[slot_tok[s] + 1]++;
+    }
+    for (size_t t = 0; t < m; t++) tok_ptr[t + 1] += tok_ptr[t];
+    {
+        std::vector<int> fill(tok_ptr.begin(), tok_ptr.end() - 1);
+        for (size_t s = 0; s < slots; s++) tok_slots[fill[slot_tok[s]]++] = (int)s;  // ascending slot order per token
+    }
+    SMX_HIP(c, hipSetDevice(c->device));
+    if (!on_device) {
+        if ((rc = ensure(c, c->xf32, m * hidden * 4)) != SMX_OK) return rc;
+        if ((rc = ensure(c, c->yf32, m * hidden * 4)) != SMX_OK) return rc;
+    }
+    const float* x_dev = on_device ? xs : (const float*)c->xf32.p;
+    float* y_dev = on_device ? y : (float*)c->yf32.p;
+    Carver ct;
+    const size_t o_st = ct.take(slots * 4), o_ws = ct.take(slots * 4), o_tp = ct.take((m + 1) * 4), o_ts = ct.take(slots * 4);
+    if ((rc = ensure(c, c->tab, ct.off + tile_table_bytes(plan, nplan, L.eff, hidden))) != SMX_OK) return rc;
+    if (!on_device) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_st, slot_tok, slots * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ws, wslot, slots * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_tp, tok_ptr.data(), (m + 1) * 4, hipMemcpyHostToDevice, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ts, tok_slots.data(), slots * 4, hipMemcpyHostToDevice, c->stream));
+    float* dy = nullptr;
+    rc = moe_slots_enqueue(c, L, plan, nplan, x_dev, m, (const int*)(c->tab.p + o_st), slots, ct.off, &dy);
+    if (rc != SMX_OK) return rc;
     {
         ProfScope ps(c, "moe_combine");
         hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((hidden + 255) / 256), (unsigned)m), dim3(256), 0, c->stream,
@@ -589,6 +622,50 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
         SMX_HIP(c, hipStreamSynchronize(c->stream));
     }
     return SMX_OK;
+}
+
+// WeightAccel::moe_layer_ffn (accel.rs:238-246, decode.rs:3552-3629): xs holds the rows of every
+// expert group back to back (expert-major, already gathered by the caller), plan = (expert, rows)
+// pairs; returns the unweighted expert outputs dy[rows][hidden] for the caller's weighted scatter.
+int smx_moe_layer_ffn(smx_ctx* c, size_t layer, const int32_t* plan, size_t nplan, const float* xs, size_t rows, float* dy,
+                      size_t dy_cap) {
+    if (!c) return SMX_ERR_ARG;
+    if (!plan || !xs || !dy) return fail(c, SMX_ERR_ARG, "moe_layer_ffn: null argument");
+    auto it = c->moe.find(layer);
+    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+    const MoeLayer& L = it->second;
+    const size_t hidden = L.hidden;
+    if (rows == 0 || nplan == 0) return fail(c, SMX_ERR_ARG, "moe_layer_ffn: %zu rows in %zu groups", rows, nplan);
+    if (dy_cap < rows * hidden) return fail(c, SMX_ERR_ARG, "moe_layer_ffn: output capacity %zu < %zu", dy_cap, rows * hidden);
+    int rc = moe_check_shape(c, L, rows, rows);
+    if (rc != SMX_OK) return rc;
+    std::vector<size_t> plan3(nplan * 3);
+    size_t off = 0;
+    for (size_t i = 0; i < nplan; i++) {
+        const int e = plan[i * 2], cnt = plan[i * 2 + 1];
+        if (e < 0 || (size_t)e >= L.ne || cnt <= 0)
+            return fail(c, SMX_ERR_ARG, "moe_layer_ffn: group %zu (expert %d, %d rows) is inconsistent", i, e, cnt);
+        plan3[i * 3] = (size_t)e; plan3[i * 3 + 1] = off; plan3[i * 3 + 2] = (size_t)cnt;
+        off += (size_t)cnt;
+    }
+    if (off != rows) return fail(c, SMX_ERR_ARG, "moe_layer_ffn: the groups hold %zu rows, the call says %zu", off, rows);
+    SMX_HIP(c, hipSetDevice(c->device));
+    if ((rc = ensure(c, c->xf32, rows * hidden * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->tab, tile_table_bytes(plan3.data(), nplan, L.eff, hidden))) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, rows * hidden * 4, hipMemcpyHostToDevice, c->stream));
+    float* dy_dev = nullptr;
+    rc = moe_slots_enqueue(c, L, plan3.data(), nplan, (const float*)c->xf32.p, rows, nullptr, rows, 0, &dy_dev);
+    if (rc != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(dy, dy_dev, rows * hidden * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+// WeightAccel::moe_expert_ffn (accel.rs:220-223): one expert's FFN for m grouped rows, one sync.
+int smx_moe_expert_ffn(smx_ctx* c, size_t layer, size_t expert, const float* xs, size_t m, float* y, size_t y_cap) {
+    if (expert > 0x7fffffffu || m > 0x7fffffffu) return c ? fail(c, SMX_ERR_ARG, "moe_expert_ffn: expert %zu, %zu rows", expert, m) : SMX_ERR_ARG;
+    const int32_t plan[2] = {(int32_t)expert, (int32_t)m};
+    return smx_moe_layer_ffn(c, layer, plan, 1, xs, m, y, y_cap);
 }
 
 int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,

@@ -101,6 +101,16 @@ class Mi355WeightAccel final : public WeightAccel {
         smx_gguf_close(g);
         return ok(ru);
     }
+    // accel.rs:238-246 moe_layer_ffn: plan = (expert, rows) pairs over expert-major rows; returns dy[rows][hidden]
+    std::optional<std::vector<float>> moe_layer_ffn(size_t layer, const std::vector<std::pair<int32_t, int32_t>>& plan,
+                                                    const std::vector<float>& xs, size_t rows) {
+        if (rows == 0 || xs.size() % rows != 0) return std::nullopt;
+        std::vector<int32_t> flat;
+        for (const auto& p : plan) { flat.push_back(p.first); flat.push_back(p.second); }
+        std::vector<float> dy(xs.size());
+        if (!ok(smx_moe_layer_ffn(ctx_, layer, flat.data(), plan.size(), xs.data(), rows, dy.data(), dy.size()))) return std::nullopt;
+        return dy;
+    }
     // accel.rs:185-196
     bool upload_moe_q6(size_t layer, const uint8_t* gate, size_t gate_n, const uint8_t* up, size_t up_n, const uint8_t* down,
                        size_t down_n, size_t hidden, size_t eff, size_t ne) {

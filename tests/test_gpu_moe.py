@@ -147,6 +147,36 @@ def test_moe_layer_q6k_experts(accel, orc, synth, relerr, ne, hidden, eff, k, m)
         assert relerr(y[t], yt) <= 2e-2
 
 
+@pytest.mark.parametrize("ty", [8, 14])
+def test_moe_layer_ffn_and_expert_ffn(accel, orc, synth, relerr, pkg, ty):
+    """moe_layer_ffn (expert-major rows in, unweighted expert outputs out; decode.rs:3552-3629) and
+    moe_expert_ffn: each output row is that expert's FFN of its input row."""
+    ne, hidden, eff, layer = 8, 512, 256, 27
+    gate, up, down = (synth.make_moe_q8 if ty == 8 else synth.make_moe_q6)(ne, hidden, eff, seed=70)
+    assert (accel.upload_moe_q8 if ty == 8 else accel.upload_moe_q6)(layer, gate, up, down, hidden, eff, ne)
+    plan = [(5, 3), (0, 140), (7, 1), (2, 33)]          # an expert may come in any order; one group spans two tiles
+    rows = sum(n for _, n in plan)
+    xs = synth.make_acts(rows, hidden, seed=71)
+    dy = accel.moe_layer_ffn(layer, plan, xs, rows)
+    assert dy.shape == (rows, hidden)
+    r = 0
+    for e, n in plan:
+        for t in (r, r + n - 1):
+            one = np.array([1.0], np.float32)
+            yd, gu, aq, ad = accel.moe_ffn_stages(layer, [e], one, xs[t], eff)      # the decode path, weight 1
+            ref, _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, np.array([e], np.int32), one, xs[t], aq_in=aq, ad_in=ad, ty=ty)
+            assert relerr(yd, ref) <= TOL
+            assert relerr(dy[t], yd) <= 2e-2            # chains differ only at quantiser rounding boundaries
+        r += n
+    ye = accel.moe_expert_ffn(layer, 2, xs[-33:], 33)
+    assert np.array_equal(ye, dy[-33:])
+    assert accel.moe_layer_ffn(999, plan, xs, rows) is None
+    with pytest.raises(pkg.SmxError):
+        accel.moe_layer_ffn(layer, [(8, 3)], xs[:3], 3)             # expert out of range
+    with pytest.raises(pkg.SmxError):
+        accel.moe_layer_ffn(layer, [(1, 3)], xs[:4], 4)             # groups do not cover the rows
+
+
 def test_moe_layer_resident_equals_host_call(accel, synth, pkg):
     ne, hidden, eff, k, m = 8, 256, 96, 3, 70
     _layer(accel, synth, 9, ne, hidden, eff, seed=33)
