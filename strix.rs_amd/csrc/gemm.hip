@@ -186,8 +186,11 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const unsigned sB = sA + A_BYTES;
         const int blk0 = s * KB;
         const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
+        // 8-row groups wholly past the tile's end (ragged expert groups) are not fetched: nothing reads
+        // their LDS rows but lanes whose results are dropped
 #pragma unroll
-        for (int ps = 0; ps < 4; ps++) load_to_lds16(p.xq + a_off[ps] + koff, sA + ps * NW * GRP);
+        for (int ps = 0; ps < 4; ps++)
+            if (tok0 + (ps * NW + wave) * 8 < M_end) load_to_lds16(p.xq + a_off[ps] + koff, sA + ps * NW * GRP);
         if (Q6) {
             const size_t sbi = (size_t)b_off[0] + (s >> 1);
             const char* ql = (const char*)op.wquants + sbi * 128 + (s & 1) * 64 + q6_p * 16;
