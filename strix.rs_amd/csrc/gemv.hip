@@ -92,7 +92,10 @@ int launch_variant(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
     }
     if (g.ks == 4) return launch_one<Ops, MT, 1, 2, 4, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
     if (g.ks == 2) return launch_one<Ops, MT, 1, 2, 2, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
-    if (g.rpw == 1) return launch_one<Ops, MT, 1, 4, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
+    // 8 activation rows (4 with Q6_K's wide units): a ring of 4 units spills (128 registers per lane at
+    // 16 waves), and the scratch traffic costs more than the shallower pipeline: 2 fit
+    constexpr int kPre1 = (MT == 8 || (kWide && MT == 4)) ? 2 : 4;
+    if (g.rpw == 1) return launch_one<Ops, MT, 1, kPre1, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
     if (g.rpw == 4 && MT == 1) return launch_one<Ops, 1, 4, 2, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
     return launch_one<Ops, MT, 2, 2, 1, 64, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
 }

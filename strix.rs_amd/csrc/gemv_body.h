@@ -412,39 +412,32 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
     }
 }
 
-// Stage m pre-quantised activation rows: every global load of all rows is requested before the
-// first LDS write, so the staging costs one memory round trip, not one per row.
+// Stage m pre-quantised activation rows, 16 bytes (half a block) per thread and load: every global
+// load of all rows is requested before the first LDS write, so the staging costs one memory round
+// trip, not one per row.  All formats keep a block's two 16-byte halves whole in LDS (xq_dword(.., 0)
+// and (.., 4) are 16-byte aligned), so a half moves as one 128-bit load and one 128-bit store.
 template <class Ops, int MT>
 __device__ __forceinline__ void stage_prequant_all(char* smem, int tokb, int nblk, const GemvX& X, int m) {
     const int nb32 = Ops::nb32(nblk);
-    const int items = nb32 * 8;
-    constexpr int SB = 2;
-    for (int i0 = threadIdx.x; i0 < items; i0 += blockDim.x * SB) {
-        int pk[MT][SB], sp[MT][SB];
-        float d[MT][SB];
+    const int items = nb32 * 2;
+    for (int i = threadIdx.x; i < items; i += blockDim.x) {
+        uint4 pk[MT];
+        int sp[MT];
+        float d[MT];
+        const bool head = (i & 1) == 0;
 #pragma unroll
-        for (int t = 0; t < MT; t++)
+        for (int t = 0; t < MT; t++) {
+            const bool live = t < m;
+            pk[t] = live ? ((const uint4*)(X.xq + (size_t)t * nb32 * 32))[i] : make_uint4(0, 0, 0, 0);
+            d[t] = (live && head) ? X.xd[(size_t)t * nb32 + (i >> 1)] : 0.f;
+            sp[t] = (live && head && Ops::kNeedsSums) ? X.xs[(size_t)t * nb32 + (i >> 1)] : 0;
+        }
 #pragma unroll
-            for (int j = 0; j < SB; j++) {
-                const int i = i0 + j * blockDim.x;
-                const bool live = i < items && t < m;
-                pk[t][j] = live ? ((const int*)(X.xq + (size_t)t * nb32 * 32))[i] : 0;
-                const bool head = live && (i & 7) == 0;
-                d[t][j] = head ? X.xd[(size_t)t * nb32 + (i >> 3)] : 0.f;
-                sp[t][j] = (head && Ops::kNeedsSums) ? X.xs[(size_t)t * nb32 + (i >> 3)] : 0;
-            }
-#pragma unroll
-        for (int t = 0; t < MT; t++)
-#pragma unroll
-            for (int j = 0; j < SB; j++) {
-                const int i = i0 + j * blockDim.x;
-                if (i < items) {
-                    char* tok = smem + t * tokb;
-                    *Ops::xq_dword(tok, nblk, i >> 3, i & 7) = pk[t][j];
-                    if ((i & 7) == 0)
-                        Ops::put_scale(tok, nblk, i >> 3, d[t][j], (int)(short)(sp[t][j] & 0xffff), sp[t][j] >> 16);
-                }
-            }
+        for (int t = 0; t < MT; t++) {
+            char* tok = smem + t * tokb;
+            *(uint4*)Ops::xq_dword(tok, nblk, i >> 1, (i & 1) * 4) = pk[t];
+            if (head) Ops::put_scale(tok, nblk, i >> 1, d[t], (int)(short)(sp[t] & 0xffff), sp[t] >> 16);
+        }
     }
 }
 
