@@ -229,6 +229,36 @@ class Bench:
                 "algorithmic_bytes": algo, "steps": steps, "ms_per_step": ms / steps, "GBps": gbs,
                 "frac_hbm_peak": gbs / HBM_PEAK_GBS}
 
+    # ------------------------------------------------------------------ dense FFN prefill block (3 GEMMs)
+    def ffn_prefill_block(self, name, ty, H, F, M, steps=None, warmup=None):
+        """M tokens through a dense FFN: rmsnorm + quantiser + gate GEMM, the same for up, then
+        SwiGLU + quantiser + down GEMM (each producer runs inside its quantiser launch)."""
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or max(5, self.steps // 20), warmup if warmup is not None else 2
+        up_fn = getattr(acc, UPLOAD[ty])
+        assert up_fn(name + ".g", sy.make_weight(ty, F, H, seed=1700), H, F)
+        assert up_fn(name + ".u", sy.make_weight(ty, F, H, seed=1701), H, F)
+        assert up_fn(name + ".d", sy.make_weight(ty, H, F, seed=1702), F, H)
+        x = sy.make_acts(M, H, seed=7)
+        xd, wd, gd, ud, yd = (acc.dev_alloc(n * 4) for n in (M * H, H, M * F, M * F, M * H))
+        acc.h2d(xd, x)
+        acc.h2d(wd, np.ones(H, np.float32))
+
+        def step(i):
+            acc.gemm_fused_dev(name + ".g", 1, xd, wd, M, gd, 1e-6)
+            acc.gemm_fused_dev(name + ".u", 1, xd, wd, M, ud, 1e-6)
+            acc.gemm_fused_dev(name + ".d", 2, gd, ud, M, yd)
+
+        ms, wall_ms = self._timed(step, steps, warmup)
+        for t in "gud":
+            acc.evict(f"{name}.{t}")
+        for p in (xd, wd, gd, ud, yd):
+            acc.dev_free(p)
+        ops = 3 * 2 * M * F * H
+        tops = ops * steps / (ms * 1e-3) / 1e12
+        return {"workload": name, "shape": {"hidden": H, "ffn": F, "M": M, "gemms_per_step": 3}, "ops": ops, "steps": steps,
+                "ms_per_step": ms / steps, "TOPS": tops, "frac_int8_peak": tops / INT8_PEAK_TOPS}
+
     # ------------------------------------------------------------------ copy (counter calibration)
     def copy_calib(self, nbytes=256 << 20, steps=20):
         """A plain copy of known size: what FETCH_SIZE / WRITE_SIZE read for it scales the counters."""
@@ -414,6 +444,7 @@ def main():
         ("gemm_q4_0_ffn_up", lambda: b.gemm("gemm_q4_0_ffn_up", Q4_0, 2048, 15360, 3840)),
         ("gemm_q8_0_ffn_down", lambda: b.gemm("gemm_q8_0_ffn_down", Q8_0, 2048, 3840, 15360)),
         ("gemm_q4_0_ffn_down", lambda: b.gemm("gemm_q4_0_ffn_down", Q4_0, 2048, 3840, 15360)),
+        ("q8_0_ffn_prefill_block_m2048", lambda: b.ffn_prefill_block("q8_0_ffn_prefill_block_m2048", Q8_0, 3840, 15360, 2048)),
         ("gemm_q6_k_ffn_up", lambda: b.gemm("gemm_q6_k_ffn_up", Q6_K, 2048, 15360, 3840)),
         ("gemm_q6_k_ffn_down", lambda: b.gemm("gemm_q6_k_ffn_down", Q6_K, 2048, 3840, 15360)),
         ("moe_decode", lambda: b.moe("moe_decode", 64, 2048, 768, 8, 1, layers=4)),

@@ -163,6 +163,12 @@ int smx_gemv_fused_dev(smx_ctx* ctx, size_t n, const char* const* keys, int act,
                        const float* b_dev, float eps, float* const* ys_dev);
 int smx_gemv_fused(smx_ctx* ctx, const char* key, int act, const float* a, const float* b, size_t in_len,
                    float eps, float* y, size_t out_cap);
+/* The prefill form (kernels.rs:1174-1187 silu_quant_rows, :1000-1013 xquant8_rows behind a norm): m rows
+ * a_dev[m][in_dim] go through the producer inside the quantiser launch that feeds the int8 GEMM, so the
+ * normalised / gated fp32 rows are never written.  b_dev: the norm weight [in_dim] (or NULL) for RMSNORM,
+ * the second operand [m][in_dim] for SILU_MUL / GEGLU.  y_dev[m][out_dim]. */
+int smx_gemm_fused_dev(smx_ctx* ctx, const char* key, int act, const float* a_dev, const float* b_dev, size_t m,
+                       float eps, float* y_dev);
 
 /* y_dev += sgate * shared_expert(x_dev) for layer `layer` (the second half of moe_ffn with a shared
  * expert, decode.rs:1820-1855), to follow smx_moe_ffn_dev on device-resident activations. */

@@ -27,7 +27,7 @@ EXPORTS = [
     "smx_resident_bytes", "smx_upload_q4_0", "smx_upload_q8_0", "smx_upload_q6_k",
     "smx_upload_moe_q8", "smx_evict", "smx_gemv", "smx_gemv_rows", "smx_gemv_batch", "smx_gemm",
     "smx_lm_head_argmax_rows", "smx_moe_ffn", "smx_moe_layer", "smx_dev_alloc", "smx_dev_free",
-    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev", "smx_moe_shexp_dev", "smx_moe_layer_ffn", "smx_moe_expert_ffn",
+    "smx_h2d", "smx_d2h", "smx_sync", "smx_gemv_dev", "smx_gemm_dev", "smx_moe_ffn_dev", "smx_moe_shexp_dev", "smx_gemm_fused_dev", "smx_moe_layer_ffn", "smx_moe_expert_ffn",
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
@@ -96,6 +96,7 @@ def load_library():
     L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_moe_shexp_dev.argtypes = [vp, sz, C.c_float, vp, vp]
+    L.smx_gemm_fused_dev.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp]
     L.smx_moe_layer_ffn.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz]
     L.smx_moe_expert_ffn.argtypes = [vp, sz, sz, vp, sz, vp, sz]
     L.smx_prof_enable.argtypes = [vp, i]
@@ -477,6 +478,10 @@ class Mi355WeightAccel:
         k = (C.c_char_p * n)(*[s.encode() for s in keys])
         yp = (C.c_void_p * n)(*ys_dev)
         return self._check(self._L.smx_gemv_fused_dev(self._h, n, k, int(act), a_dev, b_dev, float(eps), yp))
+
+    def gemm_fused_dev(self, key, act, a_dev, b_dev, m, y_dev, eps=0.0):
+        """Prefill rows through a producer + quantiser + int8 GEMM (see smx_gemm_fused_dev)."""
+        return self._check(self._L.smx_gemm_fused_dev(self._h, key.encode(), int(act), a_dev, b_dev, m, float(eps), y_dev))
 
     def gemm_dev(self, key, xs_dev, m, y_dev):
         return self._check(self._L.smx_gemm_dev(self._h, key.encode(), xs_dev, m, y_dev))

@@ -62,6 +62,73 @@ __global__ __launch_bounds__(256) void actprod_quant_kernel(const ProdRows R, in
     }
 }
 
+// m rows through an activation producer and the quantiser, one workgroup per row: the prefill form of
+// the producers (kernels.rs:101-147 rmsnorm_xquant per row, :1174-1187 silu_quant_rows).  b: rmsnorm
+// weight [K] (or null) shared by the rows (b_stride 0), or the second operand [m][K] of silu / gelu.
+__global__ __launch_bounds__(256) void rows_prod_quant_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                              size_t b_stride, int kind, float eps, int* __restrict__ xq4,
+                                                              float* __restrict__ xd, int* __restrict__ xs, int nb32) {
+#pragma clang fp contract(off)
+    __shared__ double red[4];
+    const size_t row = blockIdx.x;
+    const float* ar = a + row * (size_t)nb32 * 32;
+    const float* br = b ? b + row * b_stride : nullptr;
+    float rs = 1.f;
+    if (kind == SMX_ACT_RMSNORM) rs = rms_scale((char*)red, ar, nb32 * 32, eps);
+    const int items = nb32 * 8;
+    for (int i0 = 0; i0 < items; i0 += 256) {  // whole 8-lane groups stay together: items % 8 == 0
+        const int i = i0 + threadIdx.x;
+        const bool live = i < items;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f), g = make_float4(1.f, 1.f, 1.f, 1.f);
+        if (live) {
+            v = ((const float4*)ar)[i];
+            if (br) g = ((const float4*)br)[i];
+        }
+        float4 w;
+        if (kind == SMX_ACT_RMSNORM) {
+            w.x = (v.x * rs) * g.x; w.y = (v.y * rs) * g.y; w.z = (v.z * rs) * g.z; w.w = (v.w * rs) * g.w;
+        } else if (kind == SMX_ACT_SILU_MUL) {
+            w.x = det_silu(v.x) * g.x; w.y = det_silu(v.y) * g.y; w.z = det_silu(v.z) * g.z; w.w = det_silu(v.w) * g.w;
+        } else {
+            w.x = det_gelu_tanh(v.x) * g.x; w.y = det_gelu_tanh(v.y) * g.y;
+            w.z = det_gelu_tanh(v.z) * g.z; w.w = det_gelu_tanh(v.w) * g.w;
+        }
+        float am = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
+        am = fmaxf(am, __shfl_xor(am, 1));
+        am = fmaxf(am, __shfl_xor(am, 2));
+        am = fmaxf(am, __shfl_xor(am, 4));
+        const float d = am / 127.f;
+        const float inv = d > 0.f ? 1.f / d : 0.f;
+        const int q0 = max(-127, min(127, (int)rintf(w.x * inv)));
+        const int q1 = max(-127, min(127, (int)rintf(w.y * inv)));
+        const int q2 = max(-127, min(127, (int)rintf(w.z * inv)));
+        const int q3 = max(-127, min(127, (int)rintf(w.w * inv)));
+        int s = q0 + q1 + q2 + q3;
+        s += __shfl_xor(s, 1);
+        s += __shfl_xor(s, 2);
+        const int other = __shfl_xor(s, 4);
+        if (live) {
+            xq4[row * (size_t)items + i] = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+            if ((i & 7) == 0) {
+                xd[row * (size_t)nb32 + (i >> 3)] = d;
+                xs[row * (size_t)nb32 + (i >> 3)] = (s & 0xffff) | (other << 16);
+            }
+        }
+    }
+}
+
+int launch_rows_prod_quant(smx_ctx* c, int kind, const float* a, const float* b, size_t m, size_t K, float eps, int8_t* xq,
+                           float* xd, int32_t* xs) {
+    if (K % 32 != 0 || m == 0 || m > 0x7fffffffu) return fail(c, SMX_ERR_ARG, "producer quantiser: %zu rows of %zu", m, K);
+    if (kind != SMX_ACT_RMSNORM && kind != SMX_ACT_SILU_MUL && kind != SMX_ACT_GEGLU)
+        return fail(c, SMX_ERR_ARG, "producer quantiser: kind %d", kind);
+    ProfScope ps(c, "rows_prod_quant");
+    hipLaunchKernelGGL(rows_prod_quant_kernel, dim3((unsigned)m), dim3(256), 0, c->stream, a, b,
+                       kind == SMX_ACT_RMSNORM ? (size_t)0 : K, kind, eps, (int*)xq, xd, (int*)xs, (int)(K / 32));
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
 int launch_actprod_quant(smx_ctx* c, int kind, const float* const* as, const float* const* bs, int n, size_t K,
                          int8_t* xq, float* xd, int32_t* xs) {
     if (K % 32 != 0 || n < 1 || n > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "producer quantiser: %d rows of %zu", n, K);

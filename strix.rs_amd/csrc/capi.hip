@@ -322,6 +322,23 @@ int smx_gemv_fused(smx_ctx* c, const char* key, int act, const float* a, const f
     return SMX_OK;
 }
 
+// Prefill form of smx_gemv_fused_dev: the producer runs over m rows in the quantiser launch.
+int smx_gemm_fused_dev(smx_ctx* c, const char* key, int act, const float* a_dev, const float* b_dev, size_t m, float eps,
+                       float* y_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !y_dev) return fail(c, SMX_ERR_ARG, "gemm_fused_dev: null argument");
+    const Weight* w = find_weight(c, key);
+    if (!w) return SMX_NOT_RESIDENT;
+    if (m == 0) return fail(c, SMX_ERR_ARG, "gemm_fused_dev: zero rows");
+    int rc = gemv_fused_check(c, act, a_dev, b_dev, "gemm_fused_dev");
+    if (rc != SMX_OK) return rc;
+    if (act == SMX_ACT_NONE) return run_matmul_dev(c, *w, a_dev, m, y_dev, true, nullptr);
+    if ((rc = ensure_act(c, m, w->K)) != SMX_OK) return rc;
+    rc = launch_rows_prod_quant(c, act, a_dev, b_dev, m, w->K, eps, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+    if (rc != SMX_OK) return rc;
+    return launch_gemm(c, *w, (const int8_t*)c->xq.p, (const float*)c->xd.p, m, y_dev, nullptr);
+}
+
 int smx_gemm_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, float* y_dev) {
     if (!c) return SMX_ERR_ARG;
     if (!key || !xs_dev || !y_dev) return fail(c, SMX_ERR_ARG, "gemm_dev: null argument");

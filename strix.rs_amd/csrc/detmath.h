@@ -49,4 +49,29 @@ __device__ __forceinline__ float det_gelu_tanh(float x) {
     return 0.5f * x * (1.0f + det_tanhf(inner));
 }
 
+// 1/sqrt(mean(x^2) + eps) of one row for the rmsnorm producer (kernels.rs:101-113).  The squares are
+// summed in double by the whole workgroup (per thread, per wave, then over the waves in index order)
+// and the scale is rounded to fp32 once, so it does not depend on the workgroup's shape.  `scratch`
+// is LDS the caller has not written yet; every thread of the workgroup must call this.
+__device__ __forceinline__ float rms_scale(char* scratch, const float* x, int n, float eps) {
+#pragma clang fp contract(off)
+    double ss = 0.0;
+    for (int i = threadIdx.x; i < n / 4; i += blockDim.x) {
+        const float4 v = ((const float4*)x)[i];
+        ss += (double)v.x * (double)v.x;
+        ss += (double)v.y * (double)v.y;
+        ss += (double)v.z * (double)v.z;
+        ss += (double)v.w * (double)v.w;
+    }
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+    double* red = (double*)scratch;
+    const int nwaves = blockDim.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    double tot = 0.0;
+    for (int w = 0; w < nwaves; w++) tot += red[w];
+    __syncthreads();  // the caller overwrites the scratch next
+    return (float)(1.0 / sqrt(tot / (double)n + (double)eps));
+}
+
 }  // namespace smx

@@ -159,6 +159,10 @@ int launch_actquant(smx_ctx* c, const float* x, size_t m, size_t K, int8_t* xq, 
 // n rows act(as[j]) * bs[j] (SMX_ACT_SILU_MUL or SMX_ACT_GEGLU), quantised: row j at xq + j*K, xd/xs + j*K/32.
 int launch_actprod_quant(smx_ctx* c, int kind, const float* const* as, const float* const* bs, int n, size_t K,
                          int8_t* xq, float* xd, int32_t* xs);
+// m rows [m][K] through a producer (SMX_ACT_RMSNORM with weight b[K] or null; SMX_ACT_SILU_MUL / SMX_ACT_GEGLU with
+// b[m][K]) and the quantiser: xq[m][K], xd/xs[m][K/32].
+int launch_rows_prod_quant(smx_ctx* c, int kind, const float* a, const float* b, size_t m, size_t K, float eps, int8_t* xq,
+                           float* xd, int32_t* xs);
 // GEMV with the activation quantiser fused into its LDS staging: x fp32 [m][K] -> y[m][N],
 // m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);

@@ -81,3 +81,30 @@ def test_fused_group_launch_and_errors(accel, orc, synth, relerr, pkg):
     assert accel.gemv_fused("t.absent", 1, a, None, 8) is None
     for p in [ad, wd] + yds:
         accel.dev_free(p)
+
+
+@pytest.mark.parametrize("ty", [2, 8, 14])
+@pytest.mark.parametrize("act", [1, 2, 3])
+def test_prefill_rows_through_a_producer(accel, orc, synth, relerr, ty, act):
+    """smx_gemm_fused_dev: m rows, producer inside the quantiser launch, then the int8 GEMM; row t equals
+    the oracle's producer + quantiser + Q8 matmul of row t (kernels.rs:1174-1187 silu_quant_rows)."""
+    M, N, K = 70, 200, 1280
+    raw = synth.make_weight(ty, N, K, seed=ty + 10 * act)
+    assert getattr(accel, UP[ty])("t.pf", raw, K, N)
+    a = synth.make_acts(M, K, seed=80 + act) * 1.7
+    a[3] = 0.0                                                   # an all-zero row: scale 0, quants 0
+    b = (synth.make_acts(1, K, seed=90)[0] * 0.1 + 1.0) if act == 1 else (synth.make_acts(M, K, seed=91) * 0.5 + 1.0)
+    eps = 1e-6 if act == 1 else 0.0
+    ad, bd, yd = accel.dev_alloc(a.nbytes), accel.dev_alloc(b.nbytes), accel.dev_alloc(M * N * 4)
+    accel.h2d(ad, a)
+    accel.h2d(bd, b)
+    assert accel.gemm_fused_dev("t.pf", act, ad, bd, M, yd, eps)
+    y = accel.d2h(np.empty((M, N), np.float32), yd)
+    x = np.stack([orc.act_produce(act, a[t], b if act == 1 else b[t], eps) for t in range(M)])
+    assert relerr(y, orc.matmul_q8_from_f32(ty, raw, K, N, x)) <= TOL
+    # the decode form of the same producer gives the same row
+    for t in (0, 3, M - 1):
+        assert relerr(y[t], accel.gemv_fused("t.pf", act, a[t], b if act == 1 else b[t], N, eps)) <= TOL
+    assert accel.gemm_fused_dev("t.absent", act, ad, bd, M, yd, eps) is False
+    for p in (ad, bd, yd):
+        accel.dev_free(p)
