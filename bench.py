@@ -413,7 +413,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X "
-                 "(--gpus must be 1); how it would shard over several is described in DESIGN.md")
+                 "(--gpus must be 1); over several GPUs the path would shard by output rows, one all-gather per group of GEMVs")
     only = set(filter(None, a.only.split(",")))
     want = lambda n: not only or n in only
     b = Bench(a.steps, a.warmup)
