@@ -80,7 +80,7 @@ struct MoeRoute {
 // a time with all UNR loads issued before the first use.  Workgroup 0 also writes the quantised
 // activation out for the stage-by-stage checks.
 template <int UNR>
-__global__ __launch_bounds__(512) void moe_down_fused_kernel(const float* __restrict__ g, const float* __restrict__ u,
+__global__ __launch_bounds__(1024) void moe_down_fused_kernel(const float* __restrict__ g, const float* __restrict__ u,
                                                              const uint16_t* __restrict__ scales,
                                                              const uint4* __restrict__ quants, const MoeRoute route,
                                                              int k, int eff, int hidden, float* __restrict__ y,
@@ -116,11 +116,11 @@ __global__ __launch_bounds__(512) void moe_down_fused_kernel(const float* __rest
         }
     };
     const int items = k * eff / 4;  // float4 items, 8 per block; whole 8-lane groups are live or dead together
-    for (int it0 = 0; it0 < items; it0 += 512 * 4) {
-        float4 gv[4], uv[4];
+    for (int it0 = 0; it0 < items; it0 += 1024 * 2) {
+        float4 gv[2], uv[2];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int it = it0 + j * 512 + tid;
+        for (int j = 0; j < 2; j++) {
+            const int it = it0 + j * 1024 + tid;
             gv[j] = uv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (it < items) {
                 gv[j] = ((const float4*)g)[it];
@@ -128,8 +128,8 @@ __global__ __launch_bounds__(512) void moe_down_fused_kernel(const float* __rest
             }
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int it = it0 + j * 512 + tid;
+        for (int j = 0; j < 2; j++) {
+            const int it = it0 + j * 1024 + tid;
             int packed;
             float d;
             silu_mul_quant4(gv[j], uv[j], &packed, &d);
@@ -144,6 +144,7 @@ __global__ __launch_bounds__(512) void moe_down_fused_kernel(const float* __rest
         }
     }
     __syncthreads();
+    if (wave >= 8) return;  // waves 8..15 only help with the staging above
     int r = blockIdx.x * 8 + wave;
     if (r < hidden) load_chunk(r, 0);
 
@@ -325,7 +326,7 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
         static size_t lds_set = 0;
         if ((rc = set_dyn_lds(c, kern, lds, &lds_set)) != SMX_OK) return rc;
         const unsigned grid = (unsigned)std::min<size_t>((hidden + 7) / 8, (size_t)c->num_cu * 2);
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, c->stream, s.g, s.u, L.down.scales, (const uint4*)L.down.quants,
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(1024), lds, c->stream, s.g, s.u, L.down.scales, (const uint4*)L.down.quants,
                            route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad);
         SMX_HIP(c, hipGetLastError());
     }
