@@ -10,6 +10,7 @@
 // combine walks each token's slots in ascending slot order instead of fp32 atomics, so results do
 // not depend on scheduling.
 #include <algorithm>
+#include <cstring>
 #include <vector>
 
 #include "detmath.h"
@@ -475,13 +476,10 @@ int smx_moe_shexp_dev(smx_ctx* c, size_t layer, float sgate, const float* x_dev,
 // The grouped expert FFN over a slot table: quantise the m activation rows, gate and up of every
 // expert group in one GEMM launch (slot s reads activation row rowmap[s], or row s when rowmap is
 // null), silu(g)*u re-quantised, down in a second GEMM launch.  dy[slots][hidden] is left in c->work.
-// plan3 = (expert, slot_off, count) entries tiling [0, slots); tiles go to c->tab at tab_off.
-static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const size_t* plan3, size_t nplan, const float* x_dev, size_t m,
-                             const int* rowmap_dev, size_t slots, size_t tab_off, float** dy_out) {
+// The two tile tables (device pointers) are those of build_tiles over the plan for eff and hidden rows.
+static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const float* x_dev, size_t m, const int* rowmap_dev, size_t slots,
+                             const GemmTile* tiles_gu, size_t n_gu, const GemmTile* tiles_dn, size_t n_dn, float** dy_out) {
     const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
-    std::vector<GemmTile> tiles_gu, tiles_dn;
-    build_tiles(plan3, nplan, eff, &tiles_gu);
-    build_tiles(plan3, nplan, hidden, &tiles_dn);
     int rc;
     if ((rc = ensure(c, c->xq, m * hidden)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->xd, m * nb * 4)) != SMX_OK) return rc;
@@ -490,18 +488,11 @@ static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const size_t* plan3,
     const size_t o_g = cv.take(slots * eff * 4), o_u = cv.take(slots * eff * 4), o_aq = cv.take(slots * eff),
                  o_ad = cv.take(slots * enb * 4), o_dy = cv.take(slots * hidden * 4);
     if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
-    Carver ct;
-    ct.off = tab_off;
-    const size_t o_t1 = ct.take(tiles_gu.size() * sizeof(GemmTile)), o_t2 = ct.take(tiles_dn.size() * sizeof(GemmTile));
-    if (c->tab.cap < ct.off) return fail(c, SMX_ERR_ARG, "moe: table scratch of %zu bytes was not reserved", ct.off);
     float* g = (float*)(c->work.p + o_g);
     float* u = (float*)(c->work.p + o_u);
     int8_t* aq = (int8_t*)(c->work.p + o_aq);
     float* ad = (float*)(c->work.p + o_ad);
     float* dy = (float*)(c->work.p + o_dy);
-    // the host vectors are pageable: the copies have completed when hipMemcpyAsync returns
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t1, tiles_gu.data(), tiles_gu.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_t2, tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile), hipMemcpyHostToDevice, c->stream));
     rc = launch_actquant(c, x_dev, m, hidden, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
     if (rc != SMX_OK) return rc;
     {
@@ -511,13 +502,13 @@ static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const size_t* plan3,
         p.xq = (const int8_t*)c->xq.p;
         p.xd = (const float*)c->xd.p;
         p.a_rowmap = rowmap_dev;  // slot -> token: the gather of kernels.rs:1162-1171
-        p.tiles = (const GemmTile*)(c->tab.p + o_t1);
+        p.tiles = tiles_gu;
         p.M = (int)slots;
         p.N = (int)eff;
         p.nb = (int)nb;
         p.ldo = (int)eff;
         p.stages_per_slice = (int)((nb + 3) / 4);
-        rc = launch_gemm_grouped(c, L.type, p, (int)tiles_gu.size(), 2, "moe_gemm_gate_up");
+        rc = launch_gemm_grouped(c, L.type, p, (int)n_gu, 2, "moe_gemm_gate_up");
         if (rc != SMX_OK) return rc;
     }
     rc = silu_mul_quant(c, g, u, eff, slots, eff, aq, ad);
@@ -528,28 +519,37 @@ static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const size_t* plan3,
         p.op[1] = p.op[0];
         p.xq = aq;
         p.xd = ad;
-        p.tiles = (const GemmTile*)(c->tab.p + o_t2);
+        p.tiles = tiles_dn;
         p.M = (int)slots;
         p.N = (int)hidden;
         p.nb = (int)enb;
         p.ldo = (int)hidden;
         p.stages_per_slice = (int)((enb + 3) / 4);
-        rc = launch_gemm_grouped(c, L.type, p, (int)tiles_dn.size(), 1, "moe_gemm_down");
+        rc = launch_gemm_grouped(c, L.type, p, (int)n_dn, 1, "moe_gemm_down");
         if (rc != SMX_OK) return rc;
     }
     *dy_out = dy;
     return SMX_OK;
 }
 
-// bytes of c->tab the two tile tables of a plan need
-static size_t tile_table_bytes(const size_t* plan3, size_t nplan, size_t eff, size_t hidden) {
-    size_t n = 0;
-    for (size_t i = 0; i < nplan; i++) {
-        const size_t tm = (plan3[i * 3 + 2] + 127) / 128;
-        n += tm * ((eff + 127) / 128) + tm * ((hidden + 127) / 128);
+// The small tables of one call, packed on the host (256-byte aligned parts) and sent to c->tab in
+// ONE copy: six separate uploads cost about 4 us each.
+struct TableBlob {
+    std::vector<char> bytes;
+    size_t add(const void* p, size_t n) {
+        const size_t off = bytes.size();
+        bytes.resize(off + ((n + 255) & ~size_t(255)));
+        if (n) std::memcpy(bytes.data() + off, p, n);
+        return off;
     }
-    return n * sizeof(GemmTile) + 512;
-}
+    // pageable source: the copy has been staged when hipMemcpyAsync returns, the blob may go away
+    int upload(smx_ctx* c) {
+        int rc = ensure(c, c->tab, bytes.size());
+        if (rc != SMX_OK) return rc;
+        SMX_HIP(c, hipMemcpyAsync(c->tab.p, bytes.data(), bytes.size(), hipMemcpyHostToDevice, c->stream));
+        return SMX_OK;
+    }
+};
 
 static int moe_check_shape(smx_ctx* c, const MoeLayer& L, size_t m, size_t slots) {
     if (slots > (size_t(1) << 24) || m > (size_t(1) << 24) || m * L.hidden >= (size_t(1) << 31) || slots * L.eff >= (size_t(1) << 31) ||
@@ -600,16 +600,18 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
     }
     const float* x_dev = on_device ? xs : (const float*)c->xf32.p;
     float* y_dev = on_device ? y : (float*)c->yf32.p;
-    Carver ct;
-    const size_t o_st = ct.take(slots * 4), o_ws = ct.take(slots * 4), o_tp = ct.take((m + 1) * 4), o_ts = ct.take(slots * 4);
-    if ((rc = ensure(c, c->tab, ct.off + tile_table_bytes(plan, nplan, L.eff, hidden))) != SMX_OK) return rc;
+    std::vector<GemmTile> tiles_gu, tiles_dn;
+    build_tiles(plan, nplan, L.eff, &tiles_gu);
+    build_tiles(plan, nplan, hidden, &tiles_dn);
+    TableBlob tb;
+    const size_t o_st = tb.add(slot_tok, slots * 4), o_ws = tb.add(wslot, slots * 4), o_tp = tb.add(tok_ptr.data(), (m + 1) * 4),
+                 o_ts = tb.add(tok_slots.data(), slots * 4), o_t1 = tb.add(tiles_gu.data(), tiles_gu.size() * sizeof(GemmTile)),
+                 o_t2 = tb.add(tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile));
     if (!on_device) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_st, slot_tok, slots * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ws, wslot, slots * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_tp, tok_ptr.data(), (m + 1) * 4, hipMemcpyHostToDevice, c->stream));
-    SMX_HIP(c, hipMemcpyAsync(c->tab.p + o_ts, tok_slots.data(), slots * 4, hipMemcpyHostToDevice, c->stream));
+    if ((rc = tb.upload(c)) != SMX_OK) return rc;
     float* dy = nullptr;
-    rc = moe_slots_enqueue(c, L, plan, nplan, x_dev, m, (const int*)(c->tab.p + o_st), slots, ct.off, &dy);
+    rc = moe_slots_enqueue(c, L, x_dev, m, (const int*)(c->tab.p + o_st), slots, (const GemmTile*)(c->tab.p + o_t1), tiles_gu.size(),
+                           (const GemmTile*)(c->tab.p + o_t2), tiles_dn.size(), &dy);
     if (rc != SMX_OK) return rc;
     {
         ProfScope ps(c, "moe_combine");
@@ -652,10 +654,17 @@ int smx_moe_layer_ffn(smx_ctx* c, size_t layer, const int32_t* plan, size_t npla
     if (off != rows) return fail(c, SMX_ERR_ARG, "moe_layer_ffn: the groups hold %zu rows, the call says %zu", off, rows);
     SMX_HIP(c, hipSetDevice(c->device));
     if ((rc = ensure(c, c->xf32, rows * hidden * 4)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->tab, tile_table_bytes(plan3.data(), nplan, L.eff, hidden))) != SMX_OK) return rc;
+    std::vector<GemmTile> tiles_gu, tiles_dn;
+    build_tiles(plan3.data(), nplan, L.eff, &tiles_gu);
+    build_tiles(plan3.data(), nplan, hidden, &tiles_dn);
+    TableBlob tb;
+    const size_t o_t1 = tb.add(tiles_gu.data(), tiles_gu.size() * sizeof(GemmTile)),
+                 o_t2 = tb.add(tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile));
+    if ((rc = tb.upload(c)) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, rows * hidden * 4, hipMemcpyHostToDevice, c->stream));
     float* dy_dev = nullptr;
-    rc = moe_slots_enqueue(c, L, plan3.data(), nplan, (const float*)c->xf32.p, rows, nullptr, rows, 0, &dy_dev);
+    rc = moe_slots_enqueue(c, L, (const float*)c->xf32.p, rows, nullptr, rows, (const GemmTile*)(c->tab.p + o_t1), tiles_gu.size(),
+                           (const GemmTile*)(c->tab.p + o_t2), tiles_dn.size(), &dy_dev);
     if (rc != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(dy, dy_dev, rows * hidden * 4, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
