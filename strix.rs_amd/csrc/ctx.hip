@@ -239,8 +239,9 @@ void smx_destroy(smx_ctx* c) {
     for (DevBuf* b : {&c->xf32, &c->xq, &c->xd, &c->xs, &c->yf32, &c->work, &c->work2, &c->tab})
         if (b->p) (void)hipFree(b->p);
     for (char* p : c->retired) (void)hipFree(p);
-    for (DevBuf* b : {&c->hx, &c->hy})
+    for (DevBuf* b : {&c->hx, &c->hy, &c->htab})
         if (b->p) (void)hipHostFree(b->p);
+    if (c->htab_done) (void)hipEventDestroy(c->htab_done);
     for (auto& r : c->prof) {
         (void)hipEventDestroy(r.e0);
         (void)hipEventDestroy(r.e1);

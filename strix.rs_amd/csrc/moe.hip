@@ -542,11 +542,17 @@ struct TableBlob {
         if (n) std::memcpy(bytes.data() + off, p, n);
         return off;
     }
-    // pageable source: the copy has been staged when hipMemcpyAsync returns, the blob may go away
+    // Through the context's pinned staging buffer, so that the caller (and this blob) may go away while
+    // the copy is still queued; an event guards the buffer against the next call's tables.
     int upload(smx_ctx* c) {
         int rc = ensure(c, c->tab, bytes.size());
         if (rc != SMX_OK) return rc;
-        SMX_HIP(c, hipMemcpyAsync(c->tab.p, bytes.data(), bytes.size(), hipMemcpyHostToDevice, c->stream));
+        if (c->htab_done) SMX_HIP(c, hipEventSynchronize(c->htab_done));  // the previous copy out of htab has run
+        else SMX_HIP(c, hipEventCreateWithFlags(&c->htab_done, hipEventDisableTiming));
+        if ((rc = ensure_host(c, c->htab, bytes.size())) != SMX_OK) return rc;
+        std::memcpy(c->htab.p, bytes.data(), bytes.size());
+        SMX_HIP(c, hipMemcpyAsync(c->tab.p, c->htab.p, bytes.size(), hipMemcpyHostToDevice, c->stream));
+        SMX_HIP(c, hipEventRecord(c->htab_done, c->stream));
         return SMX_OK;
     }
 };

@@ -72,6 +72,8 @@ struct smx_ctx {
     smx::DevBuf work2;
     smx::DevBuf tab;    // small tables (ids, weights, tile tables)
     smx::DevBuf hx, hy; // pinned HOST staging of the host-pointer calls' activations and results
+    smx::DevBuf htab;   // pinned HOST staging of the small tables of enqueue-only calls
+    hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
 
     // tuning overrides (0 = automatic)
     int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
