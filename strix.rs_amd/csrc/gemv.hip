@@ -38,6 +38,13 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, in
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
+// Task-split form (one activation row): blockIdx.x of gridDim.x workgroups share a job's chunks.
+template <class Ops, int PRE, int LPR, int FQ, int NT>
+__global__ __launch_bounds__(NT) void gemv_tasks_kernel(const GemvJobs J, int nblk) {
+    const GemvJob& jb = J.job[blockIdx.y];
+    gemv_body_tasks<Ops, PRE, LPR, FQ>(jb.W, jb.X, jb.y, nblk, jb.N, blockIdx.x, gridDim.x);
+}
+
 namespace {
 
 // Row length from which silu / gelu producers run in their own launch (measured on 2560 <- 9728).
@@ -47,6 +54,7 @@ constexpr size_t kProducerSplitK = 4096;
 struct Geom {
     bool prod = false;  // an activation producer runs in the staging
     bool preq = false;  // the (single) activation row arrives quantised
+    bool tasks = false; // task-split form: (chunk, pass) items dealt to the waves of a workgroup
     int rpw, pre, ks, lpr, nt;
     unsigned grid;
     size_t lds;
@@ -74,6 +82,25 @@ int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk
     return launch_fq<Ops, MT, RPW, PRE, KS, LPR, MT == 1 ? 1 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
 }
 
+template <class Ops, int PRE, int LPR, int FQ>
+int launch_tasks_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
+    auto k = gemv_tasks_kernel<Ops, PRE, LPR, FQ, 1024>;
+    static size_t lds_set = 0;
+    int rc = set_dyn_lds(c, k, g.lds, &lds_set);
+    if (rc != SMX_OK) return rc;
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
+template <class Ops, int LPR>
+int launch_tasks(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
+    constexpr int PRE = sizeof(typename Ops::Regs) > 32 ? 3 : 4;
+    if (g.preq) return launch_tasks_fq<Ops, PRE, LPR, 0>(c, g, J, njobs, nblk);
+    if (g.prod) return launch_tasks_fq<Ops, PRE, LPR, 2>(c, g, J, njobs, nblk);
+    return launch_tasks_fq<Ops, PRE, LPR, 1>(c, g, J, njobs, nblk);
+}
+
 // The compiled variants (RPW, PRE, KS, LPR):
 //   whole-wave rows   (4,2,1,64) (2,2,1,64) (1,4,1,64) (1,2,2,64) (1,2,4,64)
 //   sub-wave rows     (2,2,1,32) (1,2,1,32) (2,2,1,16) (1,2,1,16)        [one activation row only]
@@ -82,6 +109,11 @@ int launch_variant(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
     // sub-wave rows: the pipeline is deep enough to put a whole short row set in flight before the
     // activation is staged (Q6_K units are three times as wide, so half the depth)
     constexpr bool kWide = sizeof(typename Ops::Regs) > 32;
+    if (MT == 1 && g.tasks) {
+        if (g.lpr == 16) return launch_tasks<Ops, 16>(c, g, J, njobs, nblk);
+        if (g.lpr == 32) return launch_tasks<Ops, 32>(c, g, J, njobs, nblk);
+        return launch_tasks<Ops, 64>(c, g, J, njobs, nblk);
+    }
     if (MT == 1 && g.lpr == 32) {
         if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
         return launch_one<Ops, 1, 1, kWide ? 2 : 4, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
@@ -183,6 +215,27 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
         int wpc = c->tune_gemv_wpc > 0 ? c->tune_gemv_wpc : 1;
         if (dump) wpc = 8;
         g.grid = (unsigned)std::min<size_t>(wgs, cus * wpc);
+    }
+    // Task-split form: rows of several passes where handing a wave whole chunks leaves waves idle or
+    // queues a second round of workgroups.  Taken when it cuts the longest wave's work by more than a
+    // quarter (measured: the gate/up pair 11.3 -> 9.4 us, Q8_0 2560 x 9728 10.2 -> 9.5 us; no gain where
+    // the two forms are within a pass or two of each other).
+    if (mt == 1 && !dump && c->tune_gemv_tasks != 1 && P >= 2) {
+        const size_t rs = 64 / g.lpr;
+        const size_t tchunks = (N + rs - 1) / rs, tasks = tchunks * P;
+        const size_t twgs = std::max<size_t>(1, std::min(cus, (tasks + 15) / 16));
+        const size_t wg_tasks = ((tchunks + twgs - 1) / twgs) * P;  // of the workgroup with the most chunks
+        const size_t part = (wg_tasks * rs * 4 + 15) & ~size_t(15);
+        const size_t new_max = (wg_tasks + 15) / 16;
+        size_t old_max;
+        if (g.ks > 1) old_max = ((g.grid + cus - 1) / cus) * ((P + g.ks - 1) / g.ks);
+        else old_max = ((chunks + (size_t)g.grid * 16 - 1) / ((size_t)g.grid * 16)) * P * g.rpw;
+        if (tokb + part <= 96 * 1024 && (c->tune_gemv_tasks == 2 || new_max * 4 < old_max * 3)) {
+            g.tasks = true;
+            g.nt = 1024;
+            g.grid = (unsigned)twgs;
+            g.lds = tokb + part;
+        }
     }
     return g;
 }

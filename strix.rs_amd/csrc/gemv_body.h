@@ -535,4 +535,77 @@ __device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* _
     SMX_STAMP_FLUSH();
 }
 
+// Task-split form for one activation row and few passes per wave.  A workgroup owns a contiguous range
+// of chunks (RS = 64/LPR rows each); every (chunk, pass) of the range is a task of its own, dealt round
+// robin to the workgroup's waves, so the waves of a workgroup carry equal work whatever the ratio of
+// chunks to waves (the persistent form gives a wave whole chunks: 2432 chunks of 5 passes over 4096
+// waves leave 40 % of them idle and the rest with 5 passes each).  A task's LPR-lane sum goes to LDS;
+// after a barrier the passes of a row are added in pass order and the row is written.
+template <class Ops, int PRE, int LPR, int FQ>
+__device__ __forceinline__ void gemv_body_tasks(const GemvW W, const GemvX X, float* __restrict__ y, int nblk, int N,
+                                                int wg, int n_wgs) {
+    extern __shared__ __align__(16) char smem[];
+    constexpr int RS = 64 / LPR;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int sub = lane & (LPR - 1), rsub = lane / LPR;
+    const int U = Ops::units_per_row(nblk);
+    const int P = (U + LPR - 1) / LPR;
+    const int nchunks = (N + RS - 1) / RS;
+    const int c0 = (int)((long long)nchunks * wg / n_wgs), c1 = (int)((long long)nchunks * (wg + 1) / n_wgs);
+    const int ntasks = (c1 - c0) * P;
+    const int tokb = Ops::tok_bytes(nblk);
+    float* part = (float*)(smem + tokb);  // [ntasks][RS]
+
+    typename Ops::Regs ring[PRE];
+    const int dq = nw / P, dr = nw % P;   // task index + nw = chunk + dq, pass + dr (with carry)
+    int l_i = wave, l_c = wave / P, l_p = wave % P;
+    auto issue = [&](int slot) {
+        const int u = min(l_p * LPR + sub, U - 1);
+        const size_t row = (size_t)min((c0 + l_c) * RS + rsub, N - 1);
+        Ops::load(ring[slot], W, row, nblk, u);
+        l_i += nw;
+        l_c += dq;
+        l_p += dr;
+        if (l_p >= P) {
+            l_p -= P;
+            l_c++;
+        }
+    };
+#pragma unroll
+    for (int k = 0; k < PRE; k++)
+        if (l_i < ntasks) issue(k);
+
+    if (FQ != 0) stage_token<Ops, FQ>(smem, nblk, X, 0, false);
+    else stage_prequant_all<Ops, 1>(smem, tokb, nblk, X, 1);
+    __syncthreads();
+
+    int c_i = wave, c_p = wave % P;
+    while (c_i < ntasks) {
+#pragma unroll
+        for (int k = 0; k < PRE; k++) {
+            if (c_i < ntasks) {
+                const int uu = c_p * LPR + sub;
+                const bool act = uu < U;
+                const int u = act ? uu : U - 1;
+                float acc[1] = {0.f};
+                compute_unit<1, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
+                if (l_i < ntasks) issue(k);
+                const float s = group_sum<LPR>(acc[0]);
+                if (sub == LPR - 1) part[c_i * RS + rsub] = s;
+                c_i += nw;
+                c_p += dr;
+                if (c_p >= P) c_p -= P;
+            }
+        }
+    }
+    __syncthreads();
+    for (int r = threadIdx.x; r < (c1 - c0) * RS; r += blockDim.x) {
+        const int c = r / RS, rs = r % RS;
+        float s = 0.f;
+        for (int p = 0; p < P; p++) s += part[(c * P + p) * RS + rs];
+        const int row = c0 * RS + r;
+        if (row < N) y[row] = s;
+    }
+}
+
 }  // namespace smx

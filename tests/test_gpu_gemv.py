@@ -60,6 +60,36 @@ def test_gemv_matches_q8_oracle(accel, orc, synth, relerr, ty, N, K):
     assert relerr(y, f32) <= 5e-2
 
 
+# shapes where the task-split form has something to split (several passes per row), incl. ragged row
+# counts, a scale range that does not start on a 16-byte boundary (odd blocks per row) and a weight
+# with fewer chunks than workgroups
+TASK_SHAPES = [(2, 130, 2560), (2, 9, 96 * 32), (2, 2500, 2560), (2, 3, 4128), (2, 1, 32 * 129),
+               (8, 130, 2560), (8, 37, 9728), (8, 5, 32 * 67), (14, 70, 3840), (14, 9, 4352)]
+
+
+@pytest.mark.parametrize("form", [1, 2])     # smx_tune("gemv_tasks"): 1 never, 2 wherever it fits
+@pytest.mark.parametrize("ty,N,K", TASK_SHAPES)
+def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K, form):
+    raw = synth.make_weight(ty, N, K, seed=13 * N + K)
+    x = synth.make_acts(1, K, seed=N + 7 * K)
+    _up(accel, ty, "t.form", raw, K, N)
+    accel.tune("gemv_tasks", form)
+    try:
+        y = accel.gemv("t.form", x, N)
+        # a group of two jobs with different row counts shares one launch geometry
+        raw2 = synth.make_weight(ty, N + 5, K, seed=17 * N + K)
+        _up(accel, ty, "t.form2", raw2, K, N + 5)
+        pair = accel.gemv_batch([("t.form", x), ("t.form2", x)], [N, N + 5])
+    finally:
+        accel.tune("gemv_tasks", 0)
+    ref = orc.matmul_q8_from_f32(ty, raw, K, N, x)[0]
+    assert relerr(y, ref) <= TOL
+    assert relerr(pair[0], ref) <= TOL
+    assert relerr(pair[1], orc.matmul_q8_from_f32(ty, raw2, K, N + 5, x)[0]) <= TOL
+    accel.evict("t.form")
+    accel.evict("t.form2")
+
+
 @pytest.mark.parametrize("ty", [2, 8])
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
 def test_gemv_rows_batched(accel, orc, synth, relerr, ty, m):
