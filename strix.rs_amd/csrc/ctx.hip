@@ -442,9 +442,9 @@ int smx_tune(smx_ctx* c, const char* knob, int value) {
     } else if (k == "gemv_wpc") {
         if (value > 32) return fail(c, SMX_ERR_ARG, "tune: gemv_wpc must be 0..32");
         c->tune_gemv_wpc = value;
-    } else if (k == "gemv_tasks") {
-        if (value > 2) return fail(c, SMX_ERR_ARG, "tune: gemv_tasks must be 0 (automatic), 1 (off) or 2 (wherever it fits)");
-        c->tune_gemv_tasks = value;
+    } else if (k == "gemv_flat") {
+        if (value > 1) return fail(c, SMX_ERR_ARG, "tune: gemv_flat must be 0 (automatic) or 1 (never)");
+        c->tune_gemv_flat = value;
     } else if (k == "gemm_splitk") {
         if (value > 16) return fail(c, SMX_ERR_ARG, "tune: gemm_splitk must be 0..16");
         c->tune_gemm_splitk = value;

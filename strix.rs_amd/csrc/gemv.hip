@@ -10,6 +10,7 @@
 //   * cross-lane (DPP) combination of lanes that share a block, wave-wide reduction at the end.
 // HBM-bound: algorithmic bytes per row are K/32 * {18, 34} (Q4_0, Q8_0) or K/256 * 210 (Q6_K).
 #include <algorithm>
+#include <type_traits>
 
 #include "gemv_body.h"
 #include "smx_internal.h"
@@ -38,11 +39,11 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, in
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
-// Task-split form (one activation row): blockIdx.x of gridDim.x workgroups share a job's chunks.
-template <class Ops, int PRE, int LPR, int FQ, int NT>
-__global__ __launch_bounds__(NT) void gemv_tasks_kernel(const GemvJobs J, int nblk) {
+// Flat form (one activation row, Q4_0 / Q8_0): blockIdx.x of gridDim.x workgroups share a job's rows.
+template <class Ops, int PRE, int GL, int FQ>
+__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, unsigned magic_u) {
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body_tasks<Ops, PRE, LPR, FQ>(jb.W, jb.X, jb.y, nblk, jb.N, blockIdx.x, gridDim.x);
+    gemv_body_flat<Ops, PRE, GL, FQ>(jb.W, jb.X, jb.y, nblk, jb.N, blockIdx.x, gridDim.x, magic_u);
 }
 
 namespace {
@@ -54,7 +55,8 @@ constexpr size_t kProducerSplitK = 4096;
 struct Geom {
     bool prod = false;  // an activation producer runs in the staging
     bool preq = false;  // the (single) activation row arrives quantised
-    bool tasks = false; // task-split form: (chunk, pass) items dealt to the waves of a workgroup
+    int flat = 0;       // flat form: lanes per group (16 or 8), 0 = not used
+    int flat_pre = 0;   // its loads per round (3 or 4)
     int rpw, pre, ks, lpr, nt;
     unsigned grid;
     size_t lds;
@@ -82,23 +84,32 @@ int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk
     return launch_fq<Ops, MT, RPW, PRE, KS, LPR, MT == 1 ? 1 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
 }
 
-template <class Ops, int PRE, int LPR, int FQ>
-int launch_tasks_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
-    auto k = gemv_tasks_kernel<Ops, PRE, LPR, FQ, 1024>;
+template <class Ops, int PRE, int GL, int FQ>
+int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
+    auto k = gemv_flat_kernel<Ops, PRE, GL, FQ>;
     static size_t lds_set = 0;
     int rc = set_dyn_lds(c, k, g.lds, &lds_set);
     if (rc != SMX_OK) return rc;
-    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk);
+    const unsigned units = (unsigned)nblk * (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u);   // units per row
+    const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);   // floor(f * magic / 2^32) = f / units for f < 2^16
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, magic);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
 
-template <class Ops, int LPR>
-int launch_tasks(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
-    constexpr int PRE = sizeof(typename Ops::Regs) > 32 ? 3 : 4;
-    if (g.preq) return launch_tasks_fq<Ops, PRE, LPR, 0>(c, g, J, njobs, nblk);
-    if (g.prod) return launch_tasks_fq<Ops, PRE, LPR, 2>(c, g, J, njobs, nblk);
-    return launch_tasks_fq<Ops, PRE, LPR, 1>(c, g, J, njobs, nblk);
+template <class Ops>
+int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
+    if constexpr (std::is_same<Ops, OpsQ4_0>::value || std::is_same<Ops, OpsQ8_0>::value) {
+#define SMX_FLAT(PRE, GL)                                                                         \
+    if (g.flat_pre == PRE && g.flat == GL) {                                                      \
+        if (g.preq) return launch_flat_fq<Ops, PRE, GL, 0>(c, g, J, njobs, nblk);                 \
+        if (g.prod) return launch_flat_fq<Ops, PRE, GL, 2>(c, g, J, njobs, nblk);                 \
+        return launch_flat_fq<Ops, PRE, GL, 1>(c, g, J, njobs, nblk);                             \
+    }
+        SMX_FLAT(3, 16) SMX_FLAT(4, 16) SMX_FLAT(3, 8) SMX_FLAT(4, 8)
+#undef SMX_FLAT
+    }
+    return fail(c, SMX_ERR_ARG, "gemv: no flat variant for this geometry");
 }
 
 // The compiled variants (RPW, PRE, KS, LPR):
@@ -109,11 +120,7 @@ int launch_variant(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
     // sub-wave rows: the pipeline is deep enough to put a whole short row set in flight before the
     // activation is staged (Q6_K units are three times as wide, so half the depth)
     constexpr bool kWide = sizeof(typename Ops::Regs) > 32;
-    if (MT == 1 && g.tasks) {
-        if (g.lpr == 16) return launch_tasks<Ops, 16>(c, g, J, njobs, nblk);
-        if (g.lpr == 32) return launch_tasks<Ops, 32>(c, g, J, njobs, nblk);
-        return launch_tasks<Ops, 64>(c, g, J, njobs, nblk);
-    }
+    if (MT == 1 && g.flat) return launch_flat<Ops>(c, g, J, njobs, nblk);
     if (MT == 1 && g.lpr == 32) {
         if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
         return launch_one<Ops, 1, 1, kWide ? 2 : 4, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
@@ -216,25 +223,20 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
         if (dump) wpc = 8;
         g.grid = (unsigned)std::min<size_t>(wgs, cus * wpc);
     }
-    // Task-split form: rows of several passes where handing a wave whole chunks leaves waves idle or
-    // queues a second round of workgroups.  Taken when it cuts the longest wave's work by more than a
-    // quarter (measured: the gate/up pair 11.3 -> 9.4 us, Q8_0 2560 x 9728 10.2 -> 9.5 us; no gain where
-    // the two forms are within a pass or two of each other).
-    if (mt == 1 && !dump && c->tune_gemv_tasks != 1 && P >= 2) {
-        const size_t rs = 64 / g.lpr;
-        const size_t tchunks = (N + rs - 1) / rs, tasks = tchunks * P;
-        const size_t twgs = std::max<size_t>(1, std::min(cus, (tasks + 15) / 16));
-        const size_t wg_tasks = ((tchunks + twgs - 1) / twgs) * P;  // of the workgroup with the most chunks
-        const size_t part = (wg_tasks * rs * 4 + 15) & ~size_t(15);
-        const size_t new_max = (wg_tasks + 15) / 16;
-        size_t old_max;
-        if (g.ks > 1) old_max = ((g.grid + cus - 1) / cus) * ((P + g.ks - 1) / g.ks);
-        else old_max = ((chunks + (size_t)g.grid * 16 - 1) / ((size_t)g.grid * 16)) * P * g.rpw;
-        if (tokb + part <= 96 * 1024 && (c->tune_gemv_tasks == 2 || new_max * 4 < old_max * 3)) {
-            g.tasks = true;
+    // Flat form: one activation row, Q4_0 / Q8_0, rows of a whole number of 16- or 8-unit groups, at
+    // most 8 loads per wave (small and medium GEMVs, where start-up latency decides).
+    if (mt == 1 && !dump && c->tune_gemv_flat != 1 && type != kQ6_K && (units % 8) == 0 &&
+        nblk * 8 <= 4096) {  // rows of up to 16384 elements: the row is held in registers while the weights are requested
+        const size_t fwgs = std::max<size_t>(1, std::min(cus, N));
+        const size_t rows = (N + fwgs - 1) / fwgs;                 // of the workgroup with the most rows
+        const size_t loads = (rows * units + 63) / 64, per_wave = (loads + 15) / 16;
+        if (per_wave <= 8 && rows * units < 65536) {
+            g.flat = (units % 16) == 0 ? 16 : 8;
+            const size_t waste3 = (per_wave + 2) / 3 * 3 - per_wave, waste4 = (per_wave + 3) / 4 * 4 - per_wave;
+            g.flat_pre = waste3 < waste4 ? 3 : 4;
             g.nt = 1024;
-            g.grid = (unsigned)twgs;
-            g.lds = tokb + part;
+            g.grid = (unsigned)fwgs;
+            g.lds = tokb + rows * units / g.flat * 4;
         }
     }
     return g;

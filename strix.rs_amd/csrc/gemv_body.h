@@ -113,6 +113,11 @@ struct OpsQ4_0 {
         r.q = w.quants[row * nblk + u];
         r.s = w.scales[row * nblk + u];
     }
+    // unit f of the flat [row][unit] sequence (rows are contiguous)
+    static __device__ __forceinline__ void load_flat(Regs& r, const GemvW& w, size_t f) {
+        r.q = w.quants[f];
+        r.s = w.scales[f];
+    }
 };
 
 struct OpsQ8_0 {
@@ -131,6 +136,10 @@ struct OpsQ8_0 {
     static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nblk, int u) {
         r.q = w.quants[row * nblk * 2 + u];
         r.s = w.scales[row * nblk + (u >> 1)];
+    }
+    static __device__ __forceinline__ void load_flat(Regs& r, const GemvW& w, size_t f) {
+        r.q = w.quants[f];
+        r.s = w.scales[f >> 1];   // two units per block, an even number of units per row
     }
 };
 
@@ -300,10 +309,63 @@ __device__ __forceinline__ void compute_unit(OpsQ6_K, const OpsQ6_K::Regs& r, co
     }
 }
 
-// Stage one activation row into LDS.  8 lanes per 32-block, one float4 / one packed dword each;
-// reductions inside the 8 lanes go over DPP.  With the quantiser fused, an activation producer
-// (X.prod: rmsnorm(x)*x2, silu(x)*x2, gelu_tanh(x)*x2; kernels.rs:101-226) runs on the values first.
+// One item of an activation row on its way into LDS: 8 lanes share a 32-block, each holds one float4
+// (fused quantiser) or one packed dword (pre-quantised row); reductions inside the 8 lanes go over DPP.
+// With the quantiser fused, an activation producer (X.prod: rmsnorm(x)*x2, silu(x)*x2, gelu_tanh(x)*x2;
+// kernels.rs:101-226) runs on the values first.  Whole 8-lane groups are live or not together.
 // FQ: 0 the row is pre-quantised, 1 fp32 row quantised here, 2 the same behind an activation producer.
+template <class Ops, int FQ>
+__device__ __forceinline__ void stage_item(char* tok, int nblk, const GemvX& X, int t, int i, bool live, bool zero,
+                                           float4 w, float4 g, int packed, float rs) {
+    const int nb32 = Ops::nb32(nblk);
+    const int blk = i >> 3, sub = i & 7;
+    int s_lo = 0, s_hi = 0;
+    float d = 0.f;
+    if (FQ != 0) {
+        if (FQ == 2 && X.prod != SMX_ACT_NONE) {
+#pragma clang fp contract(off)
+            if (X.prod == SMX_ACT_RMSNORM) {
+                w.x = (w.x * rs) * g.x; w.y = (w.y * rs) * g.y; w.z = (w.z * rs) * g.z; w.w = (w.w * rs) * g.w;
+            } else if (X.prod == SMX_ACT_SILU_MUL) {
+                w.x = det_silu(w.x) * g.x; w.y = det_silu(w.y) * g.y; w.z = det_silu(w.z) * g.z; w.w = det_silu(w.w) * g.w;
+            } else {
+                w.x = det_gelu_tanh(w.x) * g.x; w.y = det_gelu_tanh(w.y) * g.y;
+                w.z = det_gelu_tanh(w.z) * g.z; w.w = det_gelu_tanh(w.w) * g.w;
+            }
+        }
+        float a = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
+        a = fmaxf(a, dpp_f<0xB1>(a));
+        a = fmaxf(a, dpp_f<0x4E>(a));
+        a = fmaxf(a, dpp_f<0x141>(a));
+        d = a / 127.f;
+        const float inv = d > 0.f ? 1.f / d : 0.f;
+        const int q0 = max(-127, min(127, (int)rintf(w.x * inv)));
+        const int q1 = max(-127, min(127, (int)rintf(w.y * inv)));
+        const int q2 = max(-127, min(127, (int)rintf(w.z * inv)));
+        const int q3 = max(-127, min(127, (int)rintf(w.w * inv)));
+        packed = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
+        if (Ops::kNeedsSums) {
+            int s = q0 + q1 + q2 + q3;
+            s += dpp_i<0xB1>(s);
+            s += dpp_i<0x4E>(s);          // sum over this lane's 16-element half
+            s_lo = s;
+            s_hi = dpp_i<0x141>(s);       // the other half's sum (valid in lanes 0..3 of the group)
+        }
+    } else if (live && !zero && sub == 0) {
+        d = X.xd[(size_t)t * nb32 + blk];
+        if (Ops::kNeedsSums) {
+            const int sp = X.xs[(size_t)t * nb32 + blk];
+            s_lo = (int)(short)(sp & 0xffff);
+            s_hi = sp >> 16;
+        }
+    }
+    if (live) {
+        *Ops::xq_dword(tok, nblk, blk, sub) = packed;
+        if (sub == 0) Ops::put_scale(tok, nblk, blk, d, s_lo, s_hi);
+    }
+}
+
+// Stage one activation row into LDS (stage_item over the row, two items per thread in flight).
 template <class Ops, int FQ>
 __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X, int t, bool zero) {
     const int nb32 = Ops::nb32(nblk);
@@ -320,9 +382,9 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
             const int i = i0 + j * blockDim.x;
             const bool live = i < items && !zero;
             v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            v2[j] = make_float4(1.f, 1.f, 1.f, 1.f);
             pk[j] = 0;
             if (FUSEQ) {
-                v2[j] = make_float4(1.f, 1.f, 1.f, 1.f);
                 if (live) {
                     v[j] = ((const float4*)(X.x + (size_t)t * nb32 * 32))[i];
                     if (FQ == 2 && X.x2) v2[j] = ((const float4*)(X.x2 + (size_t)t * nb32 * 32))[i];
@@ -334,55 +396,7 @@ __device__ __forceinline__ void stage_token(char* tok, int nblk, const GemvX& X,
 #pragma unroll
         for (int j = 0; j < SB; j++) {
             const int i = i0 + j * blockDim.x;
-            // whole 8-lane groups are live or not together (items is a multiple of 8)
-            const bool live = i < items;
-            const int blk = i >> 3, sub = i & 7;
-            int packed = pk[j], s_lo = 0, s_hi = 0;
-            float d = 0.f;
-            if (FUSEQ) {
-                float4 w = v[j];
-                if (FQ == 2 && X.prod != SMX_ACT_NONE) {
-#pragma clang fp contract(off)
-                    const float4 g = v2[j];
-                    if (X.prod == SMX_ACT_RMSNORM) {
-                        w.x = (w.x * rs) * g.x; w.y = (w.y * rs) * g.y; w.z = (w.z * rs) * g.z; w.w = (w.w * rs) * g.w;
-                    } else if (X.prod == SMX_ACT_SILU_MUL) {
-                        w.x = det_silu(w.x) * g.x; w.y = det_silu(w.y) * g.y; w.z = det_silu(w.z) * g.z; w.w = det_silu(w.w) * g.w;
-                    } else {
-                        w.x = det_gelu_tanh(w.x) * g.x; w.y = det_gelu_tanh(w.y) * g.y;
-                        w.z = det_gelu_tanh(w.z) * g.z; w.w = det_gelu_tanh(w.w) * g.w;
-                    }
-                }
-                float a = fmaxf(fmaxf(fabsf(w.x), fabsf(w.y)), fmaxf(fabsf(w.z), fabsf(w.w)));
-                a = fmaxf(a, dpp_f<0xB1>(a));
-                a = fmaxf(a, dpp_f<0x4E>(a));
-                a = fmaxf(a, dpp_f<0x141>(a));
-                d = a / 127.f;
-                const float inv = d > 0.f ? 1.f / d : 0.f;
-                const int q0 = max(-127, min(127, (int)rintf(w.x * inv)));
-                const int q1 = max(-127, min(127, (int)rintf(w.y * inv)));
-                const int q2 = max(-127, min(127, (int)rintf(w.z * inv)));
-                const int q3 = max(-127, min(127, (int)rintf(w.w * inv)));
-                packed = (q0 & 0xff) | ((q1 & 0xff) << 8) | ((q2 & 0xff) << 16) | ((q3 & 0xff) << 24);
-                if (Ops::kNeedsSums) {
-                    int s = q0 + q1 + q2 + q3;
-                    s += dpp_i<0xB1>(s);
-                    s += dpp_i<0x4E>(s);          // sum over this lane's 16-element half
-                    s_lo = s;
-                    s_hi = dpp_i<0x141>(s);       // the other half's sum (valid in lanes 0..3 of the group)
-                }
-            } else if (live && !zero && sub == 0) {
-                d = X.xd[(size_t)t * nb32 + blk];
-                if (Ops::kNeedsSums) {
-                    const int sp = X.xs[(size_t)t * nb32 + blk];
-                    s_lo = (int)(short)(sp & 0xffff);
-                    s_hi = sp >> 16;
-                }
-            }
-            if (live) {
-                *Ops::xq_dword(tok, nblk, blk, sub) = packed;
-                if (sub == 0) Ops::put_scale(tok, nblk, blk, d, s_lo, s_hi);
-            }
+            stage_item<Ops, FQ>(tok, nblk, X, t, i, i < items, zero, v[j], v2[j], pk[j], rs);
         }
     }
 }
@@ -535,76 +549,167 @@ __device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* _
     SMX_STAMP_FLUSH();
 }
 
-// Task-split form for one activation row and few passes per wave.  A workgroup owns a contiguous range
-// of chunks (RS = 64/LPR rows each); every (chunk, pass) of the range is a task of its own, dealt round
-// robin to the workgroup's waves, so the waves of a workgroup carry equal work whatever the ratio of
-// chunks to waves (the persistent form gives a wave whole chunks: 2432 chunks of 5 passes over 4096
-// waves leave 40 % of them idle and the rest with 5 passes each).  A task's LPR-lane sum goes to LDS;
-// after a barrier the passes of a row are added in pass order and the row is written.
-template <class Ops, int PRE, int LPR, int FQ>
-__device__ __forceinline__ void gemv_body_tasks(const GemvW W, const GemvX X, float* __restrict__ y, int nblk, int N,
-                                                int wg, int n_wgs) {
-    extern __shared__ __align__(16) char smem[];
-    constexpr int RS = 64 / LPR;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int sub = lane & (LPR - 1), rsub = lane / LPR;
-    const int U = Ops::units_per_row(nblk);
-    const int P = (U + LPR - 1) / LPR;
-    const int nchunks = (N + RS - 1) / RS;
-    const int c0 = (int)((long long)nchunks * wg / n_wgs), c1 = (int)((long long)nchunks * (wg + 1) / n_wgs);
-    const int ntasks = (c1 - c0) * P;
-    const int tokb = Ops::tok_bytes(nblk);
-    float* part = (float*)(smem + tokb);  // [ntasks][RS]
+// Sum over groups of 8 adjacent lanes (all lanes of a group end up with the total).
+__device__ __forceinline__ float group_sum8(float v) {
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x141>(v);
+    return v;
+}
 
-    typename Ops::Regs ring[PRE];
-    const int dq = nw / P, dr = nw % P;   // task index + nw = chunk + dq, pass + dr (with carry)
-    int l_i = wave, l_c = wave / P, l_p = wave % P;
-    auto issue = [&](int slot) {
-        const int u = min(l_p * LPR + sub, U - 1);
-        const size_t row = (size_t)min((c0 + l_c) * RS + rsub, N - 1);
-        Ops::load(ring[slot], W, row, nblk, u);
-        l_i += nw;
-        l_c += dq;
-        l_p += dr;
-        if (l_p >= P) {
-            l_p -= P;
-            l_c++;
-        }
-    };
+// The activation row of the flat form: every global load is requested up front (before the weight
+// stream, so that waiting for the row does not wait for the weights: a wave's loads complete in
+// order), the values are quantised and written to LDS later.  Thread t holds items t, t + 1024, ...
+// Rows of up to 16384 elements (fp32 row) or 32768 (pre-quantised row).
+template <class Ops, int FQ>
+struct FlatX {
+    static constexpr int XI = FQ == 0 ? 2 : 4;
+    float4 v[XI], v2[XI];
+    uint4 pk[XI];
+    float d[XI];
+    int sp[XI];
+
+    __device__ __forceinline__ void request(const GemvX& X, int nblk) {
+        const int nb32 = Ops::nb32(nblk);
+        const int items = FQ == 0 ? nb32 * 2 : nb32 * 8;
 #pragma unroll
-    for (int k = 0; k < PRE; k++)
-        if (l_i < ntasks) issue(k);
-
-    if (FQ != 0) stage_token<Ops, FQ>(smem, nblk, X, 0, false);
-    else stage_prequant_all<Ops, 1>(smem, tokb, nblk, X, 1);
-    __syncthreads();
-
-    int c_i = wave, c_p = wave % P;
-    while (c_i < ntasks) {
-#pragma unroll
-        for (int k = 0; k < PRE; k++) {
-            if (c_i < ntasks) {
-                const int uu = c_p * LPR + sub;
-                const bool act = uu < U;
-                const int u = act ? uu : U - 1;
-                float acc[1] = {0.f};
-                compute_unit<1, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
-                if (l_i < ntasks) issue(k);
-                const float s = group_sum<LPR>(acc[0]);
-                if (sub == LPR - 1) part[c_i * RS + rsub] = s;
-                c_i += nw;
-                c_p += dr;
-                if (c_p >= P) c_p -= P;
+        for (int j = 0; j < XI; j++) {
+            const int i = threadIdx.x + j * 1024;
+            v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            v2[j] = make_float4(1.f, 1.f, 1.f, 1.f);
+            pk[j] = make_uint4(0, 0, 0, 0);
+            d[j] = 0.f;
+            sp[j] = 0;
+            if (i < items) {
+                if (FQ == 0) {
+                    pk[j] = ((const uint4*)X.xq)[i];
+                    if ((i & 1) == 0) {
+                        d[j] = X.xd[i >> 1];
+                        if (Ops::kNeedsSums) sp[j] = X.xs[i >> 1];
+                    }
+                } else {
+                    v[j] = ((const float4*)X.x)[i];
+                    if (FQ == 2 && X.x2) v2[j] = ((const float4*)X.x2)[i];
+                }
             }
         }
     }
+
+    // `tok`: the row's LDS area (also the scratch of the rmsnorm reduction); every thread of the
+    // 1024-thread workgroup calls this.
+    __device__ __forceinline__ void store(char* tok, int nblk, const GemvX& X) {
+        const int nb32 = Ops::nb32(nblk);
+        if (FQ == 0) {
+#pragma unroll
+            for (int j = 0; j < XI; j++) {
+                const int i = threadIdx.x + j * 1024;
+                if (i < nb32 * 2) {
+                    *(uint4*)Ops::xq_dword(tok, nblk, i >> 1, (i & 1) * 4) = pk[j];
+                    if ((i & 1) == 0) Ops::put_scale(tok, nblk, i >> 1, d[j], (int)(short)(sp[j] & 0xffff), sp[j] >> 16);
+                }
+            }
+            return;
+        }
+        const int items = nb32 * 8;
+        float rs = 1.f;
+        if (FQ == 2 && X.prod == SMX_ACT_RMSNORM) {
+            // the reduction of rms_scale over the values already in registers (same elements per thread, same order)
+#pragma clang fp contract(off)
+            double ss = 0.0;
+#pragma unroll
+            for (int j = 0; j < XI; j++) {
+                if ((int)threadIdx.x + j * 1024 < items) {
+                    ss += (double)v[j].x * (double)v[j].x;
+                    ss += (double)v[j].y * (double)v[j].y;
+                    ss += (double)v[j].z * (double)v[j].z;
+                    ss += (double)v[j].w * (double)v[j].w;
+                }
+            }
+            for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
+            double* red = (double*)tok;
+            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+            __syncthreads();
+            double tot = 0.0;
+            for (int w = 0; w < 16; w++) tot += red[w];
+            __syncthreads();
+            rs = (float)(1.0 / sqrt(tot / (double)(nb32 * 32) + (double)X.eps));
+        }
+#pragma unroll
+        for (int j = 0; j < XI; j++) {
+            const int i = threadIdx.x + j * 1024;
+            // whole waves are live or not together (items is a multiple of 8, i of a wave spans 64)
+            if ((i & ~63) < items) stage_item<Ops, FQ>(tok, nblk, X, 0, i, i < items, false, v[j], v2[j], 0, rs);
+        }
+    }
+};
+
+// Flat form for one activation row and rows that are a whole number of GL-lane groups (GL = 16 or 8
+// units).  Rows are contiguous in the planar layout, so the units of a workgroup's rows [r0, r1) are
+// one flat sequence: a wave load covers 64 consecutive units of it (1 KB of quants, whatever the row
+// length), wave w takes loads w, w + 16, ...  Every GL-lane group lies inside one row; its sum goes
+// to LDS, and after a barrier the groups of a row are added in ascending order.  All waves of a
+// workgroup carry the same number of loads, issued without conditions (lanes past the end re-read the
+// last unit) so that the wait for ring slot k is exactly "all but the loads issued after it" instead
+// of "all loads".  A round requests PRE loads and consumes them; the activation is staged during the
+// first round, after its weight loads are out.
+template <class Ops, int PRE, int GL, int FQ>
+__device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, float* __restrict__ y, int nblk, int N,
+                                               int wg, int n_wgs, unsigned magic_u) {
+    extern __shared__ __align__(16) char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int U = Ops::units_per_row(nblk);
+    // rows split evenly: the first N % n_wgs workgroups take one row more
+    const unsigned rbase = (unsigned)N / (unsigned)n_wgs, rrem = (unsigned)N - rbase * (unsigned)n_wgs;
+    const int r0 = wg * (int)rbase + min(wg, (int)rrem), r1 = r0 + (int)rbase + (wg < (int)rrem ? 1 : 0);
+    const int nunits = (r1 - r0) * U;          // < 2^16 (launcher)
+    const int nloads = (nunits + 63) >> 6;
+    const int tokb = Ops::tok_bytes(nblk);
+    float* part = (float*)(smem + tokb);       // [nunits / GL]
+    const size_t f_base = (size_t)r0 * U;
+
+    FlatX<Ops, FQ> xs;
+    xs.request(X, nblk);
+
+    typename Ops::Regs ring[PRE];
+    int l_t = wave, c_t = wave;
+    auto request = [&]() {
+#pragma unroll
+        for (int k = 0; k < PRE; k++) {
+            const int fl = min(l_t * 64 + lane, max(nunits - 1, 0));
+            Ops::load_flat(ring[k], W, f_base + fl);
+            l_t += 16;
+        }
+    };
+    auto consume = [&]() {
+#pragma unroll
+        for (int k = 0; k < PRE; k++) {
+            if (c_t < nloads) {   // wave-uniform
+                const int fl = c_t * 64 + lane;
+                const bool act = fl < nunits;
+                const int flc = act ? fl : nunits - 1;
+                const int u = flc - (int)__umulhi((unsigned)flc, magic_u) * U;   // flc mod U
+                float acc[1] = {0.f};
+                compute_unit<1, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
+                const float s = GL == 8 ? group_sum8(acc[0]) : group_sum<16>(acc[0]);
+                if (act && (lane & (GL - 1)) == GL - 1) part[fl / GL] = s;
+            }
+            c_t += 16;
+        }
+    };
+    request();
+    xs.store(smem, nblk, X);
     __syncthreads();
-    for (int r = threadIdx.x; r < (c1 - c0) * RS; r += blockDim.x) {
-        const int c = r / RS, rs = r % RS;
+    consume();
+    while (c_t < nloads) {
+        request();
+        consume();
+    }
+    __syncthreads();
+    const int G = U / GL;
+    for (int r = threadIdx.x; r < r1 - r0; r += blockDim.x) {
         float s = 0.f;
-        for (int p = 0; p < P; p++) s += part[(c * P + p) * RS + rs];
-        const int row = c0 * RS + r;
-        if (row < N) y[row] = s;
+        for (int j = 0; j < G; j++) s += part[r * G + j];
+        y[r0 + r] = s;
     }
 }
 

@@ -76,7 +76,7 @@ struct smx_ctx {
     hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
 
     // tuning overrides (0 = automatic)
-    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemv_tasks = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemv_flat = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
 
     bool capturing = false;  // between smx_graph_begin and smx_graph_end
     // A captured graph holds the addresses of the scratch buffers its kernels used.  While any graph

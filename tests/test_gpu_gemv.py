@@ -60,20 +60,22 @@ def test_gemv_matches_q8_oracle(accel, orc, synth, relerr, ty, N, K):
     assert relerr(y, f32) <= 5e-2
 
 
-# shapes where the task-split form has something to split (several passes per row), incl. ragged row
-# counts, a scale range that does not start on a 16-byte boundary (odd blocks per row) and a weight
-# with fewer chunks than workgroups
-TASK_SHAPES = [(2, 130, 2560), (2, 9, 96 * 32), (2, 2500, 2560), (2, 3, 4128), (2, 1, 32 * 129),
-               (8, 130, 2560), (8, 37, 9728), (8, 5, 32 * 67), (14, 70, 3840), (14, 9, 4352)]
+# Small single-row GEMVs have two forms: rows dealt to waves (any shape) and the flat form (rows that are
+# a whole number of 8- or 16-unit groups).  Shapes on both sides of every condition: group size 16 and 8,
+# ragged row counts, fewer rows than workgroups, one and several rounds of loads, rows too long or too
+# odd for the flat form.
+FORM_SHAPES = [(2, 130, 2560), (2, 9, 96 * 32), (2, 2500, 2560), (2, 3, 4096 + 256), (2, 1, 512), (2, 300, 256),
+               (2, 700, 8192), (2, 40, 16384), (2, 24, 16384 + 512), (2, 50, 32 * 129),
+               (8, 130, 2560), (8, 37, 9728), (8, 5, 32 * 68), (8, 1000, 1024), (8, 77, 128), (8, 60, 32 * 67)]
 
 
-@pytest.mark.parametrize("form", [1, 2])     # smx_tune("gemv_tasks"): 1 never, 2 wherever it fits
-@pytest.mark.parametrize("ty,N,K", TASK_SHAPES)
+@pytest.mark.parametrize("form", [0, 1])     # smx_tune("gemv_flat"): 0 automatic, 1 never
+@pytest.mark.parametrize("ty,N,K", FORM_SHAPES)
 def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K, form):
     raw = synth.make_weight(ty, N, K, seed=13 * N + K)
     x = synth.make_acts(1, K, seed=N + 7 * K)
     _up(accel, ty, "t.form", raw, K, N)
-    accel.tune("gemv_tasks", form)
+    accel.tune("gemv_flat", form)
     try:
         y = accel.gemv("t.form", x, N)
         # a group of two jobs with different row counts shares one launch geometry
@@ -81,7 +83,7 @@ def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K, form)
         _up(accel, ty, "t.form2", raw2, K, N + 5)
         pair = accel.gemv_batch([("t.form", x), ("t.form2", x)], [N, N + 5])
     finally:
-        accel.tune("gemv_tasks", 0)
+        accel.tune("gemv_flat", 0)
     ref = orc.matmul_q8_from_f32(ty, raw, K, N, x)[0]
     assert relerr(y, ref) <= TOL
     assert relerr(pair[0], ref) <= TOL
