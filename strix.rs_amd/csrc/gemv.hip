@@ -39,7 +39,7 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, in
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
-// Flat form (one activation row, Q4_0 / Q8_0): blockIdx.x of gridDim.x workgroups share a job's rows.
+// Flat form (one activation row): blockIdx.x of gridDim.x workgroups share a job's rows.
 template <class Ops, int PRE, int GL, int FQ>
 __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, unsigned magic_u) {
     const GemvJob& jb = J.job[blockIdx.y];
@@ -56,7 +56,7 @@ struct Geom {
     bool prod = false;  // an activation producer runs in the staging
     bool preq = false;  // the (single) activation row arrives quantised
     int flat = 0;       // flat form: lanes per group (16 or 8), 0 = not used
-    int flat_pre = 0;   // its loads per round (3 or 4)
+    int flat_pre = 0;   // its loads per round
     int rpw, pre, ks, lpr, nt;
     unsigned grid;
     size_t lds;
@@ -90,7 +90,7 @@ int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
     static size_t lds_set = 0;
     int rc = set_dyn_lds(c, k, g.lds, &lds_set);
     if (rc != SMX_OK) return rc;
-    const unsigned units = (unsigned)nblk * (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u);   // units per row
+    const unsigned units = (unsigned)nblk * (std::is_same<Ops, OpsQ6_K>::value ? 4u : (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u));   // units per row
     const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);   // floor(f * magic / 2^32) = f / units for f < 2^16
     hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, magic);
     SMX_HIP(c, hipGetLastError());
@@ -106,9 +106,11 @@ int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nbl
         if (g.prod) return launch_flat_fq<Ops, PRE, GL, 2>(c, g, J, njobs, nblk);                 \
         return launch_flat_fq<Ops, PRE, GL, 1>(c, g, J, njobs, nblk);                             \
     }
-        SMX_FLAT(3, 16) SMX_FLAT(4, 16) SMX_FLAT(3, 8) SMX_FLAT(4, 8)
-#undef SMX_FLAT
+        SMX_FLAT(3, 16) SMX_FLAT(3, 8)
+    } else if constexpr (std::is_same<Ops, OpsQ6_K>::value) {
+        SMX_FLAT(1, 16) SMX_FLAT(1, 8) SMX_FLAT(1, 4)
     }
+#undef SMX_FLAT
     return fail(c, SMX_ERR_ARG, "gemv: no flat variant for this geometry");
 }
 
@@ -223,17 +225,19 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
         if (dump) wpc = 8;
         g.grid = (unsigned)std::min<size_t>(wgs, cus * wpc);
     }
-    // Flat form: one activation row, Q4_0 / Q8_0, rows of a whole number of 16- or 8-unit groups, at
-    // most 8 loads per wave (small and medium GEMVs, where start-up latency decides).
-    if (mt == 1 && !dump && c->tune_gemv_flat != 1 && type != kQ6_K && (units % 8) == 0 &&
-        nblk * 8 <= 4096) {  // rows of up to 16384 elements: the row is held in registers while the weights are requested
+    // Flat form: one activation row of up to 16384 elements, rows of a whole number of unit groups, at
+    // most 32 loads per wave (small and medium GEMVs, where start-up latency decides; measured up to 24).
+    if (mt == 1 && !dump && c->tune_gemv_flat != 1 && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
+        nblk * (type == kQ6_K ? 256 : 32) <= 16384) {  // the row is held in registers while the weights are requested
         const size_t fwgs = std::max<size_t>(1, std::min(cus, N));
         const size_t rows = (N + fwgs - 1) / fwgs;                 // of the workgroup with the most rows
         const size_t loads = (rows * units + 63) / 64, per_wave = (loads + 15) / 16;
-        if (per_wave <= 8 && rows * units < 65536) {
-            g.flat = (units % 16) == 0 ? 16 : 8;
-            const size_t waste3 = (per_wave + 2) / 3 * 3 - per_wave, waste4 = (per_wave + 3) / 4 * 4 - per_wave;
-            g.flat_pre = waste3 < waste4 ? 3 : 4;
+        const size_t lim = c->tune_gemv_flat >= 2 ? (size_t)c->tune_gemv_flat : 32;
+        if (per_wave <= lim && rows * units < 65536) {
+            g.flat = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : 4);
+            // loads requested per round, measured: Q4_0 pair 8.2 / 8.0 / 7.7 / 8.1 / 8.9 us with 1 / 2 / 3 / 4 / 6,
+            // Q6_K 15360 x 3840 (five load instructions per unit) 11.4 / 12.5 / 14.1 / 14.8 us with 1 / 2 / 3 / 4
+            g.flat_pre = type == kQ6_K ? 1 : 3;
             g.nt = 1024;
             g.grid = (unsigned)fwgs;
             g.lds = tokb + rows * units / g.flat * 4;

@@ -178,6 +178,15 @@ struct OpsQ6_K {
         r.sc = w.sc[sb0 * 2 + (u >> 1)];
         r.d = w.scales[sb0 + (u >> 2)];
     }
+    // unit f of the flat [row][unit] sequence: four units per superblock, superblocks contiguous
+    static __device__ __forceinline__ void load_flat(Regs& r, const GemvW& w, size_t f) {
+        const size_t q = (f >> 2) * 8 + ((f & 3) >> 1) * 4 + (f & 1);
+        r.a = w.quants[q];
+        r.b = w.quants[q + 2];
+        r.h = w.qh[f];
+        r.sc = w.sc[f >> 1];
+        r.d = w.scales[f >> 2];
+    }
 };
 
 // Q4_0: whole-block i32 = sum(nibble*xq) - 8*sum(xq)  (kernels.rs:241-250), then (dw*dx)*float(isum)
@@ -549,11 +558,13 @@ __device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* _
     SMX_STAMP_FLUSH();
 }
 
-// Sum over groups of 8 adjacent lanes (all lanes of a group end up with the total).
-__device__ __forceinline__ float group_sum8(float v) {
+// Sum over groups of GL = 4, 8 or 16 adjacent lanes (all lanes of a group end up with the total).
+template <int GL>
+__device__ __forceinline__ float small_group_sum(float v) {
     v += dpp_f<0xB1>(v);
     v += dpp_f<0x4E>(v);
-    v += dpp_f<0x141>(v);
+    if (GL >= 8) v += dpp_f<0x141>(v);
+    if (GL >= 16) v += dpp_f<0x140>(v);
     return v;
 }
 
@@ -643,7 +654,7 @@ struct FlatX {
     }
 };
 
-// Flat form for one activation row and rows that are a whole number of GL-lane groups (GL = 16 or 8
+// Flat form for one activation row and rows that are a whole number of GL-lane groups (GL = 16, 8 or 4
 // units).  Rows are contiguous in the planar layout, so the units of a workgroup's rows [r0, r1) are
 // one flat sequence: a wave load covers 64 consecutive units of it (1 KB of quants, whatever the row
 // length), wave w takes loads w, w + 16, ...  Every GL-lane group lies inside one row; its sum goes
@@ -690,7 +701,7 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
                 const int u = flc - (int)__umulhi((unsigned)flc, magic_u) * U;   // flc mod U
                 float acc[1] = {0.f};
                 compute_unit<1, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
-                const float s = GL == 8 ? group_sum8(acc[0]) : group_sum<16>(acc[0]);
+                const float s = small_group_sum<GL>(acc[0]);
                 if (act && (lane & (GL - 1)) == GL - 1) part[fl / GL] = s;
             }
             c_t += 16;

@@ -66,7 +66,8 @@ def test_gemv_matches_q8_oracle(accel, orc, synth, relerr, ty, N, K):
 # odd for the flat form.
 FORM_SHAPES = [(2, 130, 2560), (2, 9, 96 * 32), (2, 2500, 2560), (2, 3, 4096 + 256), (2, 1, 512), (2, 300, 256),
                (2, 700, 8192), (2, 40, 16384), (2, 24, 16384 + 512), (2, 50, 32 * 129),
-               (8, 130, 2560), (8, 37, 9728), (8, 5, 32 * 68), (8, 1000, 1024), (8, 77, 128), (8, 60, 32 * 67)]
+               (8, 130, 2560), (8, 37, 9728), (8, 5, 32 * 68), (8, 1000, 1024), (8, 77, 128), (8, 60, 32 * 67),
+               (14, 70, 3840), (14, 9, 4352), (14, 1500, 256), (14, 33, 2048), (14, 5, 16384), (14, 3, 16640)]
 
 
 @pytest.mark.parametrize("form", [0, 1])     # smx_tune("gemv_flat"): 0 automatic, 1 never
