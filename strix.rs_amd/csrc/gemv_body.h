@@ -558,11 +558,11 @@ __device__ __forceinline__ void gemv_body(const GemvW W, const GemvX X, float* _
     SMX_STAMP_FLUSH();
 }
 
-// Sum over groups of GL = 4, 8 or 16 adjacent lanes (all lanes of a group end up with the total).
+// Sum over groups of GL = 2, 4, 8 or 16 adjacent lanes (all lanes of a group end up with the total).
 template <int GL>
 __device__ __forceinline__ float small_group_sum(float v) {
     v += dpp_f<0xB1>(v);
-    v += dpp_f<0x4E>(v);
+    if (GL >= 4) v += dpp_f<0x4E>(v);
     if (GL >= 8) v += dpp_f<0x141>(v);
     if (GL >= 16) v += dpp_f<0x140>(v);
     return v;

@@ -175,6 +175,129 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(const float* __res
     }
 }
 
+// The same work in the flat form of the dense GEMV, for layers whose k*eff intermediate values fit four
+// float4 items per thread: the units (16-byte half blocks) of a workgroup's rows, k experts side by
+// side per row, form one sequence that the 16 waves walk in 64-unit loads, three loads per round.
+// g and u are requested first and the weight loads follow without conditions, so waiting for g and u
+// does not wait for the weights (a wave's loads complete in order) and every later wait is exact.
+// Every GL-lane group lies inside one expert's row segment; its weighted sum goes to LDS and the groups
+// of a row are added in ascending order (expert k ascending, blocks ascending).
+template <int GL>
+__global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __restrict__ g, const float* __restrict__ u,
+                                                            const uint16_t* __restrict__ scales,
+                                                            const uint4* __restrict__ quants, const MoeRoute route,
+                                                            int k, int eff, int hidden, float* __restrict__ y,
+                                                            int* __restrict__ aq_out, float* __restrict__ ad_out,
+                                                            unsigned magic_units, unsigned magic_upe) {
+    extern __shared__ __align__(16) char smem[];
+    constexpr int PRE = 3, XI = 4;
+    const int nbe = eff / 32, upe = eff / 16, units = k * upe;
+    int* sxq = (int*)smem;                          // [k][eff] int8
+    float* sxd = (float*)(smem + (size_t)k * eff);  // [k][nbe]
+    int* sid = (int*)(sxd + k * nbe);               // [k] expert ids
+    float* sw = (float*)(sid + k);                  // [k] routing weights
+    float* part = sw + k;                           // [rows * units / GL]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid < k) {
+        sid[tid] = route.ids[tid];
+        sw[tid] = route.w[tid];
+    }
+    __syncthreads();
+    const unsigned rbase = (unsigned)hidden / gridDim.x, rrem = (unsigned)hidden - rbase * gridDim.x;
+    const int r0 = blockIdx.x * (int)rbase + min((int)blockIdx.x, (int)rrem);
+    const int rows = (int)rbase + ((int)blockIdx.x < (int)rrem ? 1 : 0);
+    const int nv = rows * units;                    // < 2^16 (launcher)
+    const int nloads = (nv + 63) >> 6;
+
+    const int items = k * eff / 4;                  // float4 items, 8 per block; <= XI * 1024 (launcher)
+    float4 gv[XI], uv[XI];
+#pragma unroll
+    for (int j = 0; j < XI; j++) {
+        const int it = tid + j * 1024;
+        gv[j] = uv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (it < items) {
+            gv[j] = ((const float4*)g)[it];
+            uv[j] = ((const float4*)u)[it];
+        }
+    }
+
+    uint4 q[PRE];
+    uint16_t sc[PRE];
+    int l_t = wave, c_t = wave;
+    // virtual unit v of the workgroup -> (row, expert, half block)
+    auto locate = [&](int v, int& rl, int& e, int& j16, int& uidx) {
+        rl = (int)__umulhi((unsigned)v, magic_units);
+        uidx = v - rl * units;
+        e = (int)__umulhi((unsigned)uidx, magic_upe);
+        j16 = uidx - e * upe;
+    };
+    auto request = [&]() {
+#pragma unroll
+        for (int s = 0; s < PRE; s++) {
+            int rl, e, j16, uidx;
+            locate(min(l_t * 64 + lane, max(nv - 1, 0)), rl, e, j16, uidx);
+            const size_t rowblk = ((size_t)sid[e] * hidden + min(r0 + rl, hidden - 1)) * nbe;
+            q[s] = quants[rowblk * 2 + j16];
+            sc[s] = scales[rowblk + (j16 >> 1)];
+            l_t += 16;
+        }
+    };
+    const uint4* sx16 = (const uint4*)smem;
+    auto consume = [&]() {
+#pragma unroll
+        for (int s = 0; s < PRE; s++) {
+            if (c_t < nloads) {   // wave-uniform
+                const int v = c_t * 64 + lane;
+                const bool act = v < nv;
+                int rl, e, j16, uidx;
+                locate(act ? v : nv - 1, rl, e, j16, uidx);
+                const uint4 xv = sx16[uidx];
+                int isum = dot4((int)q[s].x, (int)xv.x, 0);
+                isum = dot4((int)q[s].y, (int)xv.y, isum);
+                isum = dot4((int)q[s].z, (int)xv.z, isum);
+                isum = dot4((int)q[s].w, (int)xv.w, isum);
+                isum += swap1(isum);  // the other half of the block sits in the neighbouring lane
+                const float dx = sxd[e * nbe + (j16 >> 1)];
+                const float term = sw[e] * ((h2f(sc[s]) * dx) * (float)isum);
+                const float gs = small_group_sum<GL>((act && (lane & 1) == 0) ? term : 0.f);
+                if (act && (lane & (GL - 1)) == GL - 1) part[v / GL] = gs;
+            }
+            c_t += 16;
+        }
+    };
+    request();
+#pragma unroll
+    for (int j = 0; j < XI; j++) {
+        const int it = tid + j * 1024;
+        if ((it & ~63) < items) {   // whole waves are live or not together
+            int packed;
+            float d;
+            silu_mul_quant4(gv[j], uv[j], &packed, &d);
+            if (it < items) {
+                sxq[it] = packed;
+                if ((it & 7) == 0) sxd[it >> 3] = d;
+                if (blockIdx.x == 0 && aq_out) {
+                    aq_out[it] = packed;
+                    if ((it & 7) == 0) ad_out[it >> 3] = d;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    consume();
+    while (c_t < nloads) {
+        request();
+        consume();
+    }
+    __syncthreads();
+    const int G = units / GL;
+    for (int r = tid; r < rows; r += 1024) {
+        float s = 0.f;
+        for (int j = 0; j < G; j++) s += part[r * G + j];
+        y[r0 + r] = s;
+    }
+}
+
 // y[t][i] = sum over the token's slots (ascending slot index) of wslot[s]*dy[s][i]
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ dy, const int* __restrict__ tok_ptr,
                                                           const int* __restrict__ tok_slots,
@@ -323,13 +446,37 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
             return fail(c, SMX_ERR_LIMIT, "moe_ffn: %zu experts x %zu intermediate values need %zu bytes of LDS (limit 163840)",
                         k, eff, lds);
         ProfScope ps(c, "moe_gemv_down");
-        auto kern = moe_down_fused_kernel<6>;
-        static size_t lds_set = 0;
-        if ((rc = set_dyn_lds(c, kern, lds, &lds_set)) != SMX_OK) return rc;
-        const unsigned grid = (unsigned)std::min<size_t>((hidden + 7) / 8, (size_t)c->num_cu * 2);
-        hipLaunchKernelGGL(kern, dim3(grid), dim3(1024), lds, c->stream, s.g, s.u, L.down.scales, (const uint4*)L.down.quants,
-                           route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad);
-        SMX_HIP(c, hipGetLastError());
+        const size_t upe = eff / 16, units = k * upe;
+        const size_t fgrid = std::min<size_t>(hidden, (size_t)c->num_cu);
+        const size_t frows = (hidden + fgrid - 1) / fgrid;
+        const int gl = upe % 16 == 0 ? 16 : (upe % 8 == 0 ? 8 : (upe % 4 == 0 ? 4 : 2));
+        const size_t flds = lds + frows * units / gl * 4;
+        if (c->tune_gemv_flat != 1 && k * eff <= 4 * 1024 * 4 && frows * units < 65536 && flds <= 160 * 1024) {
+            const unsigned m_units = (unsigned)(((1ull << 32) + units - 1) / units), m_upe = (unsigned)(((1ull << 32) + upe - 1) / upe);
+            auto launch = [&](auto kern, size_t* lds_set) -> int {
+                int rc2 = set_dyn_lds(c, kern, flds, lds_set);
+                if (rc2 != SMX_OK) return rc2;
+                hipLaunchKernelGGL(kern, dim3((unsigned)fgrid), dim3(1024), flds, c->stream, s.g, s.u, L.down.scales,
+                                   (const uint4*)L.down.quants, route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad,
+                                   m_units, m_upe);
+                SMX_HIP(c, hipGetLastError());
+                return SMX_OK;
+            };
+            static size_t set16 = 0, set8 = 0, set4 = 0, set2 = 0;
+            if (gl == 16) rc = launch(moe_down_flat_kernel<16>, &set16);
+            else if (gl == 8) rc = launch(moe_down_flat_kernel<8>, &set8);
+            else if (gl == 4) rc = launch(moe_down_flat_kernel<4>, &set4);
+            else rc = launch(moe_down_flat_kernel<2>, &set2);
+            if (rc != SMX_OK) return rc;
+        } else {
+            auto kern = moe_down_fused_kernel<6>;
+            static size_t lds_set = 0;
+            if ((rc = set_dyn_lds(c, kern, lds, &lds_set)) != SMX_OK) return rc;
+            const unsigned grid = (unsigned)std::min<size_t>((hidden + 7) / 8, (size_t)c->num_cu * 2);
+            hipLaunchKernelGGL(kern, dim3(grid), dim3(1024), lds, c->stream, s.g, s.u, L.down.scales, (const uint4*)L.down.quants,
+                               route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad);
+            SMX_HIP(c, hipGetLastError());
+        }
     }
     if (out_scratch) *out_scratch = s;
     return SMX_OK;

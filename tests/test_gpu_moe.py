@@ -12,12 +12,24 @@ def _layer(accel, synth, layer, ne, hidden, eff, seed):
     return gate, up, down
 
 
-# k = 12: the 24 gate/up GEMVs exceed one grouped launch; eff = 416: down-projection units with a ragged tail
-@pytest.mark.parametrize("ne,hidden,eff,k", [(4, 64, 32, 2), (8, 256, 96, 3), (64, 2048, 768, 8), (16, 320, 416, 12)])
-def test_moe_ffn_stagewise(accel, orc, synth, relerr, ne, hidden, eff, k):
+# k = 12: the 24 gate/up GEMVs exceed one grouped launch; eff = 416: down-projection units with a ragged tail;
+# eff = 32, 96, 416, 224 / 64 / 128 / 768: unit groups of 2 / 4 / 8 / 16 lanes in the flat down kernel;
+# (8, 1024, 2560): k * eff too large for it.  form 1 = the flat GEMV / down kernels switched off.
+@pytest.mark.parametrize("form", [0, 1])
+@pytest.mark.parametrize("ne,hidden,eff,k", [(4, 64, 32, 2), (8, 256, 96, 3), (64, 2048, 768, 8), (16, 320, 416, 12),
+                                             (8, 96, 224, 4), (8, 192, 128, 4), (8, 128, 64, 2), (8, 1024, 2560, 8)])
+def test_moe_ffn_stagewise(accel, orc, synth, relerr, ne, hidden, eff, k, form):
     gate, up, down = _layer(accel, synth, 3, ne, hidden, eff, seed=ne + hidden)
     ids, w = synth.zipf_routing(1, ne, k, seed=5)
     x = synth.make_acts(1, hidden, seed=6)[0]
+    accel.tune("gemv_flat", form)
+    try:
+        _moe_stagewise(accel, orc, relerr, gate, up, down, ne, hidden, eff, k, ids, w, x)
+    finally:
+        accel.tune("gemv_flat", 0)
+
+
+def _moe_stagewise(accel, orc, relerr, gate, up, down, ne, hidden, eff, k, ids, w, x):
     y, gu, aq, ad = accel.moe_ffn_stages(3, ids[0], w[0], x, eff)
     ry, rgu, raq, rad = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[0], w[0], x)
     # stage 1: gate/up GEMVs
