@@ -197,7 +197,7 @@ void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
 /* Launch-geometry overrides for measurement sweeps; value 0 restores the built-in choice.
  * Knobs: "gemv_rpw" (rows per wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4),
  * "gemv_lpr" (lanes per row: 16, 32, 64), "gemv_wpc" (persistent workgroups per CU), "gemv_flat" (flat
- * GEMV form for small Q4_0 / Q8_0 weights: 0 automatic, 1 never), "gemm_splitk" (K slices), "gemm_nw" (waves, i.e. 32-token tiles, per GEMM workgroup: 4 or 8).  Results do not
+ * form of the single-row GEMV and of the MoE down projection: 0 automatic, 1 never), "gemm_splitk" (K slices), "gemm_nw" (waves, i.e. 32-token tiles, per GEMM workgroup: 4 or 8).  Results do not
  * depend on them beyond fp32 summation order. */
 int smx_tune(smx_ctx* ctx, const char* knob, int value);
 

@@ -40,10 +40,10 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, in
 }
 
 // Flat form (one activation row): blockIdx.x of gridDim.x workgroups share a job's rows.
-template <class Ops, int PRE, int GL, int FQ>
-__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, unsigned magic_u) {
+template <class Ops, int MT, int PRE, int GL, int FQ>
+__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, int m, unsigned magic_u) {
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body_flat<Ops, PRE, GL, FQ>(jb.W, jb.X, jb.y, nblk, jb.N, blockIdx.x, gridDim.x, magic_u);
+    gemv_body_flat<Ops, MT, PRE, GL, FQ>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u);
 }
 
 namespace {
@@ -84,33 +84,47 @@ int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk
     return launch_fq<Ops, MT, RPW, PRE, KS, LPR, MT == 1 ? 1 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
 }
 
-template <class Ops, int PRE, int GL, int FQ>
-int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
-    auto k = gemv_flat_kernel<Ops, PRE, GL, FQ>;
+template <class Ops, int MT, int PRE, int GL, int FQ>
+int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m) {
+    auto k = gemv_flat_kernel<Ops, MT, PRE, GL, FQ>;
     static size_t lds_set = 0;
     int rc = set_dyn_lds(c, k, g.lds, &lds_set);
     if (rc != SMX_OK) return rc;
-    const unsigned units = (unsigned)nblk * (std::is_same<Ops, OpsQ6_K>::value ? 4u : (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u));   // units per row
+    const unsigned upb = std::is_same<Ops, OpsQ6_K>::value ? 4u : (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u);
+    const unsigned units = (unsigned)nblk * upb;                             // units per row
     const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);   // floor(f * magic / 2^32) = f / units for f < 2^16
-    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, magic);
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, m, magic);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
 
-template <class Ops>
-int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk) {
-    if constexpr (std::is_same<Ops, OpsQ4_0>::value || std::is_same<Ops, OpsQ8_0>::value) {
-#define SMX_FLAT(PRE, GL)                                                                         \
-    if (g.flat_pre == PRE && g.flat == GL) {                                                      \
-        if (g.preq) return launch_flat_fq<Ops, PRE, GL, 0>(c, g, J, njobs, nblk);                 \
-        if (g.prod) return launch_flat_fq<Ops, PRE, GL, 2>(c, g, J, njobs, nblk);                 \
-        return launch_flat_fq<Ops, PRE, GL, 1>(c, g, J, njobs, nblk);                             \
+template <class Ops, int MT>
+int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m) {
+    constexpr bool kQ6 = std::is_same<Ops, OpsQ6_K>::value;
+    if constexpr (MT == 1) {
+#define SMX_FLAT(PRE, GL)                                                                            \
+    if (g.flat_pre == PRE && g.flat == GL) {                                                         \
+        if (g.preq) return launch_flat_fq<Ops, 1, PRE, GL, 0>(c, g, J, njobs, nblk, m);              \
+        if (g.prod) return launch_flat_fq<Ops, 1, PRE, GL, 2>(c, g, J, njobs, nblk, m);              \
+        return launch_flat_fq<Ops, 1, PRE, GL, 1>(c, g, J, njobs, nblk, m);                          \
     }
-        SMX_FLAT(3, 16) SMX_FLAT(3, 8)
-    } else if constexpr (std::is_same<Ops, OpsQ6_K>::value) {
-        SMX_FLAT(1, 16) SMX_FLAT(1, 8) SMX_FLAT(1, 4)
-    }
+        if constexpr (std::is_same<Ops, OpsQ4_0>::value || std::is_same<Ops, OpsQ8_0>::value) {
+            SMX_FLAT(3, 16) SMX_FLAT(3, 8)
+        } else if constexpr (kQ6) {
+            SMX_FLAT(1, 16) SMX_FLAT(1, 8) SMX_FLAT(1, 4)
+        }
 #undef SMX_FLAT
+    } else if constexpr (!(kQ6 && MT == 8)) {
+        // several rows arrive quantised
+        constexpr int PRE = kQ6 ? 1 : 2;
+        if (g.flat_pre == PRE) {
+            if (g.flat == 16) return launch_flat_fq<Ops, MT, PRE, 16, 0>(c, g, J, njobs, nblk, m);
+            if (g.flat == 8) return launch_flat_fq<Ops, MT, PRE, 8, 0>(c, g, J, njobs, nblk, m);
+            if constexpr (kQ6) {
+                if (g.flat == 4) return launch_flat_fq<Ops, MT, PRE, 4, 0>(c, g, J, njobs, nblk, m);
+            }
+        }
+    }
     return fail(c, SMX_ERR_ARG, "gemv: no flat variant for this geometry");
 }
 
@@ -122,7 +136,7 @@ int launch_variant(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
     // sub-wave rows: the pipeline is deep enough to put a whole short row set in flight before the
     // activation is staged (Q6_K units are three times as wide, so half the depth)
     constexpr bool kWide = sizeof(typename Ops::Regs) > 32;
-    if (MT == 1 && g.flat) return launch_flat<Ops>(c, g, J, njobs, nblk);
+    if (g.flat) return launch_flat<Ops, MT>(c, g, J, njobs, nblk, m);
     if (MT == 1 && g.lpr == 32) {
         if (g.rpw == 2) return launch_one<Ops, 1, 2, kWide ? 2 : 3, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
         return launch_one<Ops, 1, 1, kWide ? 2 : 4, 1, 32, false, 1024>(c, g, J, njobs, nblk, m, nullptr, 0);
@@ -225,22 +239,26 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
         if (dump) wpc = 8;
         g.grid = (unsigned)std::min<size_t>(wgs, cus * wpc);
     }
-    // Flat form: one activation row of up to 16384 elements, rows of a whole number of unit groups, at
-    // most 32 loads per wave (small and medium GEMVs, where start-up latency decides; measured up to 24).
-    if (mt == 1 && !dump && c->tune_gemv_flat != 1 && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
+    // Flat form: one activation row of up to 16384 elements and rows of a whole number of unit groups.
+    // Measured against the persistent form above: Q4_0 9728 x 2560 6.8 -> 5.4 us, eight of them in one
+    // launch 24.8 -> 22.4 us, Q6_K 262144 x 3840 159 -> 144 us.
+    if (!dump && c->tune_gemv_flat != 1 && !(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
         nblk * (type == kQ6_K ? 256 : 32) <= 16384) {  // the row is held in registers while the weights are requested
-        const size_t fwgs = std::max<size_t>(1, std::min(cus, N));
+        // a workgroup's units are indexed with 16 bits: whole further rounds of workgroups when a CU's share is larger
+        const size_t rounds = ((N + cus - 1) / cus * units + 65534) / 65535;
+        const size_t fwgs = std::min(N, cus * rounds);
         const size_t rows = (N + fwgs - 1) / fwgs;                 // of the workgroup with the most rows
-        const size_t loads = (rows * units + 63) / 64, per_wave = (loads + 15) / 16;
-        const size_t lim = c->tune_gemv_flat >= 2 ? (size_t)c->tune_gemv_flat : 32;
-        if (per_wave <= lim && rows * units < 65536) {
-            g.flat = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : 4);
+        g.flat = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : 4);
+        const size_t lds = tokb * (size_t)mt + rows * units / g.flat * 4 * mt;
+        if (rows * units < 65536 && lds <= 160 * 1024) {
             // loads requested per round, measured: Q4_0 pair 8.2 / 8.0 / 7.7 / 8.1 / 8.9 us with 1 / 2 / 3 / 4 / 6,
             // Q6_K 15360 x 3840 (five load instructions per unit) 11.4 / 12.5 / 14.1 / 14.8 us with 1 / 2 / 3 / 4
-            g.flat_pre = type == kQ6_K ? 1 : 3;
+            g.flat_pre = type == kQ6_K ? 1 : (mt == 1 ? 3 : 2);
             g.nt = 1024;
             g.grid = (unsigned)fwgs;
-            g.lds = tokb + rows * units / g.flat * 4;
+            g.lds = lds;
+        } else {
+            g.flat = 0;
         }
     }
     return g;

@@ -148,10 +148,21 @@ struct OpsQ8_0 {
 struct OpsQ8_0W : OpsQ8_0 {
     struct Regs { uint4 q0, q1; uint16_t s; };
     static __device__ __forceinline__ int units_per_row(int nblk) { return nblk; }
+    // LDS per token: first halves [nb] uint4 | second halves [nb] uint4 | sd[nb] f32 -- a lane reads both
+    // halves of its block, and consecutive lanes read consecutive 16-byte chunks of a plane
+    static __device__ __forceinline__ int* xq_dword(char* tok, int nblk, int blk, int sub) {
+        uint4* lo = (uint4*)tok;
+        return (int*)((sub < 4 ? lo : lo + nblk) + blk) + (sub & 3);
+    }
     static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nblk, int u) {
         r.q0 = w.quants[(row * nblk + u) * 2];
         r.q1 = w.quants[(row * nblk + u) * 2 + 1];
         r.s = w.scales[row * nblk + u];
+    }
+    static __device__ __forceinline__ void load_flat(Regs& r, const GemvW& w, size_t f) {
+        r.q0 = w.quants[f * 2];
+        r.q1 = w.quants[f * 2 + 1];
+        r.s = w.scales[f];
     }
 };
 
@@ -253,7 +264,7 @@ __device__ __forceinline__ void compute_unit(OpsQ8_0W, const OpsQ8_0W::Regs& r, 
 #pragma unroll
     for (int t = 0; t < MT; t++) {
         const char* tok = smem + t * tokb;
-        const uint4 x0 = ((const uint4*)tok)[u * 2], x1 = ((const uint4*)tok)[u * 2 + 1];
+        const uint4 x0 = ((const uint4*)tok)[u], x1 = ((const uint4*)tok)[nblk + u];
         const float dx = ((const float*)(tok + nblk * 32))[u];
         int isum = dot4((int)r.q0.x, (int)x0.x, 0);
         isum = dot4((int)r.q0.y, (int)x0.y, isum);
@@ -654,6 +665,45 @@ struct FlatX {
     }
 };
 
+// The same for m <= MT pre-quantised rows (several activation rows per weight pass): one 16-byte
+// half block per row and thread, rows of up to 16384 elements.
+template <class Ops, int MT>
+struct FlatXRows {
+    uint4 pk[MT];
+    float d[MT];
+    int sp[MT];
+
+    __device__ __forceinline__ void request(const GemvX& X, int nblk, int m) {
+        const int nb32 = Ops::nb32(nblk);
+        const int i = threadIdx.x;
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            pk[t] = make_uint4(0, 0, 0, 0);
+            d[t] = 0.f;
+            sp[t] = 0;
+            if (i < nb32 * 2 && t < m) {
+                pk[t] = ((const uint4*)(X.xq + (size_t)t * nb32 * 32))[i];
+                if ((i & 1) == 0) {
+                    d[t] = X.xd[(size_t)t * nb32 + (i >> 1)];
+                    if (Ops::kNeedsSums) sp[t] = X.xs[(size_t)t * nb32 + (i >> 1)];
+                }
+            }
+        }
+    }
+    // rows past m are staged as zeros (their results are not written)
+    __device__ __forceinline__ void store(char* smem, int tokb, int nblk) {
+        const int i = threadIdx.x;
+        if (i < Ops::nb32(nblk) * 2) {
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                char* tok = smem + t * tokb;
+                *(uint4*)Ops::xq_dword(tok, nblk, i >> 1, (i & 1) * 4) = pk[t];
+                if ((i & 1) == 0) Ops::put_scale(tok, nblk, i >> 1, d[t], (int)(short)(sp[t] & 0xffff), sp[t] >> 16);
+            }
+        }
+    }
+};
+
 // Flat form for one activation row and rows that are a whole number of GL-lane groups (GL = 16, 8 or 4
 // units).  Rows are contiguous in the planar layout, so the units of a workgroup's rows [r0, r1) are
 // one flat sequence: a wave load covers 64 consecutive units of it (1 KB of quants, whatever the row
@@ -663,9 +713,12 @@ struct FlatX {
 // last unit) so that the wait for ring slot k is exactly "all but the loads issued after it" instead
 // of "all loads".  A round requests PRE loads and consumes them; the activation is staged during the
 // first round, after its weight loads are out.
-template <class Ops, int PRE, int GL, int FQ>
-__device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, float* __restrict__ y, int nblk, int N,
-                                               int wg, int n_wgs, unsigned magic_u) {
+//
+// MT > 1: m <= MT pre-quantised activation rows (FQ = 0) share every weight load; y[t * ldy + row].
+template <class Ops, int MT, int PRE, int GL, int FQ>
+__device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, float* __restrict__ y, int ldy, int nblk,
+                                               int N, int m, int wg, int n_wgs, unsigned magic_u) {
+    static_assert(MT == 1 || FQ == 0, "several activation rows are staged from quantised rows");
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int U = Ops::units_per_row(nblk);
@@ -675,11 +728,13 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     const int nunits = (r1 - r0) * U;          // < 2^16 (launcher)
     const int nloads = (nunits + 63) >> 6;
     const int tokb = Ops::tok_bytes(nblk);
-    float* part = (float*)(smem + tokb);       // [nunits / GL]
+    float* part = (float*)(smem + MT * tokb);  // [nunits / GL][MT]
     const size_t f_base = (size_t)r0 * U;
 
     FlatX<Ops, FQ> xs;
-    xs.request(X, nblk);
+    FlatXRows<Ops, MT> xr;
+    if (MT == 1) xs.request(X, nblk);
+    else xr.request(X, nblk, m);
 
     typename Ops::Regs ring[PRE];
     int l_t = wave, c_t = wave;
@@ -699,16 +754,22 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
                 const bool act = fl < nunits;
                 const int flc = act ? fl : nunits - 1;
                 const int u = flc - (int)__umulhi((unsigned)flc, magic_u) * U;   // flc mod U
-                float acc[1] = {0.f};
-                compute_unit<1, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
-                const float s = small_group_sum<GL>(acc[0]);
-                if (act && (lane & (GL - 1)) == GL - 1) part[fl / GL] = s;
+                float acc[MT];
+#pragma unroll
+                for (int t = 0; t < MT; t++) acc[t] = 0.f;
+                compute_unit<MT, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const float s = small_group_sum<GL>(acc[t]);
+                    if (act && (lane & (GL - 1)) == GL - 1) part[(fl / GL) * MT + t] = s;
+                }
             }
             c_t += 16;
         }
     };
     request();
-    xs.store(smem, nblk, X);
+    if (MT == 1) xs.store(smem, nblk, X);
+    else xr.store(smem, tokb, nblk);
     __syncthreads();
     consume();
     while (c_t < nloads) {
@@ -717,10 +778,11 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     }
     __syncthreads();
     const int G = U / GL;
-    for (int r = threadIdx.x; r < r1 - r0; r += blockDim.x) {
+    for (int i = threadIdx.x; i < (r1 - r0) * MT; i += blockDim.x) {
+        const int r = i / MT, t = i % MT;
         float s = 0.f;
-        for (int j = 0; j < G; j++) s += part[r * G + j];
-        y[r0 + r] = s;
+        for (int j = 0; j < G; j++) s += part[(r * G + j) * MT + t];
+        if (t < m) y[(size_t)t * ldy + r0 + r] = s;
     }
 }
 
