@@ -2,12 +2,14 @@
 //
 // Stands in for the reference's decode GEMVs (crates/strix-backend-rocm/src/kernels.rs:259-287
 // q4_gemv_dp, :894-912 q8i_gemv, :1016-1045 q8i_gemm_rows32, :607-640 q6_gemv) on gfx950:
-//   * one wavefront (64 lanes) per output row, RPW rows per wave, NW waves per workgroup;
-//   * every lane streams 128-bit chunks of the row's packed quants straight from HBM, the next
-//     pass is issued before the current one is consumed;
-//   * the quantised activation (int8 + scales + 16-element sums) is staged once per workgroup in LDS;
+//   * 16-wave workgroups, one per CU; the quantised activation (int8 + scales + 16-element sums) is
+//     staged once per workgroup in LDS, quantised on the way when it arrives as fp32;
+//   * every lane streams 128-bit units of the packed quants straight from HBM;
 //   * v_dot4_i32_i8 integer block dots, exact i32 per block, then acc += (dw*dx)*float(isum);
-//   * cross-lane (DPP) combination of lanes that share a block, wave-wide reduction at the end.
+//   * cross-lane (DPP) combination of lanes that share a block and of the lanes of a row.
+// Two forms (gemv_body.h): the flat form (activation requested before the weights, a workgroup's rows
+// walked as one sequence of 64-unit loads, no conditional loads) for every shape whose rows are a whole
+// number of unit groups, and the persistent row-per-wave form for the rest.
 // HBM-bound: algorithmic bytes per row are K/32 * {18, 34} (Q4_0, Q8_0) or K/256 * 210 (Q6_K).
 #include <algorithm>
 #include <type_traits>

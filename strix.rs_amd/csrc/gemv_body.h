@@ -1,4 +1,5 @@
-// Device body of the fused block-dequant GEMV (shared by the dense and the MoE launches).
+// Device bodies of the fused block-dequant GEMV (shared by the dense and the MoE launches): the
+// persistent form described next (gemv_body) and the flat form (gemv_body_flat, further down).
 //
 // One wavefront serves RPW consecutive output rows at a time ("chunk") and walks the rows in
 // 64-lane passes; every lane streams one 16-byte unit of packed quants per row and pass:
