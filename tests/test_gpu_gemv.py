@@ -93,6 +93,19 @@ def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K, form)
     accel.evict("t.form2")
 
 
+def test_gemv_group_with_more_workgroups_than_cus(accel, orc, synth, relerr):
+    # eight jobs share the chip: a job's share of 30000 x 80 units per CU exceeds what a workgroup of the
+    # flat form indexes, so each job runs as two rounds of workgroups
+    N, K = 30000, 2560
+    raw = synth.make_weight(2, N, K, seed=99)
+    _up(accel, 2, "t.big", raw, K, N)
+    xs = [synth.make_acts(1, K, seed=300 + i)[0] for i in range(8)]
+    out = accel.gemv_batch([("t.big", x) for x in xs], [N] * 8)
+    for i in (0, 3, 7):
+        assert relerr(out[i], orc.matmul_q8_from_f32(2, raw, K, N, xs[i])[0]) <= TOL
+    accel.evict("t.big")
+
+
 @pytest.mark.parametrize("ty", [2, 8])
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
 def test_gemv_rows_batched(accel, orc, synth, relerr, ty, m):
