@@ -244,7 +244,9 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     // Flat form: one activation row of up to 16384 elements and rows of a whole number of unit groups.
     // Measured against the persistent form above: Q4_0 9728 x 2560 6.8 -> 5.4 us, eight of them in one
     // launch 24.8 -> 22.4 us, Q6_K 262144 x 3840 159 -> 144 us.
-    if (!dump && c->tune_gemv_flat != 1 && !(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
+    // (a sweep that sets one of the persistent form's knobs gets the persistent form)
+    const bool knobs = c->tune_gemv_rpw > 0 || c->tune_gemv_ks > 0 || c->tune_gemv_lpr > 0 || c->tune_gemv_wpc > 0;
+    if (!dump && !knobs && c->tune_gemv_flat != 1 && !(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
         nblk * (type == kQ6_K ? 256 : 32) <= 16384) {  // the row is held in registers while the weights are requested
         // a workgroup's units are indexed with 16 bits: whole further rounds of workgroups when a CU's share is larger
         const size_t rounds = ((N + cus - 1) / cus * units + 65534) / 65535;

@@ -730,7 +730,9 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     const int nloads = (nunits + 63) >> 6;
     const int tokb = Ops::tok_bytes(nblk);
     float* part = (float*)(smem + MT * tokb);  // [nunits / GL][MT]
-    const size_t f_base = (size_t)r0 * U;
+    // a job with fewer rows than the launch has workgroups leaves some without rows: their (unused)
+    // loads go to the weight's first unit
+    const size_t f_base = nunits > 0 ? (size_t)r0 * U : 0;
 
     FlatX<Ops, FQ> xs;
     FlatXRows<Ops, MT> xr;

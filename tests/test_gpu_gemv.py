@@ -93,6 +93,20 @@ def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K, form)
     accel.evict("t.form2")
 
 
+def test_gemv_group_of_very_different_row_counts(accel, orc, synth, relerr):
+    # the launch geometry follows the largest job: most workgroups of the 2-row job have no rows at all
+    K = 2560
+    for ty in (2, 8, 14):
+        raws = {n: synth.make_weight(ty, n, K, seed=ty * 100 + n) for n in (2, 3000)}
+        for n, raw in raws.items():
+            _up(accel, ty, f"t.n{n}", raw, K, n)
+        x = synth.make_acts(1, K, seed=ty)[0]
+        out = accel.gemv_batch([("t.n2", x), ("t.n3000", x)], [2, 3000])
+        for o, n in zip(out, (2, 3000)):
+            assert relerr(o, orc.matmul_q8_from_f32(ty, raws[n], K, n, x)[0]) <= TOL
+            accel.evict(f"t.n{n}")
+
+
 def test_gemv_group_with_more_workgroups_than_cus(accel, orc, synth, relerr):
     # eight jobs share the chip: a job's share of 30000 x 80 units per CU exceeds what a workgroup of the
     # flat form indexes, so each job runs as two rounds of workgroups
