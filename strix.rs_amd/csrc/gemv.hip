@@ -249,7 +249,8 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     if (!dump && !knobs && c->tune_gemv_flat != 1 && !(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
         nblk * (type == kQ6_K ? 256 : 32) <= 16384) {  // the row is held in registers while the weights are requested
         // a workgroup's units are indexed with 16 bits: whole further rounds of workgroups when a CU's share is larger
-        const size_t rounds = ((N + cus - 1) / cus * units + 65534) / 65535;
+        const size_t share = (N + cus - 1) / cus * units;   // units of a CU's share of the rows
+        const size_t rounds = share < 65536 ? 1 : (share + 59999) / 60000;   // margin for the rounding of rows per workgroup
         const size_t fwgs = std::min(N, cus * rounds);
         const size_t rows = (N + fwgs - 1) / fwgs;                 // of the workgroup with the most rows
         g.flat = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : 4);
