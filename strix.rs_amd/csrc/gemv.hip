@@ -118,7 +118,7 @@ int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nbl
 #undef SMX_FLAT
     } else if constexpr (!(kQ6 && MT == 8)) {
         // several rows arrive quantised
-        constexpr int PRE = kQ6 ? 1 : 2;
+        constexpr int PRE = 1;
         if (g.flat_pre == PRE) {
             if (g.flat == 16) return launch_flat_fq<Ops, MT, PRE, 16, 0>(c, g, J, njobs, nblk, m);
             if (g.flat == 8) return launch_flat_fq<Ops, MT, PRE, 8, 0>(c, g, J, njobs, nblk, m);
@@ -257,8 +257,9 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
         const size_t lds = tokb * (size_t)mt + rows * units / g.flat * 4 * mt;
         if (rows * units < 65536 && lds <= 160 * 1024) {
             // loads requested per round, measured: Q4_0 pair 8.2 / 8.0 / 7.7 / 8.1 / 8.9 us with 1 / 2 / 3 / 4 / 6,
-            // Q6_K 15360 x 3840 (five load instructions per unit) 11.4 / 12.5 / 14.1 / 14.8 us with 1 / 2 / 3 / 4
-            g.flat_pre = type == kQ6_K ? 1 : (mt == 1 ? 3 : 2);
+            // Q6_K 15360 x 3840 (five load instructions per unit) 11.4 / 12.5 / 14.1 / 14.8 us with 1 / 2 / 3 / 4,
+            // eight rows on Q8_0 2560 x 9728 14.1-14.6 / 14.8 / 15.8 us with 1 / 2 / 3
+            g.flat_pre = type == kQ6_K ? 1 : (mt == 1 ? 3 : 1);
             g.nt = 1024;
             g.grid = (unsigned)fwgs;
             g.lds = lds;
