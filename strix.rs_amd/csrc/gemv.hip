@@ -248,13 +248,18 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     const bool knobs = c->tune_gemv_rpw > 0 || c->tune_gemv_ks > 0 || c->tune_gemv_lpr > 0 || c->tune_gemv_wpc > 0;
     if (!dump && !knobs && c->tune_gemv_flat != 1 && !(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
         nblk * (type == kQ6_K ? 256 : 32) <= 16384) {  // the row is held in registers while the weights are requested
-        // a workgroup's units are indexed with 16 bits: whole further rounds of workgroups when a CU's share is larger
-        const size_t share = (N + cus - 1) / cus * units;   // units of a CU's share of the rows
-        const size_t rounds = share < 65536 ? 1 : (share + 59999) / 60000;   // margin for the rounding of rows per workgroup
-        const size_t fwgs = std::min(N, cus * rounds);
-        const size_t rows = (N + fwgs - 1) / fwgs;                 // of the workgroup with the most rows
+        // a workgroup's units are indexed with 16 bits and its group sums live in LDS: whole further
+        // rounds of workgroups when a CU's share of the rows is too large for either
         g.flat = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : 4);
-        const size_t lds = tokb * (size_t)mt + rows * units / g.flat * 4 * mt;
+        const size_t share = (N + cus - 1) / cus * units;   // units of a CU's share of the rows
+        size_t rounds = share < 65536 ? 1 : (share + 59999) / 60000;   // margin for the rounding of rows per workgroup
+        size_t fwgs, rows, lds;
+        for (;; rounds++) {
+            fwgs = std::min(N, cus * rounds);
+            rows = (N + fwgs - 1) / fwgs;                          // of the workgroup with the most rows
+            lds = tokb * (size_t)mt + rows * units / g.flat * 4 * mt;
+            if (lds <= 128 * 1024 || fwgs == N) break;
+        }
         if (rows * units < 65536 && lds <= 160 * 1024) {
             // loads requested per round, measured: Q4_0 pair 8.2 / 8.0 / 7.7 / 8.1 / 8.9 us with 1 / 2 / 3 / 4 / 6,
             // Q6_K 15360 x 3840 (five load instructions per unit) 11.4 / 12.5 / 14.1 / 14.8 us with 1 / 2 / 3 / 4,

@@ -41,6 +41,13 @@ def test_lm_head_q6k_sampled(accel, orc, synth, relerr):
     ref = orc.matmul_q8_from_f32(14, sub, K, rows.size, x)[0]
     assert np.abs(y[rows] - ref).max() / np.abs(y).max() <= TOL
     assert int(accel.lm_head_argmax_rows("t.head", x, 1)[0]) == int(np.argmax(y))
+    # three rows per weight pass (the verify step of speculative decoding): the group sums of a CU's
+    # 1024 rows x 4 rows of activations no longer fit LDS, so the launch takes two rounds of workgroups
+    xs = synth.make_acts(3, K, seed=5)
+    ys = accel.gemv_rows("t.head", xs, N)
+    refs = orc.matmul_q8_from_f32(14, sub, K, rows.size, xs)
+    assert np.abs(ys[:, rows] - refs).max() / np.abs(ys).max() <= TOL
+    assert [int(v) for v in accel.lm_head_argmax_rows("t.head", xs, 3)] == [int(np.argmax(r)) for r in ys]
     accel.evict("t.head")
 
 
