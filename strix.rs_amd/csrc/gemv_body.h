@@ -583,7 +583,7 @@ __device__ __forceinline__ float small_group_sum(float v) {
 // The activation row of the flat form: every global load is requested up front (before the weight
 // stream, so that waiting for the row does not wait for the weights: a wave's loads complete in
 // order), the values are quantised and written to LDS later.  Thread t holds items t, t + 1024, ...
-// Rows of up to 16384 elements (fp32 row) or 32768 (pre-quantised row).
+// Holds rows of up to 16384 elements (the launcher's bound for this form).
 template <class Ops, int FQ>
 struct FlatX {
     static constexpr int XI = FQ == 0 ? 2 : 4;
@@ -705,8 +705,7 @@ struct FlatXRows {
     }
 };
 
-// Flat form for one activation row and rows that are a whole number of GL-lane groups (GL = 16, 8 or 4
-// units).  Rows are contiguous in the planar layout, so the units of a workgroup's rows [r0, r1) are
+// Flat form for weight rows that are a whole number of GL-lane groups (GL = 16, 8 or 4 units).  Rows are contiguous in the planar layout, so the units of a workgroup's rows [r0, r1) are
 // one flat sequence: a wave load covers 64 consecutive units of it (1 KB of quants, whatever the row
 // length), wave w takes loads w, w + 16, ...  Every GL-lane group lies inside one row; its sum goes
 // to LDS, and after a barrier the groups of a row are added in ascending order.  All waves of a
