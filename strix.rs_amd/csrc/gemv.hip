@@ -184,7 +184,7 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     size_t tokb, units;
     if (type == kQ4_0) { tokb = (nblk * 40 + 15) & ~size_t(15); units = nblk; }
     else if (type == kQ8_0) { tokb = (nblk * 36 + 15) & ~size_t(15); units = (mt >= 4 && !dump) ? nblk : nblk * 2; }
-    else { tokb = nblk * 2 * 176; units = nblk * 4; }
+    else { tokb = nblk * 2 * (OpsQ6_K::kPad * 16 + 32); units = nblk * 4; }
     g.nt = 1024;
     g.lpr = 64;
     g.ks = 1;

@@ -171,15 +171,18 @@ struct OpsQ6_K {
     struct Regs { uint4 a, b, h; uint2 sc; uint16_t d; };
     static __device__ __forceinline__ int units_per_row(int nsb) { return nsb * 4; }
     static __device__ __forceinline__ int nb32(int nsb) { return nsb * 8; }
-    static __device__ __forceinline__ int tok_bytes(int nsb) { return nsb * 2 * (9 * 16 + 16 + 16); }
-    // LDS per token: xq 16-byte chunks, 8 per 128 elements padded to 9 | sd float4[2nsb] | ss int4[2nsb]
+    static constexpr int kPad = 10;  // 16-byte chunks per 128 elements in LDS (8 used)
+    static __device__ __forceinline__ int tok_bytes(int nsb) { return nsb * 2 * (kPad * 16 + 16 + 16); }
+    // LDS per token: xq 16-byte chunks, 8 per 128 elements padded to kPad (lanes 2g, 2g + 1 read chunks
+    // kPad * g + 2j + {0, 1}: with 10, eight consecutive lanes fall into eight different 16-byte bank groups) |
+    // sd float4[2nsb] | ss int4[2nsb]
     static __device__ __forceinline__ int* xq_dword(char* tok, int, int blk, int sub) {
         const int ci = blk * 2 + (sub >> 2);
-        return (int*)((uint4*)tok + (ci >> 3) * 9 + (ci & 7)) + (sub & 3);
+        return (int*)((uint4*)tok + (ci >> 3) * kPad + (ci & 7)) + (sub & 3);
     }
     static __device__ __forceinline__ void put_scale(char* tok, int nsb, int blk, float d, int s_lo, int s_hi) {
-        ((float*)(tok + nsb * 2 * 144))[blk] = d;
-        ((int*)(tok + nsb * 2 * 160))[blk] = (s_lo & 0xffff) | (s_hi << 16);
+        ((float*)(tok + nsb * 2 * kPad * 16))[blk] = d;
+        ((int*)(tok + nsb * 2 * (kPad * 16 + 16)))[blk] = (s_lo & 0xffff) | (s_hi << 16);
     }
     static constexpr bool kNeedsSums = true;
     static __device__ __forceinline__ void load(Regs& r, const GemvW& w, size_t row, int nsb, int u) {
@@ -306,13 +309,13 @@ __device__ __forceinline__ void compute_unit(OpsQ6_K, const OpsQ6_K::Regs& r, co
     for (int t = 0; t < MT; t++) {
         const char* tok = smem + t * tokb;
         const uint4* sq = (const uint4*)tok;
-        const float4 dx4 = ((const float4*)(tok + nsb * 2 * 144))[g];
-        const int4 sp4 = ((const int4*)(tok + nsb * 2 * 160))[g];
+        const float4 dx4 = ((const float4*)(tok + nsb * 2 * OpsQ6_K::kPad * 16))[g];
+        const int4 sp4 = ((const int4*)(tok + nsb * 2 * (OpsQ6_K::kPad * 16 + 16)))[g];
         const float dxs[4] = {dx4.x, dx4.y, dx4.z, dx4.w};
         const int sps[4] = {sp4.x, sp4.y, sp4.z, sp4.w};
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint4 xv = sq[g * 9 + 2 * j + c];
+            const uint4 xv = sq[g * OpsQ6_K::kPad + 2 * j + c];
             int is = dot4((int)q[j][0], (int)xv.x, 0);
             is = dot4((int)q[j][1], (int)xv.y, is);
             is = dot4((int)q[j][2], (int)xv.z, is);
