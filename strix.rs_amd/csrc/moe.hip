@@ -298,19 +298,44 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
     }
 }
 
-// y[t][i] = sum over the token's slots (ascending slot index) of wslot[s]*dy[s][i]
+// y[t][i] = sum over the token's slots (ascending slot index) of wslot[s]*dy[s][i].  Eight slots at a
+// time: their indices, weights and rows are requested together (clamped, not conditional, so the
+// loads of a batch are in flight at once instead of one dependent round trip per slot).
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ dy, const int* __restrict__ tok_ptr,
                                                           const int* __restrict__ tok_slots,
                                                           const float* __restrict__ wslot, float* __restrict__ y,
-                                                          int hidden) {
-    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+                                                          int hidden, bool y_vec) {
+    const int t = blockIdx.y, i = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= hidden) return;
-    float s = 0.f;
-    for (int j = tok_ptr[t]; j < tok_ptr[t + 1]; j++) {
-        const int sl = tok_slots[j];
-        s += wslot[sl] * dy[(size_t)sl * hidden + i];
+    const int j0 = tok_ptr[t], j1 = tok_ptr[t + 1];
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int jb = j0; jb < j1; jb += 8) {
+        int sl[8];
+        float w[8];
+        float4 v[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) sl[q] = tok_slots[min(jb + q, j1 - 1)];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            w[q] = wslot[sl[q]];
+            v[q] = *(const float4*)(dy + (size_t)sl[q] * hidden + i);
+        }
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            if (jb + q < j1) {
+                s.x += w[q] * v[q].x;
+                s.y += w[q] * v[q].y;
+                s.z += w[q] * v[q].z;
+                s.w += w[q] * v[q].w;
+            }
+        }
     }
-    y[(size_t)t * hidden + i] = s;
+    float* o = y + (size_t)t * hidden + i;
+    if (y_vec) {   // the caller's buffer is 16-byte aligned
+        *(float4*)o = s;
+    } else {
+        o[0] = s.x; o[1] = s.y; o[2] = s.z; o[3] = s.w;
+    }
 }
 
 static int silu_mul_quant(smx_ctx* c, const float* g, const float* u, size_t ldg, size_t rows, size_t eff, int8_t* xq,
@@ -768,9 +793,9 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
     if (rc != SMX_OK) return rc;
     {
         ProfScope ps(c, "moe_combine");
-        hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((hidden + 255) / 256), (unsigned)m), dim3(256), 0, c->stream,
+        hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((hidden / 4 + 255) / 256), (unsigned)m), dim3(256), 0, c->stream,
                            dy, (const int*)(c->tab.p + o_tp), (const int*)(c->tab.p + o_ts),
-                           (const float*)(c->tab.p + o_ws), y_dev, (int)hidden);
+                           (const float*)(c->tab.p + o_ws), y_dev, (int)hidden, ((uintptr_t)y_dev & 15) == 0);
         SMX_HIP(c, hipGetLastError());
     }
     if (!on_device) {
