@@ -62,3 +62,14 @@ def test_oracle_reproduces_golden_fixtures(orc, golden, name):
         b = raw[2:18].astype(np.int64)
         q = np.concatenate([b & 15, b >> 4]) - 8
         assert int((q * g["xq"][0, :32].astype(np.int64)).sum()) == int(g["block_dots"][0, 0, 0])
+
+
+def test_multiply_high_division_used_by_the_flat_kernels_is_exact():
+    """The flat GEMV and the flat MoE down kernel find a unit's row with one multiply-high:
+    floor(f * ceil(2^32 / U) / 2^32) must equal f // U for every unit index a workgroup can hold
+    (f < 2^16) and every row length the launchers admit (U < 2^16)."""
+    import numpy as np
+    f = np.arange(1 << 16, dtype=np.uint64)
+    for U in list(range(1, 2049)) + [3040, 4095, 4096, 6144, 12288, 32767, 32768, 65535]:
+        magic = np.uint64(((1 << 32) + U - 1) // U)
+        assert np.array_equal((f * magic) >> np.uint64(32), f // np.uint64(U)), U
