@@ -75,8 +75,13 @@ int smx_upload_moe_q8(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_
 int smx_upload_moe_q6(smx_ctx* ctx, size_t layer, const void* gate, size_t gate_nbytes,
                       const void* up, size_t up_nbytes, const void* down, size_t down_nbytes,
                       size_t hidden, size_t eff, size_t ne);
-/* Drop one resident weight (the reference never frees, decode.rs:458-460). */
+/* Drop one resident weight (the reference never frees, decode.rs:458-460).  While a captured graph of
+ * the context is alive the device memory is kept until smx_destroy (a replay may still read it); the
+ * same holds for the old allocation when a key or an expert layer is uploaded again. */
 int smx_evict(smx_ctx* ctx, const char* key);
+/* Shape of a resident weight as given at upload (what the trait's gemv sizes its result with,
+ * decode.rs:3830-3832): 1 and the dimensions, 0 when the key is not resident.  Either out pointer may be NULL. */
+int smx_weight_dims(const smx_ctx* ctx, const char* key, size_t* in_dim, size_t* out_dim);
 
 /* ---- decode GEMV ---- */
 /* WeightAccel::gemv, accel.rs:391; decode.rs:3827-3898.  y = W.x with x
@@ -194,11 +199,12 @@ int smx_graph_end(smx_ctx* ctx, smx_graph** out);
 int smx_graph_launch(smx_ctx* ctx, smx_graph* g);   /* enqueue one replay on the context's stream */
 void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
 
-/* Launch-geometry overrides for measurement sweeps; value 0 restores the built-in choice.
- * Knobs: "gemv_rpw" (rows per wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4),
- * "gemv_lpr" (lanes per row: 16, 32, 64), "gemv_wpc" (persistent workgroups per CU), "gemv_flat" (flat
- * form of the single-row GEMV and of the MoE down projection: 0 automatic, 1 never), "gemm_splitk" (K slices), "gemm_nw" (waves, i.e. 32-token tiles, per GEMM workgroup: 4 or 8).  Results do not
- * depend on them beyond fp32 summation order. */
+/* Launch-geometry overrides for measurement sweeps; value 0 restores the built-in choice.  They shape
+ * a kernel's launch, never which kernel a shape is served by.
+ * Knobs: "gemm_splitk" (K slices of the GEMM); for shapes served by the row-per-wavefront GEMV (rows that
+ * are not a whole number of 16-byte unit groups, or longer than 16384 elements): "gemv_rpw" (rows per
+ * wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4), "gemv_lpr" (lanes per row: 16, 32,
+ * 64), "gemv_wpc" (workgroups per CU).  Results do not depend on them beyond fp32 summation order. */
 int smx_tune(smx_ctx* ctx, const char* knob, int value);
 
 /* ---- GGUF file -> resident weights: the loader side of the path, crates/strix-models/src/gguf.rs:104-238
@@ -251,7 +257,8 @@ const char* smx_prof_names(smx_ctx* ctx);    /* comma-separated kernel names see
 int smx_timer_begin(smx_ctx* ctx);
 int smx_timer_end(smx_ctx* ctx, float* ms);  /* syncs */
 
-/* ---- parity instrumentation (same device code path, integer results dumped) ---- */
+/* ---- parity instrumentation: the kernel the same call would run without the dump (same launch
+ *      geometry, same device code), with the integers it forms also written out ---- */
 /* Device activation quantiser: xq[m][k] i8, xd[m][k/32] f32, xs16[m][k/16] i16. */
 int smx_quantize(smx_ctx* ctx, const float* x, size_t m, size_t k, int8_t* xq, float* xd,
                  int16_t* xs16);
@@ -266,6 +273,13 @@ int smx_gemm_block_dots(smx_ctx* ctx, const char* key, const float* xs, size_t m
  * aq[k][eff] / ad[k][eff/32] (quantised silu(g)*u).  Any of them may be NULL. */
 int smx_moe_ffn_stages(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                        const float* x, size_t x_len, float* y, float* gu, int8_t* aq, float* ad);
+/* smx_moe_layer (decode.rs:1608-1739) with the stages of its grouped path copied out per slot:
+ * gu[slots][2][eff] (gate, up outputs of the slot's expert: after gather_xq8 + the two GEMMs),
+ * aq[slots][eff] / ad[slots][eff/32] (silu_quant_rows), dy[slots][hidden] (the down GEMM, before
+ * scatter_add_w).  Any of them may be NULL. */
+int smx_moe_layer_stages(smx_ctx* ctx, size_t layer, const float* xs, size_t m, const size_t* plan,
+                         size_t nplan, const int32_t* slot_tok, const float* wslot, size_t slots,
+                         float* y, size_t y_cap, float* gu, int8_t* aq, float* ad, float* dy);
 
 #ifdef __cplusplus
 }

@@ -35,6 +35,7 @@ EXPORTS = [
     "smx_upload_moe_q6", "smx_gguf_open", "smx_gguf_close", "smx_gguf_tensor_count", "smx_gguf_tensor",
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
+    "smx_weight_dims", "smx_moe_layer_stages",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -83,6 +84,8 @@ def load_library():
     L.smx_moe_ffn.argtypes = [vp, sz, vp, vp, sz, vp, sz, C.c_float, vp, sz]
     L.smx_moe_layer.argtypes = [vp, sz, vp, sz, vp, sz, vp, vp, sz, vp, sz]
     L.smx_moe_layer_dev.argtypes = [vp, sz, vp, sz, vp, sz, vp, vp, sz, vp]
+    L.smx_moe_layer_stages.argtypes = [vp, sz, vp, sz, vp, sz, vp, vp, sz, vp, sz, vp, vp, vp, vp]
+    L.smx_weight_dims.argtypes = [vp, cp, C.POINTER(sz), C.POINTER(sz)]
     L.smx_dev_alloc.argtypes = [vp, sz, C.POINTER(vp)]
     L.smx_dev_free.argtypes = [vp, vp]
     L.smx_h2d.argtypes = [vp, vp, vp, sz]
@@ -316,6 +319,12 @@ class Mi355WeightAccel:
     def evict(self, key):
         return self._check(self._L.smx_evict(self._h, key.encode()))
 
+    def weight_dims(self, key):
+        """(in_dim, out_dim) of a resident weight, or None."""
+        i, o = C.c_size_t(), C.c_size_t()
+        ok = self._check(self._L.smx_weight_dims(self._h, key.encode(), C.byref(i), C.byref(o)))
+        return (i.value, o.value) if ok else None
+
     def gemv(self, key, x, out_dim):
         x = _c(x, np.float32).reshape(-1)
         y = np.empty(out_dim, np.float32)
@@ -439,6 +448,22 @@ class Mi355WeightAccel:
         ok = self._check(self._L.smx_moe_ffn_stages(self._h, layer, _p(ids), _p(wexp), k, _p(x), x.size,
                                                     _p(y), _p(gu), _p(aq), _p(ad)))
         return (y, gu, aq, ad) if ok else None
+
+    def moe_layer_stages(self, layer, xs, m, plan, slot_tok, wslot, eff):
+        """moe_layer_q8_dev with the per-slot stages: (y, gu[slots][2][eff], aq, ad, dy[slots][hidden])."""
+        xs = _c(xs, np.float32).reshape(m, -1)
+        hidden = xs.shape[1]
+        plan = _c(plan, np.uint64).reshape(-1, 3)
+        slot_tok, wslot = _c(slot_tok, np.int32), _c(wslot, np.float32)
+        slots = slot_tok.size
+        y = np.empty_like(xs)
+        gu = np.empty((slots, 2, eff), np.float32)
+        aq = np.empty((slots, eff), np.int8)
+        ad = np.empty((slots, eff // 32), np.float32)
+        dy = np.empty((slots, hidden), np.float32)
+        ok = self._check(self._L.smx_moe_layer_stages(self._h, layer, _p(xs), m, _p(plan), plan.shape[0], _p(slot_tok),
+                                                      _p(wslot), slots, _p(y), y.size, _p(gu), _p(aq), _p(ad), _p(dy)))
+        return (y, gu, aq, ad, dy) if ok else None
 
     # -- device-resident + timing (used by the benchmark)
     def dev_alloc(self, nbytes):

@@ -122,6 +122,7 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
                    float* const* ys, const size_t* out_caps, int* status) {
     if (!c) return SMX_ERR_ARG;
     if (!keys || !xs || !in_lens || !ys || !out_caps || !status) return fail(c, SMX_ERR_ARG, "gemv_batch: null argument");
+    return guarded(c, "gemv_batch", [&]() -> int {
     SMX_HIP(c, hipSetDevice(c->device));
     // Pass 1: validate and size one scratch region per item so the whole batch is one device job.
     std::vector<const Weight*> ws(n, nullptr);
@@ -202,6 +203,7 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
         for (size_t i = 0; i < n; i++)
             if (ws[i] && status[i] == SMX_OK) memcpy(ys[i], c->hy.p + yoff[i], ws[i]->N * 4);
     return SMX_OK;
+    });
 }
 
 int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, uint32_t* out) {

@@ -29,8 +29,7 @@ int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
         return fail(c, SMX_ERR_ARG, "scratch would grow to %zu bytes during graph capture: run the call once outside capture first", bytes);
     if (b.p) {
         SMX_HIP(c, hipStreamSynchronize(c->stream));
-        if (c->live_graphs > 0) c->retired.push_back(b.p);  // a graph may still name this buffer
-        else SMX_HIP(c, hipFree(b.p));
+        release_device(c, b.p);
         b.p = nullptr;
         b.cap = 0;
     }
@@ -43,6 +42,20 @@ int ensure(smx_ctx* c, DevBuf& b, size_t bytes) {
     }
     b.cap = cap;
     return SMX_OK;
+}
+
+void release_device(smx_ctx* c, char* p) {
+    if (!p) return;
+    if (c->live_graphs > 0) {
+        try {
+            c->retired.push_back(p);  // a graph may still name this allocation
+            return;
+        } catch (const std::bad_alloc&) {
+            // cannot record it: leak rather than free memory a replay may read
+            return;
+        }
+    }
+    (void)hipFree(p);
 }
 
 int ensure_host(smx_ctx* c, DevBuf& b, size_t bytes) {
@@ -85,8 +98,14 @@ ProfScope::~ProfScope() {
 
 static size_t align256(size_t x) { return (x + 255) & ~size_t(255); }
 
+// at context teardown (no graph can run any more)
 static void free_weight(Weight& w) {
     if (w.base) (void)hipFree(w.base);
+    w.base = nullptr;
+}
+// while the context lives: a captured graph may hold the weight's plane pointers
+static void drop_weight(smx_ctx* c, Weight& w) {
+    release_device(c, w.base);
     w.base = nullptr;
 }
 
@@ -172,15 +191,22 @@ static int upload(smx_ctx* c, QType type, const char* key, const void* bytes, si
     Weight w;
     int rc = build_weight(c, type, (const uint8_t*)bytes, nbytes, K, N, &w);
     if (rc != SMX_OK) return rc;
-    auto it = c->weights.find(key);
-    if (it != c->weights.end()) {
-        (void)hipStreamSynchronize(c->stream);
-        free_weight(it->second);
-        it->second = w;
-    } else {
-        c->weights.emplace(key, w);
-    }
-    return SMX_OK;
+    return guarded(c, "upload", [&]() -> int {
+        auto it = c->weights.find(key);
+        if (it != c->weights.end()) {
+            (void)hipStreamSynchronize(c->stream);
+            drop_weight(c, it->second);
+            it->second = w;
+        } else {
+            try {
+                c->weights.emplace(key, w);
+            } catch (...) {
+                free_weight(w);
+                throw;
+            }
+        }
+        return SMX_OK;
+    });
 }
 
 }  // namespace smx
@@ -308,17 +334,26 @@ static int upload_moe(smx_ctx* c, QType type, const char* who, size_t layer, con
         free_weight(L.up);
         return rc;
     }
-    auto it = c->moe.find(layer);
-    if (it != c->moe.end()) {
-        (void)hipStreamSynchronize(c->stream);
-        free_weight(it->second.gate);
-        free_weight(it->second.up);
-        free_weight(it->second.down);
-        it->second = L;
-    } else {
-        c->moe.emplace(layer, L);
-    }
-    return SMX_OK;
+    return guarded(c, who, [&]() -> int {
+        auto it = c->moe.find(layer);
+        if (it != c->moe.end()) {
+            (void)hipStreamSynchronize(c->stream);
+            drop_weight(c, it->second.gate);
+            drop_weight(c, it->second.up);
+            drop_weight(c, it->second.down);
+            it->second = L;
+        } else {
+            try {
+                c->moe.emplace(layer, L);
+            } catch (...) {
+                free_weight(L.gate);
+                free_weight(L.up);
+                free_weight(L.down);
+                throw;
+            }
+        }
+        return SMX_OK;
+    });
 }
 
 int smx_upload_moe_q8(smx_ctx* c, size_t layer, const void* gate, size_t gate_n, const void* up, size_t up_n,
@@ -333,12 +368,25 @@ int smx_upload_moe_q6(smx_ctx* c, size_t layer, const void* gate, size_t gate_n,
 
 int smx_evict(smx_ctx* c, const char* key) {
     if (!c || !key) return SMX_ERR_ARG;
-    auto it = c->weights.find(key);
-    if (it == c->weights.end()) return SMX_NOT_RESIDENT;
-    SMX_HIP(c, hipStreamSynchronize(c->stream));
-    free_weight(it->second);
-    c->weights.erase(it);
-    return SMX_OK;
+    return guarded(c, "evict", [&]() -> int {
+        auto it = c->weights.find(key);
+        if (it == c->weights.end()) return SMX_NOT_RESIDENT;
+        SMX_HIP(c, hipStreamSynchronize(c->stream));
+        drop_weight(c, it->second);   // kept until the context closes while a captured graph may name it
+        c->weights.erase(it);
+        return SMX_OK;
+    });
+}
+
+int smx_weight_dims(const smx_ctx* c, const char* key, size_t* in_dim, size_t* out_dim) {
+    if (!c || !key) return SMX_ERR_ARG;
+    for (const auto& kv : c->weights)   // no temporary std::string: this call allocates nothing
+        if (kv.first == key) {
+            if (in_dim) *in_dim = kv.second.K;
+            if (out_dim) *out_dim = kv.second.N;
+            return SMX_OK;
+        }
+    return SMX_NOT_RESIDENT;
 }
 
 int smx_dev_alloc(smx_ctx* c, size_t nbytes, void** dptr) {
@@ -442,15 +490,9 @@ int smx_tune(smx_ctx* c, const char* knob, int value) {
     } else if (k == "gemv_wpc") {
         if (value > 32) return fail(c, SMX_ERR_ARG, "tune: gemv_wpc must be 0..32");
         c->tune_gemv_wpc = value;
-    } else if (k == "gemv_flat") {
-        if (value > 1) return fail(c, SMX_ERR_ARG, "tune: gemv_flat must be 0 (automatic) or 1 (never)");
-        c->tune_gemv_flat = value;
     } else if (k == "gemm_splitk") {
         if (value > 16) return fail(c, SMX_ERR_ARG, "tune: gemm_splitk must be 0..16");
         c->tune_gemm_splitk = value;
-    } else if (k == "gemm_nw") {
-        if (value != 0 && value != 4 && value != 8) return fail(c, SMX_ERR_ARG, "tune: gemm_nw must be 0, 4 or 8");
-        c->tune_gemm_nw = value;
     } else {
         return fail(c, SMX_ERR_ARG, "tune: unknown knob %s", knob);
     }

@@ -466,9 +466,8 @@ static int pick_splitk(int slots, int tiles, int nstages) {
 template <int FMT, bool DUMP, int NW>
 static int launch_gemm_variant(smx_ctx* c, const GemmArgs& p, dim3 grid) {
     auto k = gemm_i8_kernel<FMT, DUMP, NW>;
-    static size_t lds_set = 0;
     const size_t lds = 2 * stage_bytes(NW, FMT == FMT_Q6);
-    int rc = set_dyn_lds(c, k, lds, &lds_set);
+    int rc = set_dyn_lds(c, k, lds);
     if (rc != SMX_OK) return rc;
     hipLaunchKernelGGL(k, grid, dim3(64 * NW), lds, c->stream, p);
     SMX_HIP(c, hipGetLastError());
@@ -501,16 +500,15 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     p.N = (int)w.N;
     p.ldo = (int)w.N;
     p.nb = (int)(w.K / 32);
-    // 128 x 128 tiles, two workgroups per CU; 256 x 128 (one 8-wave workgroup per CU) measures slower
-    int nw = 4;
-    if (w.type != kQ6_K && (c->tune_gemm_nw == 4 || c->tune_gemm_nw == 8)) nw = c->tune_gemm_nw;
+    // 128 x 128 tiles, two workgroups per CU (256 x 128 with one 8-wave workgroup per CU measured 7 % slower)
+    constexpr int nw = 4;
     const int bm = 32 * nw;
     p.tiles_m = (p.M + bm - 1) / bm;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int T = p.tiles_m * p.tiles_n;
     p.xcd_remap = (T % 8 == 0) ? 1 : 0;
     const int nstages = (p.nb + KB - 1) / KB;
-    const int slots = c->num_cu * (nw == 8 ? 1 : 2);
+    const int slots = c->num_cu * 2;
     int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(slots, T, nstages));
     p.stages_per_slice = (nstages + Z - 1) / Z;
     Z = (nstages + p.stages_per_slice - 1) / p.stages_per_slice;
@@ -527,11 +525,9 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
         if (w.type == kQ6_K) {
             rc = dump ? launch_gemm_variant<FMT_Q6, true, 4>(c, p, grid) : launch_gemm_variant<FMT_Q6, false, 4>(c, p, grid);
         } else if (w.type == kQ4_0) {
-            if (dump) rc = nw == 8 ? launch_gemm_variant<FMT_Q4, true, 8>(c, p, grid) : launch_gemm_variant<FMT_Q4, true, 4>(c, p, grid);
-            else rc = nw == 8 ? launch_gemm_variant<FMT_Q4, false, 8>(c, p, grid) : launch_gemm_variant<FMT_Q4, false, 4>(c, p, grid);
+            rc = dump ? launch_gemm_variant<FMT_Q4, true, 4>(c, p, grid) : launch_gemm_variant<FMT_Q4, false, 4>(c, p, grid);
         } else {
-            if (dump) rc = nw == 8 ? launch_gemm_variant<FMT_Q8, true, 8>(c, p, grid) : launch_gemm_variant<FMT_Q8, true, 4>(c, p, grid);
-            else rc = nw == 8 ? launch_gemm_variant<FMT_Q8, false, 8>(c, p, grid) : launch_gemm_variant<FMT_Q8, false, 4>(c, p, grid);
+            rc = dump ? launch_gemm_variant<FMT_Q8, true, 4>(c, p, grid) : launch_gemm_variant<FMT_Q8, false, 4>(c, p, grid);
         }
         if (rc != SMX_OK) return rc;
     }

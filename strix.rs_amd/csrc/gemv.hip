@@ -42,10 +42,13 @@ __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, in
 }
 
 // Flat form (one activation row): blockIdx.x of gridDim.x workgroups share a job's rows.
-template <class Ops, int MT, int PRE, int GL, int FQ>
-__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, int m, unsigned magic_u) {
+// DUMP: the per-block i32 dots of job 0 are also written to dump[row * dump_per_row + ...].
+template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP>
+__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, int m, unsigned magic_u,
+                                                         int* __restrict__ dump, int dump_per_row) {
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body_flat<Ops, MT, PRE, GL, FQ>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u);
+    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u,
+                                               dump, dump_per_row);
 }
 
 namespace {
@@ -67,8 +70,7 @@ struct Geom {
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT>
 int launch_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump, int dump_per_row) {
     auto k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP, NT>;
-    static size_t lds_set = 0;
-    int rc = set_dyn_lds(c, k, g.lds, &lds_set);
+    int rc = set_dyn_lds(c, k, g.lds);
     if (rc != SMX_OK) return rc;
     hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(NT), g.lds, c->stream, J, nblk, m, dump, dump_per_row);
     SMX_HIP(c, hipGetLastError());
@@ -86,26 +88,28 @@ int launch_one(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk
     return launch_fq<Ops, MT, RPW, PRE, KS, LPR, MT == 1 ? 1 : 0, DUMP, NT>(c, g, J, njobs, nblk, m, dump, dump_per_row);
 }
 
-template <class Ops, int MT, int PRE, int GL, int FQ>
-int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m) {
-    auto k = gemv_flat_kernel<Ops, MT, PRE, GL, FQ>;
-    static size_t lds_set = 0;
-    int rc = set_dyn_lds(c, k, g.lds, &lds_set);
+template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP = false>
+int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump = nullptr,
+                   int dump_per_row = 0) {
+    auto k = gemv_flat_kernel<Ops, MT, PRE, GL, FQ, DUMP>;
+    int rc = set_dyn_lds(c, k, g.lds);
     if (rc != SMX_OK) return rc;
     const unsigned upb = std::is_same<Ops, OpsQ6_K>::value ? 4u : (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u);
     const unsigned units = (unsigned)nblk * upb;                             // units per row
     const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);   // floor(f * magic / 2^32) = f / units for f < 2^16
-    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, m, magic);
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, m, magic, dump, dump_per_row);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
 
 template <class Ops, int MT>
-int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m) {
+int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump = nullptr,
+                int dump_per_row = 0) {
     constexpr bool kQ6 = std::is_same<Ops, OpsQ6_K>::value;
     if constexpr (MT == 1) {
 #define SMX_FLAT(PRE, GL)                                                                            \
     if (g.flat_pre == PRE && g.flat == GL) {                                                         \
+        if (dump) return launch_flat_fq<Ops, 1, PRE, GL, 1, true>(c, g, J, njobs, nblk, m, dump, dump_per_row); \
         if (g.preq) return launch_flat_fq<Ops, 1, PRE, GL, 0>(c, g, J, njobs, nblk, m);              \
         if (g.prod) return launch_flat_fq<Ops, 1, PRE, GL, 2>(c, g, J, njobs, nblk, m);              \
         return launch_flat_fq<Ops, 1, PRE, GL, 1>(c, g, J, njobs, nblk, m);                          \
@@ -160,6 +164,7 @@ int launch_variant(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
 template <class Ops>
 int launch_type(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int mt,
                 int* dump, int dump_per_row) {
+    if (dump && g.flat) return launch_flat<Ops, 1>(c, g, J, njobs, nblk, m, dump, dump_per_row);
     if (dump) {
         if (g.lpr == 16) return launch_one<Ops, 1, 1, 2, 1, 16, true, 256>(c, g, J, njobs, nblk, m, dump, dump_per_row);
         return launch_one<Ops, 1, 1, 4, 1, 64, true, 256>(c, g, J, njobs, nblk, m, dump, dump_per_row);
@@ -244,9 +249,8 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
     // Flat form: one activation row of up to 16384 elements and rows of a whole number of unit groups.
     // Measured against the persistent form above: Q4_0 9728 x 2560 6.8 -> 5.4 us, eight of them in one
     // launch 24.8 -> 22.4 us, Q6_K 262144 x 3840 159 -> 144 us.
-    // (a sweep that sets one of the persistent form's knobs gets the persistent form)
-    const bool knobs = c->tune_gemv_rpw > 0 || c->tune_gemv_ks > 0 || c->tune_gemv_lpr > 0 || c->tune_gemv_wpc > 0;
-    if (!dump && !knobs && c->tune_gemv_flat != 1 && !(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
+    // The block-dot dump of the parity tests runs in whichever form the shape gets.
+    if (!(type == kQ6_K && mt == 8) && (units % (type == kQ6_K ? 4 : 8)) == 0 &&
         nblk * (type == kQ6_K ? 256 : 32) <= 16384) {  // the row is held in registers while the weights are requested
         // a workgroup's units are indexed with 16 bits and its group sums live in LDS: whole further
         // rounds of workgroups when a CU's share of the rows is too large for either

@@ -718,10 +718,15 @@ struct FlatXRows {
 // first round, after its weight loads are out.
 //
 // MT > 1: m <= MT pre-quantised activation rows (FQ = 0) share every weight load; y[t * ldy + row].
-template <class Ops, int MT, int PRE, int GL, int FQ>
+//
+// DUMP (one activation row): every unit also writes its exact integer block dot(s) to
+// dump[row * dump_per_row + ...], the same integers that enter the fp32 combination.
+template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP = false>
 __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, float* __restrict__ y, int ldy, int nblk,
-                                               int N, int m, int wg, int n_wgs, unsigned magic_u) {
+                                               int N, int m, int wg, int n_wgs, unsigned magic_u,
+                                               int* __restrict__ dump = nullptr, int dump_per_row = 0) {
     static_assert(MT == 1 || FQ == 0, "several activation rows are staged from quantised rows");
+    static_assert(!DUMP || MT == 1, "the block-dot dump covers one activation row");
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int U = Ops::units_per_row(nblk);
@@ -758,11 +763,13 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
                 const int fl = c_t * 64 + lane;
                 const bool act = fl < nunits;
                 const int flc = act ? fl : nunits - 1;
-                const int u = flc - (int)__umulhi((unsigned)flc, magic_u) * U;   // flc mod U
+                const int rl = (int)__umulhi((unsigned)flc, magic_u);            // flc / U: row within the workgroup
+                const int u = flc - rl * U;                                      // flc mod U
                 float acc[MT];
 #pragma unroll
                 for (int t = 0; t < MT; t++) acc[t] = 0.f;
-                compute_unit<MT, false>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, nullptr);
+                int* drow = (DUMP && dump) ? dump + (size_t)(r0 + rl) * dump_per_row : nullptr;
+                compute_unit<MT, DUMP>(Ops(), ring[k], smem, tokb, nblk, u, act, acc, drow);
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const float s = small_group_sum<GL>(acc[t]);

@@ -225,6 +225,7 @@ int smx_gguf_open(const char* path, smx_gguf** out, char* err, size_t err_cap) {
     g->fd = fd;
     g->map = (const uint8_t*)map;
     g->len = (size_t)st.st_size;
+    try {
     auto bail = [&](int code, const char* what) {
         const int rc = set_err(err, err_cap, code, "gguf_open: %s: %s", path, what);
         smx_gguf_close(g);
@@ -260,6 +261,7 @@ int smx_gguf_open(const char* path, smx_gguf** out, char* err, size_t err_cap) {
         if (!c.ok) return bail(SMX_ERR_ARG, "truncated tensor index");
         const BlockFormat* f = format_of(t.type);
         if (!f) return bail(SMX_ERR_LIMIT, "unknown tensor encoding");
+        if (numel / f->elems > SIZE_MAX / f->bytes) return bail(SMX_ERR_ARG, "tensor size overflows");
         t.nbytes = (size_t)(numel / f->elems) * f->bytes;  // gguf.rs:223
         g->index[t.name] = g->tensors.size();
         g->tensors.push_back(std::move(t));
@@ -274,6 +276,13 @@ int smx_gguf_open(const char* path, smx_gguf** out, char* err, size_t err_cap) {
     for (const smx_gguf::Tensor& t : g->tensors)
         if (t.offset > g->len - g->data_offset || t.nbytes > g->len - g->data_offset - t.offset)
             return bail(SMX_ERR_ARG, "a tensor's data lies past the end of the file");  // gguf.rs:225-231
+    } catch (const std::bad_alloc&) {   // a crafted count or string length: no exception crosses the C ABI
+        smx_gguf_close(g);
+        return set_err(err, err_cap, SMX_ERR_NOMEM, "gguf_open: %s: out of host memory while reading the index", path);
+    } catch (const std::exception& e) {
+        smx_gguf_close(g);
+        return set_err(err, err_cap, SMX_ERR_ARG, "gguf_open: %s: %s", path, e.what());
+    }
     *out = g;
     return SMX_OK;
 }
@@ -344,6 +353,7 @@ int smx_gguf_meta_str(const smx_gguf* g, const char* key, const char** value) {
 int smx_gguf_attach(smx_ctx* c, const smx_gguf* g, size_t* n_weights, size_t* n_expert_layers) {
     if (!c) return SMX_ERR_ARG;
     if (!g) return smx::fail(c, SMX_ERR_ARG, "gguf_attach: null file");
+    return smx::guarded(c, "gguf_attach", [&]() -> int {
     size_t nw = 0, nl = 0;
     for (const smx_gguf::Tensor& t : g->tensors) {
         if (t.dims.size() < 2 || !ends_with(t.name, ".weight") || ends_with(t.name, "_exps.weight")) continue;
@@ -384,6 +394,7 @@ int smx_gguf_attach(smx_ctx* c, const smx_gguf* g, size_t* n_weights, size_t* n_
     if (n_weights) *n_weights = nw;
     if (n_expert_layers) *n_expert_layers = nl;
     return SMX_OK;
+    });
 }
 
 // One tensor re-encoded on the host and uploaded: the reference's repacks of a tensor whose encoding
@@ -395,6 +406,7 @@ int smx_gguf_upload_as(smx_ctx* c, const smx_gguf* g, const char* tensor, const 
     if (!g || !tensor) return smx::fail(c, SMX_ERR_ARG, "gguf_upload_as: null argument");
     if (target_type != 2 && target_type != 8)
         return smx::fail(c, SMX_ERR_ARG, "gguf_upload_as: target type %d (2 = Q4_0 or 8 = Q8_0)", target_type);
+    return smx::guarded(c, "gguf_upload_as", [&]() -> int {
     auto it = g->index.find(tensor);
     if (it == g->index.end()) return SMX_NOT_RESIDENT;
     const smx_gguf::Tensor& t = g->tensors[it->second];
@@ -424,6 +436,7 @@ int smx_gguf_upload_as(smx_ctx* c, const smx_gguf* g, const char* tensor, const 
     }
     return target_type == 2 ? smx_upload_q4_0(c, name, enc.data(), enc.size(), in_dim, out_dim)
                             : smx_upload_q8_0(c, name, enc.data(), enc.size(), in_dim, out_dim);
+    });
 }
 
 // ---- host quantisers / dequantisers (n a multiple of the block size) ----

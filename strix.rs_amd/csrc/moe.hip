@@ -476,10 +476,10 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
         const size_t frows = (hidden + fgrid - 1) / fgrid;
         const int gl = upe % 16 == 0 ? 16 : (upe % 8 == 0 ? 8 : (upe % 4 == 0 ? 4 : 2));
         const size_t flds = lds + frows * units / gl * 4;
-        if (c->tune_gemv_flat != 1 && k * eff <= 4 * 1024 * 4 && frows * units < 65536 && flds <= 160 * 1024) {
+        if (k * eff <= 4 * 1024 * 4 && frows * units < 65536 && flds <= 160 * 1024) {
             const unsigned m_units = (unsigned)(((1ull << 32) + units - 1) / units), m_upe = (unsigned)(((1ull << 32) + upe - 1) / upe);
-            auto launch = [&](auto kern, size_t* lds_set) -> int {
-                int rc2 = set_dyn_lds(c, kern, flds, lds_set);
+            auto launch = [&](auto kern) -> int {
+                int rc2 = set_dyn_lds(c, kern, flds);
                 if (rc2 != SMX_OK) return rc2;
                 hipLaunchKernelGGL(kern, dim3((unsigned)fgrid), dim3(1024), flds, c->stream, s.g, s.u, L.down.scales,
                                    (const uint4*)L.down.quants, route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad,
@@ -487,16 +487,14 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
                 SMX_HIP(c, hipGetLastError());
                 return SMX_OK;
             };
-            static size_t set16 = 0, set8 = 0, set4 = 0, set2 = 0;
-            if (gl == 16) rc = launch(moe_down_flat_kernel<16>, &set16);
-            else if (gl == 8) rc = launch(moe_down_flat_kernel<8>, &set8);
-            else if (gl == 4) rc = launch(moe_down_flat_kernel<4>, &set4);
-            else rc = launch(moe_down_flat_kernel<2>, &set2);
+            if (gl == 16) rc = launch(moe_down_flat_kernel<16>);
+            else if (gl == 8) rc = launch(moe_down_flat_kernel<8>);
+            else if (gl == 4) rc = launch(moe_down_flat_kernel<4>);
+            else rc = launch(moe_down_flat_kernel<2>);
             if (rc != SMX_OK) return rc;
         } else {
             auto kern = moe_down_fused_kernel<6>;
-            static size_t lds_set = 0;
-            if ((rc = set_dyn_lds(c, kern, lds, &lds_set)) != SMX_OK) return rc;
+            if ((rc = set_dyn_lds(c, kern, lds)) != SMX_OK) return rc;
             const unsigned grid = (unsigned)std::min<size_t>((hidden + 7) / 8, (size_t)c->num_cu * 2);
             hipLaunchKernelGGL(kern, dim3(grid), dim3(1024), lds, c->stream, s.g, s.u, L.down.scales, (const uint4*)L.down.quants,
                                route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad);
@@ -561,6 +559,7 @@ static int moe_ffn_host(smx_ctx* c, size_t layer, const int32_t* ids, const floa
                         size_t x_len, float sgate, float* y, size_t y_cap, float* gu, int8_t* aq, float* ad) {
     if (!c) return SMX_ERR_ARG;
     if (!ids || !wexp || !x || !y) return fail(c, SMX_ERR_ARG, "moe_ffn: null argument");
+    return guarded(c, "moe_ffn", [&]() -> int {
     auto it = c->moe.find(layer);
     if (it == c->moe.end()) return SMX_NOT_RESIDENT;
     const MoeLayer& L = it->second;
@@ -592,6 +591,7 @@ static int moe_ffn_host(smx_ctx* c, size_t layer, const int32_t* ids, const floa
     if (ad) SMX_HIP(c, hipMemcpyAsync(ad, s.ad, k * (L.eff / 32) * 4, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
     return SMX_OK;
+    });
 }
 
 // Tile table of one grouped GEMM stage: for every plan entry, ceil(cnt/128) x ceil(rows/128) tiles.
@@ -632,25 +632,35 @@ int smx_moe_ffn_dev(smx_ctx* c, size_t layer, const int32_t* ids, const float* w
                     float* y_dev) {
     if (!c) return SMX_ERR_ARG;
     if (!ids || !wexp || !x_dev || !y_dev) return fail(c, SMX_ERR_ARG, "moe_ffn_dev: null argument");
-    auto it = c->moe.find(layer);
-    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
-    return moe_ffn_enqueue(c, it->second, ids, wexp, k, x_dev, y_dev, nullptr);
+    return guarded(c, "moe_ffn_dev", [&]() -> int {
+        auto it = c->moe.find(layer);
+        if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+        return moe_ffn_enqueue(c, it->second, ids, wexp, k, x_dev, y_dev, nullptr);
+    });
 }
 
 int smx_moe_shexp_dev(smx_ctx* c, size_t layer, float sgate, const float* x_dev, float* y_dev) {
     if (!c) return SMX_ERR_ARG;
     if (!x_dev || !y_dev) return fail(c, SMX_ERR_ARG, "moe_shexp_dev: null argument");
-    auto it = c->moe.find(layer);
-    if (it == c->moe.end()) return SMX_NOT_RESIDENT;
-    return shexp_enqueue(c, layer, it->second.hidden, sgate, x_dev, y_dev);
+    return guarded(c, "moe_shexp_dev", [&]() -> int {
+        auto it = c->moe.find(layer);
+        if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+        return shexp_enqueue(c, layer, it->second.hidden, sgate, x_dev, y_dev);
+    });
 }
 
 // The grouped expert FFN over a slot table: quantise the m activation rows, gate and up of every
 // expert group in one GEMM launch (slot s reads activation row rowmap[s], or row s when rowmap is
 // null), silu(g)*u re-quantised, down in a second GEMM launch.  dy[slots][hidden] is left in c->work.
 // The two tile tables (device pointers) are those of build_tiles over the plan for eff and hidden rows.
+struct SlotScratch {
+    float *g, *u;   // [slots][eff] gate and up outputs
+    int8_t* aq;     // [slots][eff] quantised silu(g)*u
+    float* ad;      // [slots][eff/32]
+    float* dy;      // [slots][hidden] unweighted down outputs
+};
 static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const float* x_dev, size_t m, const int* rowmap_dev, size_t slots,
-                             const GemmTile* tiles_gu, size_t n_gu, const GemmTile* tiles_dn, size_t n_dn, float** dy_out) {
+                             const GemmTile* tiles_gu, size_t n_gu, const GemmTile* tiles_dn, size_t n_dn, SlotScratch* out) {
     const size_t hidden = L.hidden, eff = L.eff, nb = hidden / 32, enb = eff / 32;
     int rc;
     if ((rc = ensure(c, c->xq, m * hidden)) != SMX_OK) return rc;
@@ -700,9 +710,17 @@ static int moe_slots_enqueue(smx_ctx* c, const MoeLayer& L, const float* x_dev, 
         rc = launch_gemm_grouped(c, L.type, p, (int)n_dn, 1, "moe_gemm_down");
         if (rc != SMX_OK) return rc;
     }
-    *dy_out = dy;
+    *out = SlotScratch{g, u, aq, ad, dy};
     return SMX_OK;
 }
+
+// Host destinations of the stage-by-stage copy-out of a grouped layer call (any may be null).
+struct LayerStagesOut {
+    float* gu;    // [slots][2][eff]
+    int8_t* aq;   // [slots][eff]
+    float* ad;    // [slots][eff/32]
+    float* dy;    // [slots][hidden]
+};
 
 // The small tables of one call, packed on the host (256-byte aligned parts) and sent to c->tab in
 // ONE copy: six separate uploads cost about 4 us each.
@@ -739,9 +757,10 @@ static int moe_check_shape(smx_ctx* c, const MoeLayer& L, size_t m, size_t slots
 // xs / y on the host (copied in and out, one sync) or, with on_device, device pointers (enqueue only).
 static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
                           const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap,
-                          bool on_device) {
+                          bool on_device, const LayerStagesOut* stages = nullptr) {
     if (!c) return SMX_ERR_ARG;
     if (!xs || !plan || !slot_tok || !wslot || !y) return fail(c, SMX_ERR_ARG, "moe_layer: null argument");
+    return guarded(c, "moe_layer", [&]() -> int {
     auto it = c->moe.find(layer);
     if (it == c->moe.end()) return SMX_NOT_RESIDENT;
     const MoeLayer& L = it->second;
@@ -787,10 +806,11 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
                  o_t2 = tb.add(tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile));
     if (!on_device) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * hidden * 4, hipMemcpyHostToDevice, c->stream));
     if ((rc = tb.upload(c)) != SMX_OK) return rc;
-    float* dy = nullptr;
+    SlotScratch ss;
     rc = moe_slots_enqueue(c, L, x_dev, m, (const int*)(c->tab.p + o_st), slots, (const GemmTile*)(c->tab.p + o_t1), tiles_gu.size(),
-                           (const GemmTile*)(c->tab.p + o_t2), tiles_dn.size(), &dy);
+                           (const GemmTile*)(c->tab.p + o_t2), tiles_dn.size(), &ss);
     if (rc != SMX_OK) return rc;
+    float* dy = ss.dy;
     {
         ProfScope ps(c, "moe_combine");
         hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((hidden / 4 + 255) / 256), (unsigned)m), dim3(256), 0, c->stream,
@@ -800,9 +820,20 @@ static int moe_layer_impl(smx_ctx* c, size_t layer, const float* xs, size_t m, c
     }
     if (!on_device) {
         SMX_HIP(c, hipMemcpyAsync(y, c->yf32.p, m * hidden * 4, hipMemcpyDeviceToHost, c->stream));
+        if (stages) {
+            const size_t eff = L.eff;
+            if (stages->gu) {   // g and u are separate [slots][eff] planes on the device
+                SMX_HIP(c, hipMemcpy2DAsync(stages->gu, 2 * eff * 4, ss.g, eff * 4, eff * 4, slots, hipMemcpyDeviceToHost, c->stream));
+                SMX_HIP(c, hipMemcpy2DAsync(stages->gu + eff, 2 * eff * 4, ss.u, eff * 4, eff * 4, slots, hipMemcpyDeviceToHost, c->stream));
+            }
+            if (stages->aq) SMX_HIP(c, hipMemcpyAsync(stages->aq, ss.aq, slots * eff, hipMemcpyDeviceToHost, c->stream));
+            if (stages->ad) SMX_HIP(c, hipMemcpyAsync(stages->ad, ss.ad, slots * (eff / 32) * 4, hipMemcpyDeviceToHost, c->stream));
+            if (stages->dy) SMX_HIP(c, hipMemcpyAsync(stages->dy, ss.dy, slots * hidden * 4, hipMemcpyDeviceToHost, c->stream));
+        }
         SMX_HIP(c, hipStreamSynchronize(c->stream));
     }
     return SMX_OK;
+    });
 }
 
 // WeightAccel::moe_layer_ffn (accel.rs:238-246, decode.rs:3552-3629): xs holds the rows of every
@@ -812,6 +843,7 @@ int smx_moe_layer_ffn(smx_ctx* c, size_t layer, const int32_t* plan, size_t npla
                       size_t dy_cap) {
     if (!c) return SMX_ERR_ARG;
     if (!plan || !xs || !dy) return fail(c, SMX_ERR_ARG, "moe_layer_ffn: null argument");
+    return guarded(c, "moe_layer_ffn", [&]() -> int {
     auto it = c->moe.find(layer);
     if (it == c->moe.end()) return SMX_NOT_RESIDENT;
     const MoeLayer& L = it->second;
@@ -840,13 +872,14 @@ int smx_moe_layer_ffn(smx_ctx* c, size_t layer, const int32_t* plan, size_t npla
                  o_t2 = tb.add(tiles_dn.data(), tiles_dn.size() * sizeof(GemmTile));
     if ((rc = tb.upload(c)) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, rows * hidden * 4, hipMemcpyHostToDevice, c->stream));
-    float* dy_dev = nullptr;
+    SlotScratch ss;
     rc = moe_slots_enqueue(c, L, (const float*)c->xf32.p, rows, nullptr, rows, (const GemmTile*)(c->tab.p + o_t1), tiles_gu.size(),
-                           (const GemmTile*)(c->tab.p + o_t2), tiles_dn.size(), &dy_dev);
+                           (const GemmTile*)(c->tab.p + o_t2), tiles_dn.size(), &ss);
     if (rc != SMX_OK) return rc;
-    SMX_HIP(c, hipMemcpyAsync(dy, dy_dev, rows * hidden * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(dy, ss.dy, rows * hidden * 4, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
     return SMX_OK;
+    });
 }
 
 // WeightAccel::moe_expert_ffn (accel.rs:220-223): one expert's FFN for m grouped rows, one sync.
@@ -859,6 +892,13 @@ int smx_moe_expert_ffn(smx_ctx* c, size_t layer, size_t expert, const float* xs,
 int smx_moe_layer(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
                   const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap) {
     return moe_layer_impl(c, layer, xs, m, plan, nplan, slot_tok, wslot, slots, y, y_cap, false);
+}
+
+int smx_moe_layer_stages(smx_ctx* c, size_t layer, const float* xs, size_t m, const size_t* plan, size_t nplan,
+                         const int32_t* slot_tok, const float* wslot, size_t slots, float* y, size_t y_cap, float* gu,
+                         int8_t* aq, float* ad, float* dy) {
+    const LayerStagesOut so = {gu, aq, ad, dy};
+    return moe_layer_impl(c, layer, xs, m, plan, nplan, slot_tok, wslot, slots, y, y_cap, false, &so);
 }
 
 int smx_moe_layer_dev(smx_ctx* c, size_t layer, const float* xs_dev, size_t m, const size_t* plan, size_t nplan,

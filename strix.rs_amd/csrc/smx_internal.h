@@ -5,6 +5,8 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <new>
+#include <stdexcept>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -76,7 +78,10 @@ struct smx_ctx {
     hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
 
     // tuning overrides (0 = automatic)
-    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemv_flat = 0, tune_gemm_splitk = 0, tune_gemm_nw = 0;
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0;
+
+    // dynamic-LDS limit already raised on this context's device, per kernel (see set_dyn_lds)
+    std::unordered_map<const void*, size_t> lds_set;
 
     bool capturing = false;  // between smx_graph_begin and smx_graph_end
     // A captured graph holds the addresses of the scratch buffers its kernels used.  While any graph
@@ -105,18 +110,36 @@ int hip_fail(smx_ctx* c, hipError_t e, const char* what);
         if (e_ != hipSuccess) return ::smx::hip_fail((c), e_, #call);      \
     } while (0)
 
+// No C++ exception may cross the C ABI: entry points that use standard containers run their body
+// through this and report allocation failure as SMX_ERR_NOMEM.
+template <class F>
+int guarded(smx_ctx* c, const char* who, F&& body) {
+    try {
+        return body();
+    } catch (const std::bad_alloc&) {
+        return fail(c, SMX_ERR_NOMEM, "%s: out of host memory", who);
+    } catch (const std::exception& e) {
+        return fail(c, SMX_ERR_ARG, "%s: %s", who, e.what());
+    }
+}
+
 int ensure(smx_ctx* c, DevBuf& b, size_t bytes);
+// Frees a device allocation that kernels of the context may name, or, while a captured graph of the
+// context is alive, keeps it until the context closes (a replay may still read it).
+void release_device(smx_ctx* c, char* p);
 // the same for a pinned host buffer (hipHostMalloc)
 int ensure_host(smx_ctx* c, DevBuf& b, size_t bytes);
 
 // Raises a kernel's dynamic-LDS limit when it asks for more than the 48 KB default (remembered per
-// kernel so that replays and captured launches do not repeat the call).
+// context and kernel so that replays and captured launches do not repeat the call).
 template <typename Kern>
-int set_dyn_lds(smx_ctx* c, Kern kern, size_t lds, size_t* cached) {
-    if (lds <= 48 * 1024 || lds <= *cached) return SMX_OK;
+int set_dyn_lds(smx_ctx* c, Kern kern, size_t lds) {
+    if (lds <= 48 * 1024) return SMX_OK;
+    size_t& cached = c->lds_set[(const void*)kern];
+    if (lds <= cached) return SMX_OK;
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return hip_fail(c, e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-    *cached = lds;
+    cached = lds;
     return SMX_OK;
 }
 

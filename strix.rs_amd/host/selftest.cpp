@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <memory>
+#include <string>
 
 #include "weight_accel.hpp"
 
@@ -30,7 +31,8 @@ int main() {
         raw[b * 34 + 1] = 0x24;  // f16 0.015625
         for (int i = 0; i < 32; i++) raw[b * 34 + 2 + i] = (uint8_t)(int8_t)((int)(lcg(seed) % 255) - 127);
     }
-    if (!acc->adopt(8, "blk.0.attn_q.weight", raw, K, N)) return 1;
+    // uploaded the way the trait does it (upload_q8_0, accel.rs:163), not through a convenience wrapper
+    if (!acc->upload_q8_0("blk.0.attn_q.weight", raw.data(), raw.size(), K, N)) return 1;
     std::vector<float> x(K);
     for (size_t i = 0; i < K; i++) x[i] = 0.5f * std::sin(0.017f * (float)i);
     auto y = acc->gemv("blk.0.attn_q.weight", x);
@@ -68,6 +70,31 @@ int main() {
         for (size_t r = 0; r < N; r++)
             if (std::fabs((*yf)[r] - (*yn)[r]) > 1e-5 * maxref * scale) return 8;
         if (acc->gemv_fused("never.adopted", SMX_ACT_RMSNORM, x, nullptr, 1e-6f)) return 9;
+    }
+    {   // a weight that arrives through a GGUF file (attach_gguf) is served the same way
+        const char* path = "/tmp/strix_selftest.gguf";
+        std::FILE* f = std::fopen(path, "wb");
+        if (!f) return 10;
+        auto put = [&](const void* p, size_t n) { std::fwrite(p, 1, n, f); };
+        auto put_u32 = [&](uint32_t v) { put(&v, 4); };
+        auto put_u64 = [&](uint64_t v) { put(&v, 8); };
+        const std::string tname = "blk.1.attn_q.weight";
+        put_u32(0x46554747u); put_u32(3); put_u64(1); put_u64(0);          // magic, version, 1 tensor, 0 metadata
+        put_u64(tname.size()); put(tname.data(), tname.size());
+        put_u32(2); put_u64(K); put_u64(N); put_u32(8); put_u64(0);       // 2 dims (in_dim first), Q8_0, offset 0
+        long pos = std::ftell(f);
+        for (; pos % 32 != 0; pos++) std::fputc(0, f);                     // data section is 32-byte aligned
+        put(raw.data(), raw.size());
+        std::fclose(f);
+        if (acc->attach_gguf(path) != 1) return 11;
+        std::remove(path);
+        auto yg = acc->gemv(tname, x);
+        if (!yg || yg->size() != N) return 12;
+        for (size_t r = 0; r < N; r++)
+            if ((*yg)[r] != (*y)[r]) return 13;                            // same bytes, same kernel, same result
+        std::vector<std::pair<std::string, const std::vector<float>*>> calls = {{tname, &x}, {"never.adopted", &x}};
+        auto yb = acc->gemv_batch(calls);
+        if (!yb[0] || yb[0]->size() != N || yb[1]) return 14;
     }
     std::printf("selftest ok\n");
     return 0;

@@ -14,7 +14,6 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
-#include <unordered_map>
 #include <utility>
 #include <vector>
 
@@ -118,16 +117,14 @@ class Mi355WeightAccel final : public WeightAccel {
     }
     bool upload_moe_q8(size_t layer, const uint8_t* gate, size_t gate_n, const uint8_t* up, size_t up_n, const uint8_t* down,
                        size_t down_n, size_t hidden, size_t eff, size_t ne) override {
-        hidden_[layer] = hidden;
         return ok(smx_upload_moe_q8(ctx_, layer, gate, gate_n, up, up_n, down, down_n, hidden, eff, ne));
     }
-    // The C ABI writes into caller-provided buffers; out_dim is remembered per key at upload time by
-    // the caller of this class, or supplied through set_out_dim() for weights uploaded elsewhere.
-    void set_out_dim(const std::string& key, size_t out_dim) { out_dim_[key] = out_dim; }
+    // The C ABI writes into caller-provided buffers: results are sized with what the library holds for
+    // the key (smx_weight_dims), however the weight got there (upload_*, attach_gguf, upload_as).
 
     std::optional<std::vector<float>> gemv(const std::string& key, const std::vector<float>& x) override {
         std::vector<float> y(out_of(key));
-        if (!ok(smx_gemv(ctx_, key.c_str(), x.data(), x.size(), y.data(), y.size()))) return std::nullopt;
+        if (!ok(smx_gemv(ctx_, key.c_str(), x.data(), x.size(), y.empty() ? &dummy_ : y.data(), y.size()))) return std::nullopt;
         return y;
     }
     std::vector<std::optional<std::vector<float>>> gemv_batch(
@@ -140,7 +137,7 @@ class Mi355WeightAccel final : public WeightAccel {
         std::vector<size_t> il(n), oc(n);
         std::vector<int> st(n);
         for (size_t i = 0; i < n; i++) {
-            ys[i].resize(out_of(calls[i].first, /*required=*/false));
+            ys[i].resize(out_of(calls[i].first));
             keys[i] = calls[i].first.c_str();
             xs[i] = calls[i].second->data();
             il[i] = calls[i].second->size();
@@ -161,7 +158,7 @@ class Mi355WeightAccel final : public WeightAccel {
     std::optional<std::vector<float>> gemv_fused(const std::string& key, int act, const std::vector<float>& a,
                                                  const std::vector<float>* b, float eps) {
         if (b && b->size() != a.size()) throw BackendError(SMX_ERR_ARG, "gemv_fused: operand lengths differ");
-        std::vector<float> y(out_of(key, /*required=*/false));
+        std::vector<float> y(out_of(key));
         if (!ok(smx_gemv_fused(ctx_, key.c_str(), act, a.data(), b ? b->data() : nullptr, a.size(), eps,
                                y.empty() ? &dummy_ : y.data(), y.size())))
             return std::nullopt;
@@ -170,7 +167,7 @@ class Mi355WeightAccel final : public WeightAccel {
     std::optional<std::vector<float>> prefill_q8_gemm(const std::string& key, const std::vector<float>& xs, size_t m) override {
         if (m == 0) throw BackendError(SMX_ERR_ARG, "prefill_q8_gemm: m == 0");
         std::vector<float> y(m * out_of(key));
-        if (!ok(smx_gemm(ctx_, key.c_str(), xs.data(), m, xs.size() / m, y.data(), y.size()))) return std::nullopt;
+        if (!ok(smx_gemm(ctx_, key.c_str(), xs.data(), m, xs.size() / m, y.empty() ? &dummy_ : y.data(), y.size()))) return std::nullopt;
         return y;
     }
     std::optional<std::vector<uint32_t>> lm_head_argmax_rows(const std::string& key, const std::vector<float>& xs, size_t m) override {
@@ -209,14 +206,12 @@ class Mi355WeightAccel final : public WeightAccel {
     std::string name() const override { return smx_name(ctx_); }
     smx_ctx* raw() { return ctx_; }
 
-    // convenience: upload and remember out_dim in one call
+    // convenience: upload by GGML type number
     bool adopt(int ggml_type, const std::string& key, const std::vector<uint8_t>& bytes, size_t in_dim, size_t out_dim) {
-        bool r = false;
-        if (ggml_type == 2) r = upload_q4_0(key, bytes.data(), bytes.size(), in_dim, out_dim);
-        else if (ggml_type == 8) r = upload_q8_0(key, bytes.data(), bytes.size(), in_dim, out_dim);
-        else if (ggml_type == 14) r = upload_q6_k(key, bytes.data(), bytes.size(), in_dim, out_dim);
-        if (r) out_dim_[key] = out_dim;
-        return r;
+        if (ggml_type == 2) return upload_q4_0(key, bytes.data(), bytes.size(), in_dim, out_dim);
+        if (ggml_type == 8) return upload_q8_0(key, bytes.data(), bytes.size(), in_dim, out_dim);
+        if (ggml_type == 14) return upload_q6_k(key, bytes.data(), bytes.size(), in_dim, out_dim);
+        return false;
     }
 
   private:
@@ -224,15 +219,12 @@ class Mi355WeightAccel final : public WeightAccel {
         if (rc < 0) throw BackendError(rc, smx_last_error(ctx_));
         return rc == SMX_OK;
     }
-    size_t out_of(const std::string& key, bool required = true) const {
-        auto it = out_dim_.find(key);
-        if (it != out_dim_.end()) return it->second;
-        if (required) return 0;  // unknown key: the library answers "not resident"
-        return 0;
+    // out_dim of a resident weight; 0 for an unknown key (the library then answers "not resident")
+    size_t out_of(const std::string& key) const {
+        size_t out_dim = 0;
+        return smx_weight_dims(ctx_, key.c_str(), nullptr, &out_dim) == SMX_OK ? out_dim : 0;
     }
     smx_ctx* ctx_ = nullptr;
-    std::unordered_map<std::string, size_t> out_dim_;
-    std::unordered_map<size_t, size_t> hidden_;
     float dummy_ = 0.f;
 };
 

@@ -68,3 +68,48 @@ def golden():
     def load(name):
         return np.load(os.path.join(GOLDEN_DIR, name), allow_pickle=False)
     return load
+
+
+EXPERT_BLOCK = {8: (32, 34), 14: (256, 210)}   # ggml type -> (elements, bytes) per block
+
+
+def expert_rows(raw, ty, e, rows, in_dim):
+    """Raw bytes of expert e out of a stacked expert tensor [ne][rows][in_dim/QK blocks]."""
+    be, bb = EXPERT_BLOCK[ty]
+    per = rows * (in_dim // be) * bb
+    return np.asarray(raw, np.uint8).reshape(-1)[e * per:(e + 1) * per]
+
+
+def moe_layer_stagewise(accel, orc, layer, ty, gate, up, down, ne, hidden, eff, xs, plan, slot_tok, wslot, groups=None, tol=1e-5):
+    """Stage-by-stage parity of the grouped (prefill) MoE path, the way the decode path is checked:
+    gate/up of every slot against the oracle's Q8 matmul of the slot's expert on the slot's token;
+    the re-quantised silu(g)*u bit-exact on the device's own g, u; the down GEMM from the device's own
+    quants; the weighted combine in ascending slot order.  `groups`: indices of the plan entries to
+    check against the oracle (all when None); the combine is always checked for every token."""
+    m = xs.shape[0]
+    y, gu, aq, ad, dy = accel.moe_layer_stages(layer, xs, m, plan, slot_tok, wslot, eff)
+    xq, xd, _ = orc.actquant(xs, hidden)
+    worst = {"gate_up": 0.0, "down": 0.0, "combine": 0.0}
+    for gi in (range(len(plan)) if groups is None else groups):
+        e, off, cnt = (int(v) for v in plan[gi])
+        toks = slot_tok[off:off + cnt]
+        for z, w3 in enumerate((gate, up)):
+            ref = orc.matmul_q8(ty, expert_rows(w3, ty, e, eff, hidden), hidden, eff, xq[toks], xd[toks])
+            worst["gate_up"] = max(worst["gate_up"], rel_err(gu[off:off + cnt, z], ref))
+        a = orc.act_produce(2, gu[off:off + cnt, 0].reshape(-1), gu[off:off + cnt, 1].reshape(-1)).reshape(cnt, eff)
+        q2, d2, _ = orc.actquant(a, eff)
+        assert np.array_equal(aq[off:off + cnt], q2), f"group {gi}: quantised silu(g)*u differs"
+        assert np.array_equal(ad[off:off + cnt].view(np.uint32), d2.view(np.uint32)), f"group {gi}: block scales differ"
+        ref = orc.matmul_q8(ty, expert_rows(down, ty, e, hidden, eff), eff, hidden, aq[off:off + cnt], ad[off:off + cnt])
+        worst["down"] = max(worst["down"], rel_err(dy[off:off + cnt], ref))
+    want = np.zeros((m, hidden), np.float32)
+    for s in range(slot_tok.size):          # ascending slot index per token, fp32 multiply then add
+        want[slot_tok[s]] += np.float32(wslot[s]) * dy[s]
+    worst["combine"] = rel_err(y, want)
+    assert worst["gate_up"] <= tol and worst["down"] <= tol and worst["combine"] <= tol, worst
+    return y, worst
+
+
+@pytest.fixture(scope="session")
+def moe_stagewise():
+    return moe_layer_stagewise

@@ -74,6 +74,23 @@ def test_prefill_gemm_full_size_sampled(accel, orc, synth, relerr, ty, M, N, K):
 
 
 @pytest.mark.parametrize("ty", [8, 14])
+def test_moe_full_size_prefill_stagewise(accel, orc, synth, moe_stagewise, ty):
+    """cfg5 prefill (64 experts, hidden 2048, eff 768, top-8, 512 tokens = 4096 slots): every stage of the
+    grouped path against the oracle at 1e-5 / bit-exact quants; the gate/up and down GEMMs on a sample of the
+    expert groups (the largest, the smallest and six others), the combine on every token."""
+    ne, hidden, eff, k, m = 64, 2048, 768, 8, 512
+    gate, up, down = (synth.make_moe_q8 if ty == 8 else synth.make_moe_q6)(ne, hidden, eff, seed=30)
+    assert (accel.upload_moe_q8 if ty == 8 else accel.upload_moe_q6)(22, gate, up, down, hidden, eff, ne)
+    ids, w = synth.zipf_routing(m, ne, k, seed=31)
+    xs = synth.make_acts(m, hidden, seed=32)
+    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
+    assert slot_tok.size == 4096
+    by_size = np.argsort(plan[:, 2])
+    groups = sorted(set([int(by_size[0]), int(by_size[-1])] + [int(g) for g in np.random.default_rng(3).choice(len(plan), 6, replace=False)]))
+    moe_stagewise(accel, orc, 22, ty, gate, up, down, ne, hidden, eff, xs, plan, slot_tok, wslot, groups=groups)
+
+
+@pytest.mark.parametrize("ty", [8, 14])
 def test_moe_full_size_decode_and_prefill(accel, orc, synth, relerr, ty):
     ne, hidden, eff, k, m = 64, 2048, 768, 8, 512
     gate, up, down = (synth.make_moe_q8 if ty == 8 else synth.make_moe_q6)(ne, hidden, eff, seed=30)

@@ -70,21 +70,20 @@ FORM_SHAPES = [(2, 130, 2560), (2, 9, 96 * 32), (2, 2500, 2560), (2, 3, 4096 + 2
                (14, 70, 3840), (14, 9, 4352), (14, 1500, 256), (14, 33, 2048), (14, 5, 16384), (14, 3, 16640)]
 
 
-@pytest.mark.parametrize("form", [0, 1])     # smx_tune("gemv_flat"): 0 automatic, 1 never
 @pytest.mark.parametrize("ty,N,K", FORM_SHAPES)
-def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K, form):
+def test_gemv_forms_agree_with_oracle(accel, orc, synth, relerr, ty, N, K):
     raw = synth.make_weight(ty, N, K, seed=13 * N + K)
     x = synth.make_acts(1, K, seed=N + 7 * K)
     _up(accel, ty, "t.form", raw, K, N)
-    accel.tune("gemv_flat", form)
-    try:
-        y = accel.gemv("t.form", x, N)
-        # a group of two jobs with different row counts shares one launch geometry
-        raw2 = synth.make_weight(ty, N + 5, K, seed=17 * N + K)
-        _up(accel, ty, "t.form2", raw2, K, N + 5)
-        pair = accel.gemv_batch([("t.form", x), ("t.form2", x)], [N, N + 5])
-    finally:
-        accel.tune("gemv_flat", 0)
+    y = accel.gemv("t.form", x, N)
+    # the integers behind y, dumped by the same kernel form the call above ran (flat or row-per-wave)
+    xq, _, _ = orc.actquant(x, K)
+    per = K // 16 if ty == 14 else K // 32
+    assert np.array_equal(accel.gemv_block_dots("t.form", x, N, per), orc.block_dots(ty, raw, K, N, xq[0]))
+    # a group of two jobs with different row counts shares one launch geometry
+    raw2 = synth.make_weight(ty, N + 5, K, seed=17 * N + K)
+    _up(accel, ty, "t.form2", raw2, K, N + 5)
+    pair = accel.gemv_batch([("t.form", x), ("t.form2", x)], [N, N + 5])
     ref = orc.matmul_q8_from_f32(ty, raw, K, N, x)[0]
     assert relerr(y, ref) <= TOL
     assert relerr(pair[0], ref) <= TOL

@@ -14,19 +14,16 @@ def _layer(accel, synth, layer, ne, hidden, eff, seed):
 
 # k = 12: the 24 gate/up GEMVs exceed one grouped launch; eff = 416: down-projection units with a ragged tail;
 # eff = 32, 96, 416, 224 / 64 / 128 / 768: unit groups of 2 / 4 / 8 / 16 lanes in the flat down kernel;
-# (8, 1024, 2560): k * eff too large for it.  form 1 = the flat GEMV / down kernels switched off.
-@pytest.mark.parametrize("form", [0, 1])
+# (8, 1024, 2560): k * eff too large for it (the row-per-wave down kernel); hidden 2592 / 2336: gate and up
+# rows that are not a whole number of unit groups (the row-per-wave GEMV).
 @pytest.mark.parametrize("ne,hidden,eff,k", [(4, 64, 32, 2), (8, 256, 96, 3), (64, 2048, 768, 8), (16, 320, 416, 12),
-                                             (8, 96, 224, 4), (8, 192, 128, 4), (8, 128, 64, 2), (8, 1024, 2560, 8)])
-def test_moe_ffn_stagewise(accel, orc, synth, relerr, ne, hidden, eff, k, form):
+                                             (8, 96, 224, 4), (8, 192, 128, 4), (8, 128, 64, 2), (8, 1024, 2560, 8),
+                                             (4, 2592, 96, 2), (4, 2336, 64, 3)])
+def test_moe_ffn_stagewise(accel, orc, synth, relerr, ne, hidden, eff, k):
     gate, up, down = _layer(accel, synth, 3, ne, hidden, eff, seed=ne + hidden)
     ids, w = synth.zipf_routing(1, ne, k, seed=5)
     x = synth.make_acts(1, hidden, seed=6)[0]
-    accel.tune("gemv_flat", form)
-    try:
-        _moe_stagewise(accel, orc, relerr, gate, up, down, ne, hidden, eff, k, ids, w, x)
-    finally:
-        accel.tune("gemv_flat", 0)
+    _moe_stagewise(accel, orc, relerr, gate, up, down, ne, hidden, eff, k, ids, w, x)
 
 
 def _moe_stagewise(accel, orc, relerr, gate, up, down, ne, hidden, eff, k, ids, w, x):
@@ -120,6 +117,32 @@ def _moe_layer_oracle(orc, gate, up, down, hidden, eff, ne, xs, ids, w, ty=8):
         order = np.argsort(ids[t], kind="stable")
         out[t], _, _, _ = orc.moe_ffn_q8(gate, up, down, hidden, eff, ne, ids[t][order], w[t][order], xs[t], ty=ty)
     return out
+
+
+# (16, 512, 256, 4, 300): expert groups that span several 128-token tiles with ragged tails;
+# (8, 256, 160, 3, 37): weight-row tiles with a ragged tail (eff 160, hidden 256); (4, 64, 32, 2, 5): one tiny tile each
+@pytest.mark.parametrize("ne,hidden,eff,k,m", [(4, 64, 32, 2, 5), (8, 256, 160, 3, 37), (16, 512, 256, 4, 300), (3, 384, 416, 2, 700)])
+def test_moe_layer_stagewise(accel, orc, synth, moe_stagewise, ne, hidden, eff, k, m):
+    """The grouped prefill path (decode.rs:1608-1739: gather -> per-expert GEMMs -> silu_quant_rows ->
+    per-expert GEMMs -> weighted scatter) held to the decode path's bar at every stage."""
+    gate, up, down = _layer(accel, synth, 7, ne, hidden, eff, seed=hidden + m)
+    ids, w = synth.zipf_routing(m, ne, k, seed=9)
+    xs = synth.make_acts(m, hidden, seed=10)
+    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
+    y, worst = moe_stagewise(accel, orc, 7, 8, gate, up, down, ne, hidden, eff, xs, plan, slot_tok, wslot)
+    assert np.array_equal(y, accel.moe_layer_q8_dev(7, xs, m, plan, slot_tok, wslot))   # the plain call is the same computation
+
+
+@pytest.mark.parametrize("ne,hidden,eff,k,m", [(4, 256, 256, 2, 5), (8, 512, 256, 3, 37), (16, 512, 768, 4, 300)])
+def test_moe_layer_q6k_stagewise(accel, orc, synth, moe_stagewise, ne, hidden, eff, k, m):
+    """The same for Q6_K expert layers (q6_gemm_moe, kernels.rs:1688-1735): two K = 16 MFMAs per 32-block."""
+    gate, up, down = synth.make_moe_q6(ne, hidden, eff, seed=hidden + m)
+    assert accel.upload_moe_q6(17, gate, up, down, hidden, eff, ne)
+    ids, w = synth.zipf_routing(m, ne, k, seed=19)
+    xs = synth.make_acts(m, hidden, seed=20)
+    plan, slot_tok, wslot = synth.group_by_expert(ids, w, ne)
+    y, worst = moe_stagewise(accel, orc, 17, 14, gate, up, down, ne, hidden, eff, xs, plan, slot_tok, wslot)
+    assert np.array_equal(y, accel.moe_layer_q8_dev(17, xs, m, plan, slot_tok, wslot))
 
 
 @pytest.mark.parametrize("ne,hidden,eff,k,m", [(4, 64, 32, 2, 5), (8, 256, 160, 3, 37), (16, 512, 256, 4, 300)])

@@ -111,8 +111,9 @@ def test_capture_refuses_scratch_growth(accel, synth, pkg):
 
 
 def test_tuning_knobs_keep_results(accel, orc, synth, relerr, pkg):
-    N, K = 1000, 2560
-    for ty, up in ((2, accel.upload_q4_0), (8, accel.upload_q8_0), (14, accel.upload_q6_k)):
+    # the GEMV knobs shape the row-per-wavefront kernel: rows that are not a whole number of unit groups
+    # (81 blocks) or longer than 16384 elements (Q6_K rows are always whole groups)
+    for ty, up, N, K in ((2, accel.upload_q4_0, 1000, 2592), (8, accel.upload_q8_0, 1000, 2592), (14, accel.upload_q6_k, 300, 16640)):
         raw = synth.make_weight(ty, N, K, seed=ty)
         x = synth.make_acts(1, K, seed=9)
         assert up("t.tune", raw, K, N)
@@ -132,17 +133,8 @@ def test_tuning_knobs_keep_results(accel, orc, synth, relerr, pkg):
         accel.tune("gemm_splitk", sk)
         assert relerr(accel.prefill_q8_gemm("t.tune", xs, 64, 256), ref) <= 1e-5
     accel.tune("gemm_splitk", 0)
-    # 256 x 128 tiles (8 waves per workgroup), both weight formats, ragged M and N
-    for ty, up in ((8, accel.upload_q8_0), (2, accel.upload_q4_0)):
-        raw = synth.make_weight(ty, 200, 1056, seed=13)
-        xs = synth.make_acts(300, 1056, seed=14)
-        assert up("t.tune8", raw, 1056, 200)
-        ref = orc.matmul_q8_from_f32(ty, raw, 1056, 200, xs)
-        for nw in (8, 4, 0):
-            accel.tune("gemm_nw", nw)
-            assert relerr(accel.prefill_q8_gemm("t.tune8", xs, 300, 200), ref) <= 1e-5, nw
     with pytest.raises(pkg.SmxError):
-        accel.tune("gemm_nw", 3)
+        accel.tune("gemv_flat", 1)          # no knob re-routes a shape to another kernel
     with pytest.raises(pkg.SmxError):
         accel.tune("no_such_knob", 1)
     with pytest.raises(pkg.SmxError):
@@ -234,3 +226,55 @@ def test_ffn_block_two_launches_in_a_graph(accel, orc, synth, relerr, act):
     accel.graph_destroy(graph)
     for p in (xd, wd, gd, ud, yd):
         accel.dev_free(p)
+
+
+def test_evict_and_reupload_keep_a_live_graph_valid(pkg, synth):
+    """A captured graph holds the plane pointers of the weights it uses.  While it is alive, evicting or
+    replacing such a weight must not free the device memory under it: replays keep giving the result
+    they were captured with."""
+    acc = pkg.Mi355WeightAccel(0)
+    N, K = 384, 1024
+    raw_a, raw_b = synth.make_weight(8, N, K, seed=61), synth.make_weight(8, N, K, seed=62)
+    gate, up, down = synth.make_moe_q8(4, K, 64, seed=63)
+    gate2, up2, down2 = synth.make_moe_q8(4, K, 64, seed=64)
+    assert acc.upload_q8_0("t.live", raw_a, K, N) and acc.upload_moe_q8(5, gate, up, down, K, 64, 4)
+    assert acc.weight_dims("t.live") == (K, N) and acc.weight_dims("t.none") is None
+    x = synth.make_acts(1, K, seed=65)
+    ids, w = synth.zipf_routing(1, 4, 2, seed=66)
+    xd, yd, zd = acc.dev_alloc(x.nbytes), acc.dev_alloc(N * 4), acc.dev_alloc(K * 4)
+    acc.h2d(xd, x)
+
+    def chain():
+        acc.gemv_dev("t.live", xd, 1, yd)
+        acc.moe_ffn_dev(5, ids[0], w[0], xd, zd)
+
+    def read():
+        return acc.d2h(np.empty(N, np.float32), yd).copy(), acc.d2h(np.empty(K, np.float32), zd).copy()
+
+    chain()
+    want = read()
+    acc.graph_begin()
+    chain()
+    g = acc.graph_end()
+    assert acc.upload_q8_0("t.live", raw_b, K, N)                    # replaces the weight the graph reads
+    assert acc.upload_moe_q8(5, gate2, up2, down2, K, 64, 4)         # and the expert layer
+    junk = [acc.dev_alloc(raw_a.size) for _ in range(4)]             # allocations that would reuse freed memory
+    for p in junk:
+        acc.h2d(p, np.full(raw_a.size, 0x55, np.uint8))
+    for rep in range(2):
+        acc.h2d(yd, np.zeros(N, np.float32))
+        acc.h2d(zd, np.zeros(K, np.float32))
+        acc.graph_launch(g)
+        acc.sync()
+        got = read()
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), f"replay {rep}"
+    assert acc.evict("t.live") and acc.weight_dims("t.live") is None
+    acc.graph_launch(g)                                              # still reads memory the context keeps
+    acc.sync()
+    assert np.array_equal(read()[0], want[0])
+    chain_new = acc.gemv_dev("t.live", xd, 1, yd)                    # eager calls see the eviction
+    assert chain_new is False
+    acc.graph_destroy(g)
+    for p in junk + [xd, yd, zd]:
+        acc.dev_free(p)
+    acc.close()
