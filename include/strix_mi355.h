@@ -145,6 +145,14 @@ int smx_sync(smx_ctx* ctx);
  * Also the known-size reference kernel against which hardware traffic counters are scaled. */
 int smx_dev_copy(smx_ctx* ctx, void* dst_dev, const void* src_dev, size_t nbytes);
 int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
+/* smx_gemv_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same kernels and results
+ * as smx_gemv_dev; the rows quantised for m >= 2 live in a static device array of the library (160 KB per
+ * GPU, held until the process ends) instead of the context's growable scratch, so the call never
+ * allocates or frees device or host memory.  Limits: m <= SMX_GEMV_MAX_M, in_dim <= SMX_NOALLOC_MAX_IN_DIM
+ * (SMX_ERR_LIMIT beyond).  All contexts of one GPU share the array: calls that overlap on one GPU race. */
+#define SMX_NOALLOC_MAX_IN_DIM 16384
+int smx_gemv_noalloc_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 /* Up to 8 single-row GEMVs of one format and in_dim in ONE launch (gate+up, q/k/v, a batch of
  * weights against their activations); 0 if any key is not resident. */
 int smx_gemv_batch_dev(smx_ctx* ctx, size_t n, const char* const* keys, const float* const* xs_dev,

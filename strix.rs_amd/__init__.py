@@ -35,7 +35,7 @@ EXPORTS = [
     "smx_upload_moe_q6", "smx_gguf_open", "smx_gguf_close", "smx_gguf_tensor_count", "smx_gguf_tensor",
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
-    "smx_weight_dims", "smx_moe_layer_stages",
+    "smx_weight_dims", "smx_moe_layer_stages", "smx_gemv_noalloc_dev",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -94,6 +94,7 @@ def load_library():
     L.smx_dev_copy.argtypes = [vp, vp, vp, sz]
     L.smx_gemv_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemm_dev.argtypes = [vp, cp, vp, sz, vp]
+    L.smx_gemv_noalloc_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemv_batch_dev.argtypes = [vp, sz, vp, vp, vp]
     L.smx_gemv_fused_dev.argtypes = [vp, sz, vp, i, vp, vp, C.c_float, vp]
     L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
@@ -490,6 +491,10 @@ class Mi355WeightAccel:
 
     def gemv_dev(self, key, xs_dev, m, y_dev):
         return self._check(self._L.smx_gemv_dev(self._h, key.encode(), xs_dev, m, y_dev))
+
+    def gemv_noalloc_dev(self, key, xs_dev, m, y_dev):
+        """gemv_dev that allocates nothing (static device scratch; m <= 8, in_dim <= 16384)."""
+        return self._check(self._L.smx_gemv_noalloc_dev(self._h, key.encode(), xs_dev, m, y_dev))
 
     def gemv_batch_dev(self, keys, xs_dev, ys_dev):
         n = len(keys)

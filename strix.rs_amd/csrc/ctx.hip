@@ -248,6 +248,14 @@ int smx_create(int device, smx_ctx** out) {
         delete c;
         return fail(nullptr, SMX_ERR_HIP, "smx_create: hipEventCreate failed");
     }
+    if (noalloc_init(c) != SMX_OK) {   // the static scratch array of the allocation-free entry point, on this device
+        g_create_err = c->err;
+        (void)hipEventDestroy(c->t0);
+        (void)hipEventDestroy(c->t1);
+        (void)hipStreamDestroy(c->stream);
+        delete c;
+        return SMX_ERR_HIP;
+    }
     *out = c;
     return SMX_OK;
 }

@@ -295,14 +295,14 @@ static int launch_jobs(smx_ctx* c, QType type, const Geom& g, const GemvJobs& J,
     return launch_type<OpsQ6_K>(c, g, J, njobs, nblk, m, mt, dump, dump_per_row);
 }
 
-int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump) {
+int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump, const ActScratch* sc) {
     if (m == 0 || m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv: %zu rows (1..%d supported)", m, SMX_GEMV_MAX_M);
     if (w.N > 0x7fffffffu / 4 || w.K > (size_t(1) << 20))
         return fail(c, SMX_ERR_LIMIT, "gemv: shape %zu x %zu exceeds the kernel's index range", w.N, w.K);
     if (w.type == kQ6_K && m > 4) {  // Q6_K keeps at most 4 activation rows in registers per launch
-        int rc = launch_gemv(c, w, x, 4, y, nullptr);
+        int rc = launch_gemv(c, w, x, 4, y, nullptr, sc);
         if (rc != SMX_OK) return rc;
-        return launch_gemv(c, w, x + 4 * w.K, m - 4, y + 4 * w.N, nullptr);
+        return launch_gemv(c, w, x + 4 * w.K, m - 4, y + 4 * w.N, nullptr, sc);   // same stream: the second pass may reuse sc
     }
     const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8));
     const Geom g = pick_geom(c, w.type, w.N, w.nblk, mt, dump != nullptr, 1);
@@ -316,12 +316,18 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
     if (mt > 1) {
         // each of the persistent workgroups would repeat the quantiser for all m rows: do it once instead
         int rc;
-        if ((rc = ensure(c, c->xq, m * w.K)) != SMX_OK) return rc;
-        if ((rc = ensure(c, c->xd, m * (w.K / 32) * 4)) != SMX_OK) return rc;
-        if ((rc = ensure(c, c->xs, m * (w.K / 32) * 4)) != SMX_OK) return rc;
-        rc = launch_actquant(c, x, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
+        ActScratch a;
+        if (sc) {
+            a = *sc;
+        } else {
+            if ((rc = ensure(c, c->xq, m * w.K)) != SMX_OK) return rc;
+            if ((rc = ensure(c, c->xd, m * (w.K / 32) * 4)) != SMX_OK) return rc;
+            if ((rc = ensure(c, c->xs, m * (w.K / 32) * 4)) != SMX_OK) return rc;
+            a = ActScratch{(int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p};
+        }
+        rc = launch_actquant(c, x, m, w.K, a.xq, a.xd, a.xs);
         if (rc != SMX_OK) return rc;
-        J.job[0].X = {nullptr, (const int8_t*)c->xq.p, (const float*)c->xd.p, (const int*)c->xs.p};
+        J.job[0].X = {nullptr, a.xq, a.xd, (const int*)a.xs};
     }
     return launch_jobs(c, w.type, g, J, 1, (int)w.nblk, (int)m, mt, dump, (int)(w.type == kQ6_K ? w.K / 16 : w.K / 32));
 }

@@ -80,8 +80,14 @@ struct smx_ctx {
     // tuning overrides (0 = automatic)
     int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0;
 
-    // dynamic-LDS limit already raised on this context's device, per kernel (see set_dyn_lds)
-    std::unordered_map<const void*, size_t> lds_set;
+    // dynamic-LDS limit already raised on this context's device, per kernel (see set_dyn_lds): a fixed
+    // open-addressing table, so that a launch never allocates host memory
+    static constexpr int kLdsSlots = 512;
+    const void* lds_kern[kLdsSlots] = {};
+    size_t lds_size[kLdsSlots] = {};
+
+    // device address of the library's static scratch array on this context's device (see noalloc.hip)
+    void* static_scratch = nullptr;
 
     bool capturing = false;  // between smx_graph_begin and smx_graph_end
     // A captured graph holds the addresses of the scratch buffers its kernels used.  While any graph
@@ -135,11 +141,21 @@ int ensure_host(smx_ctx* c, DevBuf& b, size_t bytes);
 template <typename Kern>
 int set_dyn_lds(smx_ctx* c, Kern kern, size_t lds) {
     if (lds <= 48 * 1024) return SMX_OK;
-    size_t& cached = c->lds_set[(const void*)kern];
-    if (lds <= cached) return SMX_OK;
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    const void* key = (const void*)kern;
+    unsigned slot = (unsigned)(((uintptr_t)key >> 4) * 2654435761u) % smx_ctx::kLdsSlots;
+    int probes = 0;
+    while (c->lds_kern[slot] && c->lds_kern[slot] != key && probes < smx_ctx::kLdsSlots) {
+        slot = (slot + 1) % smx_ctx::kLdsSlots;
+        probes++;
+    }
+    const bool have_slot = probes < smx_ctx::kLdsSlots;   // a full table only costs the repeated attribute call
+    if (have_slot && c->lds_kern[slot] == key && lds <= c->lds_size[slot]) return SMX_OK;
+    hipError_t e = hipFuncSetAttribute(key, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return hip_fail(c, e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-    cached = lds;
+    if (have_slot) {
+        c->lds_kern[slot] = key;
+        c->lds_size[slot] = lds;
+    }
     return SMX_OK;
 }
 
@@ -188,9 +204,19 @@ int launch_actprod_quant(smx_ctx* c, int kind, const float* const* as, const flo
 // b[m][K]) and the quantiser: xq[m][K], xd/xs[m][K/32].
 int launch_rows_prod_quant(smx_ctx* c, int kind, const float* a, const float* b, size_t m, size_t K, float eps, int8_t* xq,
                            float* xd, int32_t* xs);
+// Room for m quantised activation rows of length K: xq[m][K], xd[m][K/32], xs[m][K/32].
+struct ActScratch {
+    int8_t* xq;
+    float* xd;
+    int32_t* xs;
+};
 // GEMV with the activation quantiser fused into its LDS staging: x fp32 [m][K] -> y[m][N],
-// m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.
-int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump);
+// m <= SMX_GEMV_MAX_M.  dump (optional): per-block i32 dots of row 0.  Several rows are quantised once
+// into `sc`, or into the context's own scratch (grown on demand) when sc is null.
+int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump,
+                const ActScratch* sc = nullptr);
+// Looks the library's static scratch array up on the context's device (called once by smx_create).
+int noalloc_init(smx_ctx* c);
 // n <= 8 single-row GEMVs of one format and row length in one launch (device pointers).
 // prod (optional): activation producer applied to every job's x before the fused quantiser.
 struct ActProd {
