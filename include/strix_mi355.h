@@ -89,6 +89,15 @@ int smx_weight_dims(const smx_ctx* ctx, const char* key, size_t* in_dim, size_t*
  * dots (kernels.rs:259-287, 894-912).  in_len must equal in_dim, out_cap >= out_dim. */
 int smx_gemv(smx_ctx* ctx, const char* key, const float* x, size_t in_len, float* y,
              size_t out_cap);
+/* The same product with fp32 activations: no quantiser, every weight widened to fp32 and multiplied with x,
+ * the arithmetic of the kernels the reference launches for WeightAccel::gemv (kernels.rs:41-69 q4_gemv,
+ * :646-668 q8_0_gemv, :607-640 q6_gemv) and of strix-backend-cpu, whose result it matches to fp32 rounding
+ * (the reference's own device test asks for rel < 1e-3, strix-backend-rocm/src/lib.rs:231).  smx_gemv above
+ * differs from the CPU result by the activation rounding of the decode path (about 1e-2 relative).
+ * in_dim <= SMX_GEMV_F32_MAX_IN_DIM (the fp32 row is staged in LDS). */
+#define SMX_GEMV_F32_MAX_IN_DIM 32768
+int smx_gemv_f32(smx_ctx* ctx, const char* key, const float* x, size_t in_len, float* y, size_t out_cap);
+int smx_gemv_f32_dev(smx_ctx* ctx, const char* key, const float* x_dev, float* y_dev);
 /* Small-batch GEMV, m <= SMX_GEMV_MAX_M rows against one weight read once
  * (kernels.rs:1016-1045, the n-gram verify path): xs[m][in_dim] -> y[m][out_dim]. */
 #define SMX_GEMV_MAX_M 8
@@ -188,6 +197,18 @@ int smx_gemm_fused_dev(smx_ctx* ctx, const char* key, int act, const float* a_de
 int smx_moe_shexp_dev(smx_ctx* ctx, size_t layer, float sgate, const float* x_dev, float* y_dev);
 int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float* wexp, size_t k,
                     const float* x_dev, float* y_dev);
+/* The router on the device (kernels.rs:1846-1872 topk_router; mellum.rs:1178-1192): softmax over the ne
+ * logits, the k largest probabilities in descending order (equal ones: lowest index first), weights
+ * renormalised over the chosen k.  ids_dev[k] i32, w_dev[k] f32; ne <= 1024, k <= 64.  smx_moe_route is the
+ * same with host buffers (one sync). */
+int smx_moe_route_dev(smx_ctx* ctx, const float* logits_dev, size_t ne, size_t k, int32_t* ids_dev, float* w_dev);
+int smx_moe_route(smx_ctx* ctx, const float* logits, size_t ne, size_t k, int32_t* ids, float* w);
+/* smx_moe_ffn_dev with the routing read from device memory when the kernels run (what smx_moe_route_dev
+ * wrote): router + expert FFN of a decode token can be captured once and replayed with every token's own
+ * routing (decode.rs:1923-2128 reads the router's device output the same way).  Ids outside 0 .. ne - 1
+ * are clamped. */
+int smx_moe_ffn_routed_dev(smx_ctx* ctx, size_t layer, const int32_t* ids_dev, const float* w_dev, size_t k,
+                           const float* x_dev, float* y_dev);
 /* smx_moe_layer with the activations and the result on the device (y_dev: m x hidden floats); the
  * routing tables still come from the host at every call, so it cannot be captured in a graph. */
 int smx_moe_layer_dev(smx_ctx* ctx, size_t layer, const float* xs_dev, size_t m, const size_t* plan,

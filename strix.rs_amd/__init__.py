@@ -36,6 +36,7 @@ EXPORTS = [
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
     "smx_weight_dims", "smx_moe_layer_stages", "smx_gemv_noalloc_dev",
+    "smx_gemv_f32", "smx_gemv_f32_dev", "smx_moe_route_dev", "smx_moe_route", "smx_moe_ffn_routed_dev",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -77,6 +78,8 @@ def load_library():
     L.smx_upload_moe_q6.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz, sz, sz, sz]
     L.smx_evict.argtypes = [vp, cp]
     L.smx_gemv.argtypes = [vp, cp, vp, sz, vp, sz]
+    L.smx_gemv_f32.argtypes = [vp, cp, vp, sz, vp, sz]
+    L.smx_gemv_f32_dev.argtypes = [vp, cp, vp, vp]
     L.smx_gemv_rows.argtypes = [vp, cp, vp, sz, sz, vp, sz]
     L.smx_gemv_batch.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp]
     L.smx_gemm.argtypes = [vp, cp, vp, sz, sz, vp, sz]
@@ -100,6 +103,9 @@ def load_library():
     L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_moe_shexp_dev.argtypes = [vp, sz, C.c_float, vp, vp]
+    L.smx_moe_route_dev.argtypes = [vp, vp, sz, sz, vp, vp]
+    L.smx_moe_route.argtypes = [vp, vp, sz, sz, vp, vp]
+    L.smx_moe_ffn_routed_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_gemm_fused_dev.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp]
     L.smx_moe_layer_ffn.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz]
     L.smx_moe_expert_ffn.argtypes = [vp, sz, sz, vp, sz, vp, sz]
@@ -332,6 +338,16 @@ class Mi355WeightAccel:
         ok = self._check(self._L.smx_gemv(self._h, key.encode(), _p(x), x.size, _p(y), y.size))
         return y if ok else None
 
+    def gemv_f32(self, key, x, out_dim):
+        """gemv with fp32 activations (the arithmetic of the reference's per-weight gemv and of its CPU path)."""
+        x = _c(x, np.float32).reshape(-1)
+        y = np.empty(out_dim, np.float32)
+        ok = self._check(self._L.smx_gemv_f32(self._h, key.encode(), _p(x), x.size, _p(y), y.size))
+        return y if ok else None
+
+    def gemv_f32_dev(self, key, x_dev, y_dev):
+        return self._check(self._L.smx_gemv_f32_dev(self._h, key.encode(), x_dev, y_dev))
+
     def gemv_fused(self, key, act, a, b, out_dim, eps=0.0):
         """GEMV of producer(a, b): rmsnorm(a)*b, silu(a)*b or gelu_tanh(a)*b (kernels.rs:101-226), one launch."""
         a = _c(a, np.float32).reshape(-1)
@@ -519,6 +535,20 @@ class Mi355WeightAccel:
     def moe_ffn_dev(self, layer, ids, wexp, x_dev, y_dev):
         ids, wexp = _c(ids, np.int32), _c(wexp, np.float32)
         return self._check(self._L.smx_moe_ffn_dev(self._h, layer, _p(ids), _p(wexp), ids.size, x_dev, y_dev))
+
+    def moe_route(self, logits, k):
+        """Router on the device (topk_router, kernels.rs:1846-1872): (ids[k] i32, w[k] f32)."""
+        logits = _c(logits, np.float32).reshape(-1)
+        ids, w = np.empty(k, np.int32), np.empty(k, np.float32)
+        self._check(self._L.smx_moe_route(self._h, _p(logits), logits.size, k, _p(ids), _p(w)))
+        return ids, w
+
+    def moe_route_dev(self, logits_dev, ne, k, ids_dev, w_dev):
+        return self._check(self._L.smx_moe_route_dev(self._h, logits_dev, ne, k, ids_dev, w_dev))
+
+    def moe_ffn_routed_dev(self, layer, ids_dev, w_dev, k, x_dev, y_dev):
+        """moe_ffn_dev reading the routing from device memory at run time (capturable with new routing)."""
+        return self._check(self._L.smx_moe_ffn_routed_dev(self._h, layer, ids_dev, w_dev, k, x_dev, y_dev))
 
     def moe_shexp_dev(self, layer, sgate, x_dev, y_dev):
         """y_dev += sgate * shared_expert(x_dev) (decode.rs:1820-1855)."""

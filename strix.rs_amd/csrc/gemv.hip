@@ -30,14 +30,30 @@ struct GemvJob {
 };
 struct GemvJobs {
     GemvJob job[SMX_GEMV_GROUP_MAX];
+    // expert indirection (MoE decode routed on the device): job j reads expert ids[slot[j]] of a stacked tensor
+    const int* ids;
+    int ne;
+    unsigned long long blocks_per_expert;
+    int slot[SMX_GEMV_GROUP_MAX];
 };
+
+// The planes of a job's weight, moved to the expert the device-side routing names.
+template <class Ops>
+__device__ __forceinline__ GemvW job_weight(const GemvJobs& J, int j) {
+    GemvW W = J.job[j].W;
+    if (J.ids) {
+        const size_t b0 = (size_t)min(max(J.ids[J.slot[j]], 0), J.ne - 1) * J.blocks_per_expert;
+        Ops::advance(W, b0);
+    }
+    return W;
+}
 
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT>
 __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, int m, int* __restrict__ dump,
                                                   int dump_per_row) {
     const int nw = NT / 64;
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
+    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(job_weight<Ops>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
@@ -47,7 +63,7 @@ template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP>
 __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, int m, unsigned magic_u,
                                                          int* __restrict__ dump, int dump_per_row) {
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(jb.W, jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u,
+    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(job_weight<Ops>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u,
                                                dump, dump_per_row);
 }
 
@@ -334,10 +350,16 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
 
 // n <= SMX_GEMV_GROUP_MAX single-row GEMVs of one format and row length in one launch.
 int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
-                      const char* name, const ActProd* prod, const float* const* x2s) {
+                      const char* name, const ActProd* prod, const float* const* x2s, const GemvIndirect* ind) {
     if (n < 1 || n > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "gemv group of %d", n);
     size_t maxN = 0;
     GemvJobs J = {};
+    if (ind) {
+        J.ids = ind->ids;
+        J.ne = ind->ne;
+        J.blocks_per_expert = ind->blocks_per_expert;
+        for (int i = 0; i < n; i++) J.slot[i] = ind->slot[i];
+    }
     for (int i = 0; i < n; i++) {
         const Weight& w = *ws[i];
         if (w.type != ws[0]->type || w.K != ws[0]->K) return fail(c, SMX_ERR_ARG, "gemv group mixes formats or row lengths");

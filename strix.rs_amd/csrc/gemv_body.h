@@ -119,6 +119,11 @@ struct OpsQ4_0 {
         r.q = w.quants[f];
         r.s = w.scales[f];
     }
+    // move the planes b0 blocks further (to another expert of a stacked tensor)
+    static __device__ __forceinline__ void advance(GemvW& w, size_t b0) {
+        w.scales += b0;
+        w.quants += b0;
+    }
 };
 
 struct OpsQ8_0 {
@@ -141,6 +146,10 @@ struct OpsQ8_0 {
     static __device__ __forceinline__ void load_flat(Regs& r, const GemvW& w, size_t f) {
         r.q = w.quants[f];
         r.s = w.scales[f >> 1];   // two units per block, an even number of units per row
+    }
+    static __device__ __forceinline__ void advance(GemvW& w, size_t b0) {
+        w.scales += b0;
+        w.quants += b0 * 2;
     }
 };
 
@@ -201,6 +210,12 @@ struct OpsQ6_K {
         r.h = w.qh[f];
         r.sc = w.sc[f >> 1];
         r.d = w.scales[f >> 2];
+    }
+    static __device__ __forceinline__ void advance(GemvW& w, size_t sb0) {
+        w.scales += sb0;
+        w.quants += sb0 * 8;
+        w.qh += sb0 * 4;
+        w.sc += sb0 * 2;
     }
 };
 

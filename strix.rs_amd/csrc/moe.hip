@@ -67,11 +67,75 @@ __global__ __launch_bounds__(256) void silu_mul_quant_kernel(const float* __rest
     }
 }
 
-// Routed expert ids and weights travel as kernel arguments (no table upload on the decode path).
+// Routed expert ids and weights travel as kernel arguments (no table upload on the decode path), or,
+// when the router ran on the device, are read from its output at run time (ids_dev / w_dev non-null):
+// a captured graph then serves every token's own routing.
 struct MoeRoute {
     int ids[64];
     float w[64];
+    const int* ids_dev;
+    const float* w_dev;
+    int ne;   // expert ids read from the device are clamped to 0 .. ne - 1
 };
+__device__ __forceinline__ int route_id(const MoeRoute& r, int i) {
+    return r.ids_dev ? min(max(r.ids_dev[i], 0), r.ne - 1) : r.ids[i];
+}
+__device__ __forceinline__ float route_w(const MoeRoute& r, int i) { return r.w_dev ? r.w_dev[i] : r.w[i]; }
+
+// Router (kernels.rs:1846-1872 topk_router; crates/strix-backend-cpu/src/mellum.rs:1178-1192): softmax over
+// all ne logits, the k largest probabilities in descending order (equal probabilities: lowest index
+// first, the order of the reference's stable sort), weights renormalised over the chosen k.  Experts more
+// than 87 below the largest logit all get the probability exp(-87) (the fixed-sequence exp clamps its
+// argument) and tie to the lowest index; their weight is below 2e-38 either way.  One wave;
+// lane l holds experts l, l + 64, ...  The softmax denominator is summed in double in a fixed order.
+constexpr int kRouterPerLane = 16;   // ne <= 1024
+__global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict__ logits, int ne, int k,
+                                                         int* __restrict__ ids, float* __restrict__ w) {
+#pragma clang fp contract(off)
+    const int lane = threadIdx.x;
+    float v[kRouterPerLane];
+    float mx = -3.40282347e+38f;
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; j++) {
+        const int e = lane + 64 * j;
+        v[j] = e < ne ? logits[e] : -3.40282347e+38f;
+        mx = fmaxf(mx, v[j]);
+    }
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    double sum = 0.0;
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; j++) {
+        const int e = lane + 64 * j;
+        v[j] = e < ne ? det_expf(v[j] - mx) : -1.f;   // probabilities are >= 0: -1 marks "absent or taken"
+        if (e < ne) sum += (double)v[j];
+    }
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    const float fsum = (float)sum;
+#pragma unroll
+    for (int j = 0; j < kRouterPerLane; j++)
+        if (v[j] >= 0.f) v[j] = v[j] / fsum;
+    float wsum = 0.f;
+    float mine = 0.f;   // lane i keeps the probability of pick i (k <= 64)
+    for (int i = 0; i < k; i++) {
+        float b = -1.f;
+        int bi = 1 << 30;
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++)
+            if (v[j] > b) { b = v[j]; bi = lane + 64 * j; }   // ascending index within the lane: '>' keeps the lowest
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(b, off);
+            const int oi = __shfl_xor(bi, off);
+            if (ob > b || (ob == b && oi < bi)) { b = ob; bi = oi; }
+        }
+#pragma unroll
+        for (int j = 0; j < kRouterPerLane; j++)
+            if (lane + 64 * j == bi) v[j] = -1.f;
+        if (lane == i) mine = b;
+        if (lane == 0) ids[i] = bi;
+        wsum += b;   // in pick order, as the reference sums the chosen probabilities
+    }
+    if (lane < k) w[lane] = mine / wsum;
+}
 
 // Decode, second half, in one launch: a_k = quantised silu(g_k)*u_k is rebuilt in LDS by every
 // workgroup (k*eff elements; measured faster than a launch of its own), then each wave computes
@@ -94,8 +158,8 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(const float* __res
     float* sw = (float*)(sid + k);                  // [k] routing weights
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid < k) {
-        sid[tid] = route.ids[tid];
-        sw[tid] = route.w[tid];
+        sid[tid] = route_id(route, tid);
+        sw[tid] = route_w(route, tid);
     }
     __syncthreads();
 
@@ -199,8 +263,8 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
     float* part = sw + k;                           // [rows * units / GL]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid < k) {
-        sid[tid] = route.ids[tid];
-        sw[tid] = route.w[tid];
+        sid[tid] = route_id(route, tid);
+        sw[tid] = route_w(route, tid);
     }
     __syncthreads();
     const unsigned rbase = (unsigned)hidden / gridDim.x, rrem = (unsigned)hidden - rbase * gridDim.x;
@@ -354,7 +418,7 @@ __global__ __launch_bounds__(256) void moe_wsum_kernel(const float* __restrict__
     const int o = blockIdx.x * 256 + threadIdx.x;
     if (o >= n) return;
     float s = 0.f;
-    for (int e = 0; e < k; e++) s += route.w[e] * dy[(size_t)e * n + o];
+    for (int e = 0; e < k; e++) s += route_w(route, e) * dy[(size_t)e * n + o];
     out[o] = s;
 }
 
@@ -393,10 +457,13 @@ struct MoeScratch {
     float* ad;
 };
 
+// ids / wexp: the routing on the host; or, with ids_dev / w_dev, device memory read when the kernels run.
 static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, const float* wexp, size_t k,
-                           const float* x_dev, float* y_dev, MoeScratch* out_scratch) {
+                           const float* x_dev, float* y_dev, MoeScratch* out_scratch, const int32_t* ids_dev = nullptr,
+                           const float* w_dev = nullptr) {
     if (k == 0 || k > 64) return fail(c, SMX_ERR_LIMIT, "moe_ffn: %zu routed experts (1..64 supported)", k);
-    for (size_t i = 0; i < k; i++)
+    const bool routed_on_device = ids_dev != nullptr;
+    for (size_t i = 0; i < k && !routed_on_device; i++)
         if (ids[i] < 0 || (size_t)ids[i] >= L.ne)
             return fail(c, SMX_ERR_ARG, "moe_ffn: expert id %d outside 0..%zu", ids[i], L.ne - 1);
     const size_t hidden = L.hidden, eff = L.eff;
@@ -406,10 +473,18 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
                  o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(L.type == kQ6_K ? k * hidden * 4 : 0);
     if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
     MoeRoute route = {};
-    for (size_t i = 0; i < k; i++) {
+    route.ids_dev = ids_dev;
+    route.w_dev = w_dev;
+    route.ne = (int)L.ne;
+    for (size_t i = 0; i < k && !routed_on_device; i++) {
         route.ids[i] = ids[i];
         route.w[i] = wexp[i];
     }
+    // With the routing on the device every job is a view of expert 0 and the kernel moves it to the
+    // expert it reads from ids_dev (GemvIndirect).
+    GemvIndirect ind = {};
+    ind.ids = ids_dev;
+    ind.ne = (int)L.ne;
     MoeScratch s;
     s.g = (float*)(c->work.p + o_g);
     s.u = (float*)(c->work.p + o_u);
@@ -424,13 +499,16 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
         std::vector<float*> ys(2 * k);
         for (size_t i = 0; i < k; i++)
             for (int z = 0; z < 2; z++) {
-                views[2 * i + z] = expert_view(z ? L.up : L.gate, (size_t)ids[i], eff);
+                views[2 * i + z] = expert_view(z ? L.up : L.gate, routed_on_device ? 0 : (size_t)ids[i], eff);
                 ws[2 * i + z] = &views[2 * i + z];
                 ys[2 * i + z] = (z ? s.u : s.g) + i * eff;
             }
+        ind.blocks_per_expert = eff * L.gate.nblk;
         for (size_t i = 0; i < 2 * k; i += SMX_GEMV_GROUP_MAX) {
             const int n = (int)std::min<size_t>(SMX_GEMV_GROUP_MAX, 2 * k - i);
-            rc = launch_gemv_group(c, &ws[i], &xs[i], &ys[i], n, "moe_gemv_gate_up");
+            for (int j = 0; j < n; j++) ind.slot[j] = (int)((i + j) / 2);
+            rc = launch_gemv_group(c, &ws[i], &xs[i], &ys[i], n, "moe_gemv_gate_up", nullptr, nullptr,
+                                   routed_on_device ? &ind : nullptr);
             if (rc != SMX_OK) return rc;
         }
     }
@@ -443,16 +521,18 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
         std::vector<const float*> gs(k), us(k);
         std::vector<float*> ys(k);
         for (size_t i = 0; i < k; i++) {
-            views[i] = expert_view(L.down, (size_t)ids[i], hidden);
+            views[i] = expert_view(L.down, routed_on_device ? 0 : (size_t)ids[i], hidden);
             ws[i] = &views[i];
             gs[i] = s.g + i * eff;
             us[i] = s.u + i * eff;
             ys[i] = dy + i * hidden;
         }
         const ActProd prod = {SMX_ACT_SILU_MUL, nullptr, 0.f};
+        ind.blocks_per_expert = hidden * L.down.nblk;
         for (size_t i = 0; i < k; i += SMX_GEMV_GROUP_MAX) {
             const int n = (int)std::min<size_t>(SMX_GEMV_GROUP_MAX, k - i);
-            rc = launch_gemv_group(c, &ws[i], &gs[i], &ys[i], n, "moe_gemv_down", &prod, &us[i]);
+            for (int j = 0; j < n; j++) ind.slot[j] = (int)(i + j);
+            rc = launch_gemv_group(c, &ws[i], &gs[i], &ys[i], n, "moe_gemv_down", &prod, &us[i], routed_on_device ? &ind : nullptr);
             if (rc != SMX_OK) return rc;
         }
         {
@@ -636,6 +716,45 @@ int smx_moe_ffn_dev(smx_ctx* c, size_t layer, const int32_t* ids, const float* w
         auto it = c->moe.find(layer);
         if (it == c->moe.end()) return SMX_NOT_RESIDENT;
         return moe_ffn_enqueue(c, it->second, ids, wexp, k, x_dev, y_dev, nullptr);
+    });
+}
+
+int smx_moe_route_dev(smx_ctx* c, const float* logits_dev, size_t ne, size_t k, int32_t* ids_dev, float* w_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!logits_dev || !ids_dev || !w_dev) return fail(c, SMX_ERR_ARG, "moe_route_dev: null argument");
+    if (ne == 0 || ne > 64 * kRouterPerLane || k == 0 || k > 64 || k > ne)
+        return fail(c, SMX_ERR_LIMIT, "moe_route_dev: %zu experts, top %zu (up to %d experts, top 64)", ne, k, 64 * kRouterPerLane);
+    ProfScope ps(c, "topk_router");
+    hipLaunchKernelGGL(topk_router_kernel, dim3(1), dim3(64), 0, c->stream, logits_dev, (int)ne, (int)k, ids_dev, w_dev);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
+}
+
+int smx_moe_route(smx_ctx* c, const float* logits, size_t ne, size_t k, int32_t* ids, float* w) {
+    if (!c) return SMX_ERR_ARG;
+    if (!logits || !ids || !w) return fail(c, SMX_ERR_ARG, "moe_route: null argument");
+    if (ne == 0 || k == 0 || k > 64) return fail(c, SMX_ERR_LIMIT, "moe_route: %zu experts, top %zu", ne, k);
+    SMX_HIP(c, hipSetDevice(c->device));
+    int rc;
+    if ((rc = ensure(c, c->xf32, ne * 4)) != SMX_OK) return rc;
+    if ((rc = ensure(c, c->tab, 2 * 64 * 4)) != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, logits, ne * 4, hipMemcpyHostToDevice, c->stream));
+    rc = smx_moe_route_dev(c, (const float*)c->xf32.p, ne, k, (int32_t*)c->tab.p, (float*)(c->tab.p + 256));
+    if (rc != SMX_OK) return rc;
+    SMX_HIP(c, hipMemcpyAsync(ids, c->tab.p, k * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipMemcpyAsync(w, c->tab.p + 256, k * 4, hipMemcpyDeviceToHost, c->stream));
+    SMX_HIP(c, hipStreamSynchronize(c->stream));
+    return SMX_OK;
+}
+
+int smx_moe_ffn_routed_dev(smx_ctx* c, size_t layer, const int32_t* ids_dev, const float* w_dev, size_t k, const float* x_dev,
+                           float* y_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!ids_dev || !w_dev || !x_dev || !y_dev) return fail(c, SMX_ERR_ARG, "moe_ffn_routed_dev: null argument");
+    return guarded(c, "moe_ffn_routed_dev", [&]() -> int {
+        auto it = c->moe.find(layer);
+        if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+        return moe_ffn_enqueue(c, it->second, nullptr, nullptr, k, x_dev, y_dev, nullptr, ids_dev, w_dev);
     });
 }
 

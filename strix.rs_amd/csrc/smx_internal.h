@@ -215,6 +215,8 @@ struct ActScratch {
 // into `sc`, or into the context's own scratch (grown on demand) when sc is null.
 int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump,
                 const ActScratch* sc = nullptr);
+// y[N] = dequant(W) . x with fp32 activations (no quantiser): the arithmetic of the reference's per-weight gemv.
+int launch_gemv_f32(smx_ctx* c, const Weight& w, const float* x, float* y);
 // Looks the library's static scratch array up on the context's device (called once by smx_create).
 int noalloc_init(smx_ctx* c);
 // n <= 8 single-row GEMVs of one format and row length in one launch (device pointers).
@@ -224,9 +226,19 @@ struct ActProd {
     const float* b;  // rmsnorm weight (or null) / the `up` operand of silu_mul, geglu
     float eps;
 };
+// Jobs whose weight is one expert of a stacked expert tensor chosen on the device: job j reads expert
+// ids[slot[j]] (clamped to 0 .. ne - 1); its Weight is the view of expert 0, blocks_per_expert the
+// number of blocks (Q6_K: superblocks) from one expert's rows to the next.
+struct GemvIndirect {
+    const int* ids;
+    int ne;
+    size_t blocks_per_expert;
+    int slot[SMX_GEMV_GROUP_MAX];
+};
 // x2s (optional, with prod): a second operand per job instead of prod->b.
 int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,
-                      const char* name = nullptr, const ActProd* prod = nullptr, const float* const* x2s = nullptr);
+                      const char* name = nullptr, const ActProd* prod = nullptr, const float* const* x2s = nullptr,
+                      const GemvIndirect* ind = nullptr);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);

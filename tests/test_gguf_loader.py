@@ -82,6 +82,13 @@ def test_host_quantisers_match_the_oracle(pkg, orc, synth):
                         rng.normal(0, 300, 64)]).astype(np.float32)
     assert np.array_equal(pkg.host_quantize_q8_0(x), orc.quantize_q8_0(x))
     assert np.array_equal(pkg.host_quantize_q4_0(x), orc.quantize_q4_0(x))
+    # and against blocks worked out by hand from ggml_quant.rs:212-237 (sign of d, +8.5 truncation, clamping)
+    a = np.zeros(32, np.float32)
+    a[[0, 1, 2, 3, 16, 17, 31]] = [8.0, -4.0, 1.0, 0.4, 3.0, -7.0, 7.9]
+    assert bytes(pkg.host_quantize_q4_0(a)) == bytes([0x00, 0xBC, 0x50, 0xFC, 0x87, 0x88] + [0x88] * 11 + [0x08])
+    b = np.zeros(32, np.float32)
+    b[[5, 0, 1, 2, 20, 21]] = [-4.0, 2.0, -1.0, 3.9, 0.26, -0.24]
+    assert bytes(pkg.host_quantize_q4_0(b)) == bytes([0x00, 0x38, 0x8C, 0x86, 0x8F, 0x88, 0x98, 0x80] + [0x88] * 10)
     for ty, n_rows, K in ((2, 16, 256), (8, 16, 256), (14, 8, 512)):
         raw = synth.make_weight(ty, n_rows, K, seed=ty)
         assert np.array_equal(pkg.host_dequantize(ty, raw, n_rows * K), orc.dequantize(ty, raw, n_rows * K))

@@ -55,9 +55,10 @@ def test_gemv_matches_q8_oracle(accel, orc, synth, relerr, ty, N, K):
     y = accel.gemv("t.gemv", x, N)
     ref = orc.matmul_q8_from_f32(ty, raw, K, N, x)[0]
     assert relerr(y, ref) <= TOL
-    # the f32 oracle (what strix-backend-cpu computes) differs only by activation rounding
+    # the f32 oracle (what strix-backend-cpu computes) differs only by activation rounding: single rows
+    # of a few blocks cancel badly, everything longer stays within 2e-2
     f32 = orc.matmul_f32(ty, raw, K, N, x, order=1)[0]
-    assert relerr(y, f32) <= 5e-2
+    assert relerr(y, f32) <= (5e-2 if N * K <= 4096 else 2e-2)
 
 
 # Small single-row GEMVs have two forms: rows dealt to waves (any shape) and the flat form (rows that are
@@ -189,3 +190,61 @@ def test_lm_head_argmax_rows(accel, orc, synth):
         # compare through values: a near-tie may legitimately resolve differently under fp32 reassociation
         for t in range(m):
             assert ref[t, got[t]] >= ref[t].max() - 1e-5 * np.abs(ref[t]).max()
+
+
+def _reference_device_test_data(orc, in_dim=15360, out_dim=3840):
+    """The data of the reference's own device test (strix-backend-rocm/src/lib.rs:135-153): LCG
+    0xA5A5_1234, per block one draw for the scale 0.03 + (r % 32) * 0.003 (made f16 by truncating the
+    mantissa, lib.rs:110-119) and four draws for the nibble words; x = 0.5 sin(0.017 i)."""
+    nblk = in_dim // 32
+    total = nblk * out_dim
+    draws, _ = orc.lcg(0xA5A51234, total * 5)
+    draws = draws.reshape(total, 5)
+    sc = (np.float32(0.03) + (draws[:, 0] % 32).astype(np.float32) * np.float32(0.003)).astype(np.float32)
+    bits = sc.view(np.uint32)
+    h = (((bits >> 16) & 0x8000) | ((((bits >> 23) & 0xff).astype(np.int64) - 112) << 10) | ((bits & 0x7fffff) >> 13)).astype(np.uint16)
+    raw = np.empty((total, 18), np.uint8)
+    raw[:, :2] = h.view(np.uint8).reshape(total, 2)
+    raw[:, 2:] = draws[:, 1:].astype("<u4").view(np.uint8).reshape(total, 16)
+    x = (np.sin(np.arange(in_dim, dtype=np.float32) * np.float32(0.017)) * np.float32(0.5)).astype(np.float32)
+    return raw.reshape(-1), x
+
+
+def test_reference_device_test_through_both_gemv_forms(accel, orc):
+    """What WeightAccel::gemv becomes after the swap.  The reference's gemv kernels take fp32 activations
+    and its device test holds them to rel < 1e-3 of the CPU (lib.rs:216-231).  smx_gemv_f32 is that
+    arithmetic; smx_gemv is the decode path's Q8-activation arithmetic and differs from the CPU result by the
+    activation rounding.  Both are measured on the reference's own test data and gated at what they give."""
+    in_dim, out_dim = 15360, 3840
+    raw, x = _reference_device_test_data(orc, in_dim, out_dim)
+    cpu = orc.matmul_f32(2, raw, in_dim, out_dim, x, order=0)[0]     # the test's sequential CPU sum
+    scale = max(float(np.abs(cpu).max()), 1e-6)
+    assert accel.upload_q4_0("t.ref", raw, in_dim, out_dim)
+    e_f32 = float(np.abs(accel.gemv_f32("t.ref", x, out_dim) - cpu).max()) / scale
+    e_q8 = float(np.abs(accel.gemv("t.ref", x, out_dim) - cpu).max()) / scale
+    print(f"reference device test 3840<-15360: gemv_f32 rel {e_f32:.3e}, gemv (Q8 activations) rel {e_q8:.3e}")
+    assert e_f32 < 1e-3           # the reference's bar for the method
+    assert e_f32 < 1e-5           # what fp32 accumulation gives
+    assert e_q8 < 5e-3            # measured 2.4e-3: activation rounding (d = amax/127 per 32-block), above the 1e-3 bar
+    accel.evict("t.ref")
+
+
+@pytest.mark.parametrize("ty,N,K", SHAPES + [(2, 9728, 2560), (8, 2560, 9728), (14, 1000, 3840), (2, 5, 32768)])
+def test_gemv_f32_matches_f32_oracle(accel, orc, synth, relerr, ty, N, K):
+    raw = synth.make_weight(ty, N, K, seed=19 * N + K)
+    x = synth.make_acts(1, K, seed=3 * N + K)
+    _up(accel, ty, "t.f32", raw, K, N)
+    y = accel.gemv_f32("t.f32", x, N)
+    for order in (0, 1):      # both summation orders of strix-backend-cpu (gemma.rs:323-326, mellum.rs:278-293)
+        assert relerr(y, orc.matmul_f32(ty, raw, K, N, x, order=order)[0]) <= 1e-5
+    accel.evict("t.f32")
+
+
+def test_gemv_f32_limits(accel, synth, pkg):
+    raw = synth.make_weight(2, 2, 32768 + 32, seed=1)
+    assert accel.upload_q4_0("t.f32big", raw, 32768 + 32, 2)
+    with pytest.raises(pkg.SmxError) as ei:
+        accel.gemv_f32("t.f32big", np.zeros(32768 + 32, np.float32), 2)
+    assert ei.value.code == -3
+    assert accel.gemv_f32("t.absent", np.zeros(32, np.float32), 1) is None
+    accel.evict("t.f32big")

@@ -240,3 +240,65 @@ def test_moe_layer_rejects_bad_plan(accel, synth, pkg):
     with pytest.raises(pkg.SmxError):   # token index out of range
         accel.moe_layer_q8_dev(8, xs, 2, [(0, 0, 2)], [0, 5], [0.5, 0.5])
     assert accel.moe_layer_q8_dev(12345, xs, 2, [(0, 0, 2)], [0, 1], [0.5, 0.5]) is None
+
+
+@pytest.mark.parametrize("ne,k", [(8, 2), (64, 8), (128, 16), (300, 5), (1024, 64), (5, 5), (64, 1)])
+def test_device_router_matches_oracle(accel, orc, ne, k):
+    """topk_router (kernels.rs:1846-1872) against the CPU routing of mellum.rs:1178-1192: same experts in the
+    same order, weights to fp32 rounding; equal logits keep ascending index order."""
+    rng = np.random.default_rng(ne * 100 + k)
+    for case in range(4):
+        logits = rng.standard_normal(ne).astype(np.float32) * np.float32(2.0)
+        if case == 1:
+            logits = np.round(logits * 2) / 2          # many exact ties
+        if case == 2:
+            logits[:] = np.float32(0.75)                 # all equal: experts 0 .. k - 1 in order
+        if case == 3:
+            logits = logits * np.float32(6.0)            # a peaked distribution (probabilities down to e-40 are told apart)
+        ids, w = accel.moe_route(logits, k)
+        rids, rw = orc.route_topk(logits, k)
+        assert np.array_equal(ids, rids), (case, ids, rids)
+        assert np.abs(w - rw).max() <= 2e-6 * max(float(rw.max()), 1e-30)
+        assert abs(float(w.sum()) - 1.0) < 1e-5
+
+
+@pytest.mark.parametrize("ty", [8, 14])
+def test_moe_decode_graph_serves_each_tokens_own_routing(accel, orc, synth, ty):
+    """Router and expert FFN of a decode token captured once (decode.rs:3053-3203): the replays read the
+    routing the router wrote for THAT token, so each equals the eager host-routed call for its token."""
+    ne, hidden, eff, k, layer = 16, 512, 256, 4, 41
+    gate, up, down = (synth.make_moe_q8 if ty == 8 else synth.make_moe_q6)(ne, hidden, eff, seed=80)
+    assert (accel.upload_moe_q8 if ty == 8 else accel.upload_moe_q6)(layer, gate, up, down, hidden, eff, ne)
+    rng = np.random.default_rng(81)
+    toks = [(rng.standard_normal(ne).astype(np.float32) * 3, synth.make_acts(1, hidden, seed=82 + t)[0]) for t in range(4)]
+    want = []
+    for logits, x in toks:
+        ids, w = accel.moe_route(logits, k)
+        assert np.array_equal(ids, orc.route_topk(logits, k)[0])
+        want.append(accel.moe_ffn(layer, ids, w, x))
+    assert len({tuple(accel.moe_route(l, k)[0]) for l, _ in toks}) > 1           # the tokens do route differently
+    ld, xd, yd = accel.dev_alloc(ne * 4), accel.dev_alloc(hidden * 4), accel.dev_alloc(hidden * 4)
+    idd, wd = accel.dev_alloc(k * 4), accel.dev_alloc(k * 4)
+
+    def step():
+        assert accel.moe_route_dev(ld, ne, k, idd, wd)
+        assert accel.moe_ffn_routed_dev(layer, idd, wd, k, xd, yd)
+
+    accel.h2d(ld, toks[0][0])
+    accel.h2d(xd, toks[0][1])
+    step()                                                                        # scratch sized outside capture
+    assert np.array_equal(accel.d2h(np.empty(hidden, np.float32), yd), want[0])   # eager device-routed == host-routed
+    accel.graph_begin()
+    step()
+    g = accel.graph_end()
+    for t in (1, 2, 3, 0, 2):
+        accel.h2d(ld, toks[t][0])
+        accel.h2d(xd, toks[t][1])
+        accel.h2d(yd, np.zeros(hidden, np.float32))
+        accel.graph_launch(g)
+        accel.sync()
+        assert np.array_equal(accel.d2h(np.empty(hidden, np.float32), yd), want[t]), f"token {t}"
+    accel.graph_destroy(g)
+    for p in (ld, xd, yd, idd, wd):
+        accel.dev_free(p)
+    assert accel.moe_ffn_routed_dev(999, idd, wd, k, xd, yd) is False

@@ -449,3 +449,30 @@ def test_moe_ffn_equals_sum_of_dense_experts(orc, synth, TY):
         a = (g / (1 + np.exp(-g)) * u).astype(np.float32)
         accf += w[0][kk] * orc.matmul_f32(TY, down[e * deb:(e + 1) * deb], eff, hidden, a, 1)[0]
     assert np.abs(y - accf).max() / np.abs(accf).max() < 5e-2
+
+
+def q4_0_literal_blocks():
+    """Two Q4_0 blocks worked out by hand from ggml_quant.rs:212-237 (d = vmax / -8 with vmax the signed
+    value of largest magnitude, q = clamp(trunc(x / d + 8.5), 0, 15), byte j = q[j] | q[j + 16] << 4).
+    A: vmax = +8 -> d = -1 (f16 0xBC00): 8 -> 0, -4 -> 12, 1 -> 7, 0.4 -> 8, 0 -> 8, 3 -> 5, -7 -> 15, 7.9 -> 0.
+    B: vmax = -4 -> d = +0.5 (f16 0x3800): -4 -> 0, 2 -> 12, -1 -> 6, 3.9 -> 16 clamped to 15, 0.26 -> 9, -0.24 -> 8."""
+    a = np.zeros(32, np.float32)
+    a[[0, 1, 2, 3, 16, 17, 31]] = [8.0, -4.0, 1.0, 0.4, 3.0, -7.0, 7.9]
+    a_bytes = bytes([0x00, 0xBC, 0x50, 0xFC, 0x87, 0x88] + [0x88] * 11 + [0x08])
+    b = np.zeros(32, np.float32)
+    b[[5, 0, 1, 2, 20, 21]] = [-4.0, 2.0, -1.0, 3.9, 0.26, -0.24]
+    b_bytes = bytes([0x00, 0x38, 0x8C, 0x86, 0x8F, 0x88, 0x98, 0x80] + [0x88] * 10)
+    return (a, a_bytes), (b, b_bytes)
+
+
+def test_quantize_q4_0_literal_blocks(orc):
+    """Pins the sign convention (the value of largest magnitude maps to nibble 0, the scale takes its
+    negated sign) and the +8.5 truncation, which a round-trip bound cannot tell from their mirror images."""
+    for x, want in q4_0_literal_blocks():
+        got = orc.quantize_q4_0(x)
+        assert bytes(got) == want, (bytes(got).hex(), want.hex())
+    both = np.concatenate([q4_0_literal_blocks()[0][0], q4_0_literal_blocks()[1][0]])
+    assert bytes(orc.quantize_q4_0(both)) == q4_0_literal_blocks()[0][1] + q4_0_literal_blocks()[1][1]
+    # the decoded values land where the encoding says: (q - 8) * d
+    y = orc.dequantize(Q4_0, np.frombuffer(q4_0_literal_blocks()[0][1], np.uint8), 32)
+    assert y[0] == 8.0 and y[1] == -4.0 and y[17] == -7.0 and y[31] == 8.0
