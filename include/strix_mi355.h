@@ -98,9 +98,12 @@ int smx_gemv(smx_ctx* ctx, const char* key, const float* x, size_t in_len, float
 #define SMX_GEMV_F32_MAX_IN_DIM 32768
 int smx_gemv_f32(smx_ctx* ctx, const char* key, const float* x, size_t in_len, float* y, size_t out_cap);
 int smx_gemv_f32_dev(smx_ctx* ctx, const char* key, const float* x_dev, float* y_dev);
-/* Small-batch GEMV, m <= SMX_GEMV_MAX_M rows against one weight read once
- * (kernels.rs:1016-1045, the n-gram verify path): xs[m][in_dim] -> y[m][out_dim]. */
+/* Small batches, m <= SMX_GEMV_ROWS_MAX rows against one weight read once (kernels.rs:1605-1632 q8_gemm_rows,
+ * :830-857 q8_gemm_rows32, :1016-1045 q8i_gemm_rows32; the n-gram verify step and short prefill chunks):
+ * xs[m][in_dim] -> y[m][out_dim].  Up to SMX_GEMV_MAX_M rows of a Q6_K weight and the first few rows of the
+ * others run in the dot4 GEMV, more rows of a Q8_0 / Q4_0 weight in the small-batch kernel on the matrix cores. */
 #define SMX_GEMV_MAX_M 8
+#define SMX_GEMV_ROWS_MAX 32
 int smx_gemv_rows(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim,
                   float* y, size_t y_cap);
 /* WeightAccel::gemv_batch, accel.rs:397; decode.rs:3227-3255.  n (key, x)
@@ -158,9 +161,10 @@ int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, f
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same kernels and results
  * as smx_gemv_dev; the rows quantised for m >= 2 live in a static device array of the library (160 KB per
  * GPU, held until the process ends) instead of the context's growable scratch, so the call never
- * allocates or frees device or host memory.  Limits: m <= SMX_GEMV_MAX_M, in_dim <= SMX_NOALLOC_MAX_IN_DIM
+ * allocates or frees device or host memory.  Limits: m <= SMX_NOALLOC_MAX_ROWS, in_dim <= SMX_NOALLOC_MAX_IN_DIM
  * (SMX_ERR_LIMIT beyond).  All contexts of one GPU share the array: calls that overlap on one GPU race. */
 #define SMX_NOALLOC_MAX_IN_DIM 16384
+#define SMX_NOALLOC_MAX_ROWS 8
 int smx_gemv_noalloc_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 /* Up to 8 single-row GEMVs of one format and in_dim in ONE launch (gate+up, q/k/v, a batch of
  * weights against their activations); 0 if any key is not resident. */

@@ -88,19 +88,34 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 //   MODE 0: MFMAs only            MODE 1: FMAs only (the MFMA result registers are reused unchanged)
 //   MODE 2: MFMAs + FMAs, operand fragments kept in registers
 //   MODE 3: MFMAs + FMAs + the five 16-byte fragment reads per block from LDS (double-buffered in registers)
+//   MODE 4: MFMAs + FMAs, B fragments from LDS, A fragment straight from global memory (fragment-ordered
+//           activations: one coalesced 1 KB load per wave and block), the 16 activation scales of a block
+//           as ONE dword per lane read through a DPP row broadcast in the second FMA
+//   MODE 5: as 4 with the activation scales as four 16-byte LDS reads (16 registers)
 constexpr int kMagicI = 0x4B400000;
 constexpr float kMagicF = 12582912.f;
 
+#define SBK_FMAC_BC(I)                                                                     \
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I " row_mask:0xf bank_mask:0xf" : "+v"(accv[I]) : "v"(dxv), "v"(t[I]))
+__device__ __forceinline__ void scale_accumulate_dpp(float (&accv)[16], const v16i& dn, float dw, float ndw, float dxv) {
+    float t[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) t[i] = fmaf(dw, __int_as_float(dn[i]), ndw);
+    SBK_FMAC_BC(0); SBK_FMAC_BC(1); SBK_FMAC_BC(2); SBK_FMAC_BC(3); SBK_FMAC_BC(4); SBK_FMAC_BC(5); SBK_FMAC_BC(6); SBK_FMAC_BC(7);
+    SBK_FMAC_BC(8); SBK_FMAC_BC(9); SBK_FMAC_BC(10); SBK_FMAC_BC(11); SBK_FMAC_BC(12); SBK_FMAC_BC(13); SBK_FMAC_BC(14); SBK_FMAC_BC(15);
+}
+
 template <int MODE, int NT, int OCC>
 __global__ __launch_bounds__(256, OCC) void mfma_valu_kernel(const float* __restrict__ scales, int nblocks, float* __restrict__ out,
-                                                           unsigned long long* __restrict__ cycles) {
+                                                           unsigned long long* __restrict__ cycles, const v4i* __restrict__ aglob) {
     extern __shared__ __align__(16) char smem[];
     // LDS: 32 KB of operand bytes (what one stage of the GEMM holds) + 64 blocks of scales
-    float* sdx = (float*)(smem + 32768);            // [64][32 tokens]
-    float* sdw = sdx + 64 * 32;                     // [64][128 rows]
+    // LDS: 32 KB of operand bytes (what one stage of the GEMM holds) + 16 blocks of scales
+    float* sdx = (float*)(smem + 32768);            // [16][128 tokens]
+    float* sdw = sdx + 16 * 128;                    // [16][128 rows]
     for (int i = threadIdx.x; i < 32768 / 4; i += 256) ((int*)smem)[i] = (i * 2654435761u) >> 7;
-    for (int i = threadIdx.x; i < 64 * 32; i += 256) sdx[i] = scales[i & 1023];
-    for (int i = threadIdx.x; i < 64 * 128; i += 256) sdw[i] = (float)__half2float(__float2half(scales[(i * 7) & 1023]));
+    for (int i = threadIdx.x; i < 16 * 128; i += 256) sdx[i] = scales[i & 1023];
+    for (int i = threadIdx.x; i < 16 * 128; i += 256) sdw[i] = (float)__half2float(__float2half(scales[(i * 7) & 1023]));
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int half = lane >> 5, col = lane & 31;
@@ -121,17 +136,34 @@ __global__ __launch_bounds__(256, OCC) void mfma_valu_kernel(const float* __rest
 #pragma unroll
     for (int i = 0; i < 16; i++) d[0][i] = d[1][i] = kMagicI + lane + i;
     const unsigned long long t0 = clock64();
+    // MODE 4: lane n of each 16-lane row holds the scale of accumulator n of that row's lane half
+    const int dx_tok = ((lane & 15) >> 2) * 8 + half * 4 + (lane & 3);
+    const v4i* ag = aglob + ((size_t)(blockIdx.x * 4 + wave) * 64) * 64 + lane;   // 64 blocks of 1 KB per wave, reused
+    v4i fa_next = fa;
+    if (MODE >= 4) fa_next = ag[0];
     for (int b = 0; b < nblocks; b++) {
-        const int bs = b & 63;
+        const int bs = b & 15;
         float dxr[16], dw[NT];
+        float dxv = 0.f;
         if (MODE != 0) {
+            if (MODE == 4) {
+                dxv = sdx[bs * 128 + wave * 32 + dx_tok];
+            } else {
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4 v = *(const float4*)(sdx + bs * 32 + g * 8 + half * 4);
-                dxr[4 * g] = v.x; dxr[4 * g + 1] = v.y; dxr[4 * g + 2] = v.z; dxr[4 * g + 3] = v.w;
+                for (int g = 0; g < 4; g++) {
+                    const float4 v = *(const float4*)(sdx + bs * 128 + wave * 32 + g * 8 + half * 4);
+                    dxr[4 * g] = v.x; dxr[4 * g + 1] = v.y; dxr[4 * g + 2] = v.z; dxr[4 * g + 3] = v.w;
+                }
             }
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) dw[nt] = sdw[bs * 128 + nt * 32 + col];
+        }
+        if (MODE >= 4) {
+            fa = fa_next;
+            fa_next = ag[(size_t)((b + 1) & 63) * 64];
+            const int rot = ((b & 3) * 2 + half + col) & 7;
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) fb[nt] = *(const v4i*)(smem + 16384 + nt * 4096 + (col >> 3) * 1024 + (col & 7) * 128 + rot * 16);
         }
         if (MODE == 3) {   // the next block's fragments (the GEMM rotates its reads over the 8 chunks of a 128-byte row)
             const int rot = ((b & 3) * 2 + half + col) & 7;
@@ -151,8 +183,12 @@ __global__ __launch_bounds__(256, OCC) void mfma_valu_kernel(const float* __rest
             if (MODE != 0) {
                 const v16i dn = d[u & 1];
                 const float ndw = -dw[u] * kMagicF;
+                if (MODE == 4) {
+                    scale_accumulate_dpp(acc[u], dn, dw[u], ndw, dxv);
+                } else {
 #pragma unroll
-                for (int i = 0; i < 16; i++) acc[u][i] = fmaf(dxr[i], fmaf(dw[u], __int_as_float(dn[i]), ndw), acc[u][i]);
+                    for (int i = 0; i < 16; i++) acc[u][i] = fmaf(dxr[i], fmaf(dw[u], __int_as_float(dn[i]), ndw), acc[u][i]);
+                }
                 asm volatile("" : "+v"(acc[u][0]), "+v"(acc[u][1]), "+v"(acc[u][2]), "+v"(acc[u][3]), "+v"(acc[u][4]),
                                   "+v"(acc[u][5]), "+v"(acc[u][6]), "+v"(acc[u][7]), "+v"(acc[u][8]), "+v"(acc[u][9]),
                                   "+v"(acc[u][10]), "+v"(acc[u][11]), "+v"(acc[u][12]), "+v"(acc[u][13]),
@@ -275,29 +311,35 @@ int sbk_copy(size_t bytes, int launches, double* us_per_launch) {
 // `row_tiles` (4 or 2): 32-row tiles per wave, i.e. a 32 x 128 or 32 x 64 wave tile; wgs_per_cu 1..4 (4-wave workgroups,
 // so also waves per SIMD; 32 x 128 tiles fit at most 3 per SIMD in registers).
 int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, double* us, double* tops, double* cycles_per_unit) {
-    if (!us || !tops || !cycles_per_unit || mode < 0 || mode > 3 || wgs_per_cu < 1 || wgs_per_cu > 4 || nblocks <= 0) return SBK_ERR;
+    if (!us || !tops || !cycles_per_unit || mode < 0 || mode > 5 || wgs_per_cu < 1 || wgs_per_cu > 4 || nblocks <= 0) return SBK_ERR;
     if ((row_tiles != 4 && row_tiles != 2) || (row_tiles == 4 && wgs_per_cu > 3)) return SBK_ERR;
     Timer t;
     if (!t.ok) return SBK_ERR;
     const unsigned grid = (unsigned)(num_cus() * wgs_per_cu);
-    const size_t lds = 32768 + 64 * 32 * 4 + 64 * 128 * 4;
+    const size_t lds = 32768 + 2 * 16 * 128 * 4;
     float *scales = nullptr, *out = nullptr;
     unsigned long long* cyc = nullptr;
+    v4i* aglob = nullptr;
     int rc = SBK_OK;
-    if (hipMalloc((void**)&scales, 1024 * 4) != hipSuccess || hipMalloc((void**)&out, (size_t)grid * 256 * 4) != hipSuccess ||
-        hipMalloc((void**)&cyc, (size_t)grid * 4 * 8) != hipSuccess)
+    const size_t abytes = (size_t)grid * 4 * 64 * 1024;   // 64 fragment blocks of 1 KB per wave
+    if (hipMalloc((void**)&aglob, abytes) != hipSuccess || hipMemset(aglob, 3, abytes) != hipSuccess) rc = SBK_ERR;
+    if (rc == SBK_OK && (hipMalloc((void**)&scales, 1024 * 4) != hipSuccess || hipMalloc((void**)&out, (size_t)grid * 256 * 4) != hipSuccess ||
+        hipMalloc((void**)&cyc, (size_t)grid * 4 * 8) != hipSuccess))
         rc = SBK_ERR;
     if (rc == SBK_OK) {
         std::vector<float> h(1024);
         for (int i = 0; i < 1024; i++) h[(size_t)i] = 0.001f + 0.00001f * (float)((i * 37) % 1024);
         (void)hipMemcpy(scales, h.data(), 1024 * 4, hipMemcpyHostToDevice);
-        typedef void (*kern_t)(const float*, int, float*, unsigned long long*);
+        typedef void (*kern_t)(const float*, int, float*, unsigned long long*, const v4i*);
         // [mode][tile 4/2][occupancy class: waves per SIMD the register budget is set for]
-        static const kern_t k4lo[4] = {mfma_valu_kernel<0, 4, 2>, mfma_valu_kernel<1, 4, 2>, mfma_valu_kernel<2, 4, 2>, mfma_valu_kernel<3, 4, 2>};
-        static const kern_t k4hi[4] = {mfma_valu_kernel<0, 4, 3>, mfma_valu_kernel<1, 4, 3>, mfma_valu_kernel<2, 4, 3>, mfma_valu_kernel<3, 4, 3>};
-        static const kern_t k2[4] = {mfma_valu_kernel<0, 2, 4>, mfma_valu_kernel<1, 2, 4>, mfma_valu_kernel<2, 2, 4>, mfma_valu_kernel<3, 2, 4>};
+        static const kern_t k4lo[6] = {mfma_valu_kernel<0, 4, 2>, mfma_valu_kernel<1, 4, 2>, mfma_valu_kernel<2, 4, 2>, mfma_valu_kernel<3, 4, 2>,
+                                       mfma_valu_kernel<4, 4, 2>, mfma_valu_kernel<5, 4, 2>};
+        static const kern_t k4hi[6] = {mfma_valu_kernel<0, 4, 3>, mfma_valu_kernel<1, 4, 3>, mfma_valu_kernel<2, 4, 3>, mfma_valu_kernel<3, 4, 3>,
+                                       mfma_valu_kernel<4, 4, 3>, mfma_valu_kernel<5, 4, 3>};
+        static const kern_t k2[6] = {mfma_valu_kernel<0, 2, 4>, mfma_valu_kernel<1, 2, 4>, mfma_valu_kernel<2, 2, 4>, mfma_valu_kernel<3, 2, 4>,
+                                     mfma_valu_kernel<4, 2, 4>, mfma_valu_kernel<5, 2, 4>};
         const kern_t kern = row_tiles == 2 ? k2[mode] : (wgs_per_cu <= 2 ? k4lo[mode] : k4hi[mode]);
-        auto launch = [&]() { hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, t.s, (const float*)scales, nblocks, out, cyc); };
+        auto launch = [&]() { hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, t.s, (const float*)scales, nblocks, out, cyc, (const v4i*)aglob); };
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) rc = SBK_ERR;
         if (rc == SBK_OK) {
             launch();
@@ -323,6 +365,7 @@ int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, double* 
     if (scales) (void)hipFree(scales);
     if (out) (void)hipFree(out);
     if (cyc) (void)hipFree(cyc);
+    if (aglob) (void)hipFree(aglob);
     return rc;
 }
 

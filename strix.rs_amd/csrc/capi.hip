@@ -60,15 +60,35 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restric
 }
 
 // quantise m device rows and run the right matmul kernel into y_dev
+// Which kernel serves m rows: the dot4 GEMV up to SMX_GEMV_MAX_M rows, the small-batch MFMA kernel from there
+// to SMX_SKINNY_MAX_M rows of a Q8_0 / Q4_0 weight of moderate height (skinny_serves), the tiled GEMM otherwise.
+}  // namespace
+
+namespace smx {
+// sc (optional): room for the m quantised rows instead of the context's growable scratch; only for calls
+// the GEMV or the small-batch kernel serves (m <= SMX_SKINNY_MAX_M).
 int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm,
-                   int32_t* dump) {
-    if (m <= SMX_GEMV_MAX_M && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump);  // quantiser fused
-    int rc = ensure_act(c, m, w.K);
+                   int32_t* dump, const ActScratch* sc) {
+    const bool skinny = skinny_serves(w, m);
+    if (!skinny && m <= SMX_GEMV_MAX_M && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump, sc);  // quantiser fused
+    if (sc && !skinny) return fail(c, SMX_ERR_LIMIT, "%zu rows of this weight need the tiled GEMM, which sizes its scratch from the call", m);
+    ActScratch a;
+    int rc;
+    if (sc) {
+        a = *sc;   // m <= 8 rows: the fragment-ordered quants take 8 * K bytes, what m = 8 plain rows take
+    } else {
+        if ((rc = ensure_act(c, std::max(m, skinny ? skinny_xq_bytes(m, w.K) / w.K : m), w.K)) != SMX_OK) return rc;
+        if (skinny && (rc = ensure(c, c->xd, skinny_xd_bytes(m, w.K))) != SMX_OK) return rc;
+        a = ActScratch{(int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p};
+    }
+    if (skinny) return launch_skinny(c, w, xs_dev, m, y_dev, dump, a);
+    rc = launch_actquant(c, xs_dev, m, w.K, a.xq, a.xd, a.xs);
     if (rc != SMX_OK) return rc;
-    rc = launch_actquant(c, xs_dev, m, w.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
-    if (rc != SMX_OK) return rc;
-    return launch_gemm(c, w, (const int8_t*)c->xq.p, (const float*)c->xd.p, m, y_dev, dump);
+    return launch_gemm(c, w, a.xq, a.xd, m, y_dev, dump);
 }
+}  // namespace smx
+
+namespace {
 
 int matmul_host(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, float* y, size_t y_cap,
                 bool force_gemm, const char* who) {
@@ -93,7 +113,7 @@ int matmul_host(smx_ctx* c, const char* key, const float* xs, size_t m, size_t i
         memcpy(c->hx.p, xs, xb);
     }
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, pinned ? (const void*)c->hx.p : (const void*)xs, xb, hipMemcpyHostToDevice, c->stream));
-    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, force_gemm, nullptr);
+    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, force_gemm, nullptr, nullptr);
     if (rc != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(pinned ? (void*)c->hy.p : (void*)y, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
@@ -110,7 +130,7 @@ int smx_gemv(smx_ctx* c, const char* key, const float* x, size_t in_len, float* 
 }
 
 int smx_gemv_rows(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, float* y, size_t y_cap) {
-    if (c && m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv_rows: %zu rows (limit %d)", m, SMX_GEMV_MAX_M);
+    if (c && m > SMX_GEMV_ROWS_MAX) return fail(c, SMX_ERR_LIMIT, "gemv_rows: %zu rows (limit %d)", m, SMX_GEMV_ROWS_MAX);
     return matmul_host(c, key, xs, m, in_dim, y, y_cap, false, "gemv_rows");
 }
 
@@ -228,7 +248,7 @@ int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t
             rc = launch_gemv(c, *w, (const float*)c->xf32.p + t * w->K, mm, (float*)c->yf32.p + t * w->N, nullptr);
         }
     } else {
-        rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr);
+        rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr, nullptr);
     }
     if (rc != SMX_OK) return rc;
     {
@@ -247,8 +267,8 @@ int smx_gemv_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, flo
     if (!key || !xs_dev || !y_dev) return fail(c, SMX_ERR_ARG, "gemv_dev: null argument");
     const Weight* w = find_weight(c, key);
     if (!w) return SMX_NOT_RESIDENT;
-    if (m == 0 || m > SMX_GEMV_MAX_M) return fail(c, SMX_ERR_LIMIT, "gemv_dev: %zu rows (1..%d)", m, SMX_GEMV_MAX_M);
-    return run_matmul_dev(c, *w, xs_dev, m, y_dev, false, nullptr);
+    if (m == 0 || m > SMX_GEMV_ROWS_MAX) return fail(c, SMX_ERR_LIMIT, "gemv_dev: %zu rows (1..%d)", m, SMX_GEMV_ROWS_MAX);
+    return run_matmul_dev(c, *w, xs_dev, m, y_dev, false, nullptr, nullptr);
 }
 
 int smx_gemv_batch_dev(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs_dev, float* const* ys_dev) {
@@ -334,7 +354,7 @@ int smx_gemm_fused_dev(smx_ctx* c, const char* key, int act, const float* a_dev,
     if (m == 0) return fail(c, SMX_ERR_ARG, "gemm_fused_dev: zero rows");
     int rc = gemv_fused_check(c, act, a_dev, b_dev, "gemm_fused_dev");
     if (rc != SMX_OK) return rc;
-    if (act == SMX_ACT_NONE) return run_matmul_dev(c, *w, a_dev, m, y_dev, true, nullptr);
+    if (act == SMX_ACT_NONE) return run_matmul_dev(c, *w, a_dev, m, y_dev, true, nullptr, nullptr);
     if ((rc = ensure_act(c, m, w->K)) != SMX_OK) return rc;
     rc = launch_rows_prod_quant(c, act, a_dev, b_dev, m, w->K, eps, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
     if (rc != SMX_OK) return rc;
@@ -347,7 +367,7 @@ int smx_gemm_dev(smx_ctx* c, const char* key, const float* xs_dev, size_t m, flo
     const Weight* w = find_weight(c, key);
     if (!w) return SMX_NOT_RESIDENT;
     if (m == 0) return fail(c, SMX_ERR_ARG, "gemm_dev: zero rows");
-    return run_matmul_dev(c, *w, xs_dev, m, y_dev, true, nullptr);
+    return run_matmul_dev(c, *w, xs_dev, m, y_dev, true, nullptr, nullptr);
 }
 
 int smx_quantize(smx_ctx* c, const float* x, size_t m, size_t k, int8_t* xq, float* xd, int16_t* xs16) {
@@ -385,7 +405,7 @@ static int block_dots(smx_ctx* c, const char* key, const float* xs, size_t m, si
     if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->work, need * 4)) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
-    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, gemm, (int32_t*)c->work.p);
+    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, gemm, (int32_t*)c->work.p, nullptr);
     if (rc != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(out, c->work.p, need * 4, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));

@@ -18,7 +18,7 @@
 namespace smx {
 
 // 8 rows of at most 16384 elements: quants 8 x 16384, scales and sums 8 x 512 dwords each
-constexpr size_t kNoallocMaxRows = SMX_GEMV_MAX_M;
+constexpr size_t kNoallocMaxRows = SMX_NOALLOC_MAX_ROWS;
 constexpr size_t kNoallocMaxK = SMX_NOALLOC_MAX_IN_DIM;
 constexpr size_t kScratchQ = kNoallocMaxRows * kNoallocMaxK;
 constexpr size_t kScratchD = kNoallocMaxRows * (kNoallocMaxK / 32) * 4;
@@ -66,7 +66,7 @@ extern "C" int smx_gemv_noalloc_dev(smx_ctx* c, const char* key, const float* xs
     const ActScratch sc = {(int8_t*)base, (float*)(base + kScratchQ), (int32_t*)(base + kScratchQ + kScratchD)};
     const bool prof = c->prof_on;   // per-kernel timing creates events on first use: off for this call
     c->prof_on = false;
-    const int rc = launch_gemv(c, *w, xs_dev, m, y_dev, nullptr, &sc);
+    const int rc = run_matmul_dev(c, *w, xs_dev, m, y_dev, false, nullptr, &sc);   // the kernels smx_gemv_dev runs for this call
     c->prof_on = prof;
     return rc;
 }

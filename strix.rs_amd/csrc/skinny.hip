@@ -1,0 +1,372 @@
+// Small-batch matmul on the matrix cores: 5..32 activation rows against one resident Q8_0 / Q4_0 weight
+// that is streamed from HBM exactly once.  Stands in for the reference's token-tile kernels
+// (crates/strix-backend-rocm/src/kernels.rs:1605-1632 q8_gemm_rows, :830-857 q8_gemm_rows32, :1016-1045
+// q8i_gemm_rows32; dispatch decode.rs:1742-1766): the n-gram verify step and short prefill chunks.
+//
+// The dot4 GEMV pays its integer dots and LDS reads once per activation row, the tiled GEMM reads
+// 128-byte row pieces of mostly empty 128-token tiles; this kernel has the GEMV's memory side and the
+// GEMM's arithmetic:
+//   * a workgroup (8 waves, one per CU) owns 32 consecutive weight rows and a slice of K; wave w takes
+//     the 4-block (128 elements per row) pieces w, w + 8, ... of the slice, so the workgroup as a whole
+//     reads 32 contiguous row segments;
+//   * a wave's piece (32 rows x 128 B) goes global -> LDS directly into the wave's own corner of LDS (no
+//     registers, no workgroup barrier), four pieces in flight per wave (128 KB per CU); LDS turns "lane = 16 bytes of one
+//     row" into the MFMA operand "lane = row, k-half", chunk-rotated so the transposed reads spread over
+//     the banks (Q4_0 nibbles land raw and are widened to int8 in a second step);
+//   * v_mfma_i32_32x32x32_i8 with the (up to 32) activation rows as the other operand gives the exact
+//     i32 block dots of 32 tokens x 32 rows; per block acc += dx * (dw * I) as in the prefill GEMM
+//     (magic-constant conversion, activation scale through a DPP row broadcast);
+//   * the 8 waves' partial tiles meet in LDS and are added in wave order (deterministic).  With two K
+//     slices per row group the two workgroups add onto an output the quantiser launch has zeroed:
+//     0 + a + b does not depend on which arrives first.
+// HBM-bound: weight bytes once + m * K activation bytes per workgroup from L2.
+#include <hip/hip_fp16.h>
+
+#include <algorithm>
+
+#include "smx_internal.h"
+
+namespace smx {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int kMagicI = 0x4B400000;       // float 12582912 = 1.5 * 2^23: adding an i32 |I| < 2^22 to its bits adds I to its value
+constexpr float kMagicF = 12582912.f;
+constexpr int kPiece = 32 * 128;          // LDS bytes of one piece: 32 rows x 4 blocks of int8
+constexpr int kWaves = 8;            // one workgroup per CU, two waves per SIMD: 256 registers per lane
+constexpr int kDepth = 4;            // pieces in flight per wave
+constexpr int kWaveLds = 16384;      // LDS bytes per wave
+
+struct SkinnyArgs {
+    const uint16_t* wscales;  // f16 [N][nb]
+    const void* wquants;      // Q8_0: i8 [N][K]; Q4_0: 16 B [N][nb]
+    const int8_t* xq;         // fragment order: [nb][2 k-halves][tslots tokens][16 B] (see skinny_quant_kernel)
+    const float* xd;          // [pieces][tslots][4]: the four block scales of a piece side by side per token slot
+    float* y;                 // [m][N]
+    int* dump;                // optional [m][N][nb] i32 block dots
+    int m, N, nb;
+    int tslots;               // token slots of the fragment-ordered activations: 8, 16 or 32
+    int ksplit;               // K slices per row group (1 or 2)
+    int pieces_per_slice;     // 4-block pieces in a slice
+};
+
+__device__ __forceinline__ float h2f_s(uint16_t h) { return __half2float(__ushort_as_half(h)); }
+__device__ __forceinline__ unsigned sub8s(unsigned x) { return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
+
+#define SMX_SK_FMAC(I)                                                                      \
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I " row_mask:0xf bank_mask:0xf" : "+v"(acc[I]) : "v"(dxv), "v"(t[I]))
+
+// 64 lanes x 16 bytes from global memory straight into LDS (no register round trip): lane i's bytes land at
+// LDS byte address lds_base + 16 * i; lds_base is wave-uniform (M0).  Completion is counted by vmcnt.
+__device__ __forceinline__ void load_to_lds16(const void* g, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(g)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ unsigned lds_addr(const void* p) {
+    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
+}
+
+// What travels in registers for one piece: the activation fragments of its four blocks and the raw scales.
+// (Named members, no arrays: the struct travels by value and must stay in registers.)  The weight bytes
+// go global -> LDS directly and are counted by vmcnt only.
+struct PieceRegs {
+    v4i a0, a1, a2, a3;    // activation fragment of each block: lane = (token lane % 32, k-half lane / 32)
+    uint2 dw;              // four f16 scales of this lane's weight row
+    uint4 dx;              // four f32 scales (one per block) of the token whose accumulators this lane feeds by row broadcast
+};
+// vector-memory loads per piece: 6 that return into registers (issued first), then 4 (Q8_0: 8 rows x 128 B each)
+// or 2 (Q4_0: 16 rows x 64 B of nibbles each) LDS-direct ones
+
+template <bool Q4, bool DUMP>
+__global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p) {
+    extern __shared__ __align__(16) char smem[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int K = p.nb * 32;
+    const int rg = blockIdx.x / p.ksplit, slice = blockIdx.x - rg * p.ksplit;
+    const int r0 = rg * 32;
+    const int piece0 = slice * p.pieces_per_slice;
+    const int npieces_total = (p.nb + 3) >> 2;
+    const int piece_end = min(piece0 + p.pieces_per_slice, npieces_total);
+    // per wave: kDepth landing areas for pieces in flight (Q8_0: 4 KB each, already in operand order; Q4_0: 2 KB of
+    // raw nibbles each) and, for Q4_0, one 4 KB area the widened piece is built in
+    char* mine = smem + wave * kWaveLds;
+    const unsigned mine_lds = __builtin_amdgcn_readfirstlane(lds_addr(mine));
+
+    // loop-invariant lane roles
+    const int wrow = min(r0 + col, p.N - 1);                        // this lane's weight row (MFMA operand and scales)
+    const int atok = min(col, p.m - 1);                             // this lane's token as the other MFMA operand
+    const int dx_tok = min(((lane & 15) >> 2) * 8 + half * 4 + (lane & 3), p.m - 1);   // token of accumulator lane % 16 in this lane half
+    const bool vec_sc = (p.nb & 3) == 0;
+    // Q8_0 landing: lane = [row:3][slot:3] of an 8-row group; the lane fetches chunk (slot - row) % 8 of its row, so
+    // chunk c of row r sits in slot (c + r) % 8 and the transposed fragment reads spread over the banks
+    const int g_rowlo = lane >> 3, g_chunk = ((lane & 7) - g_rowlo) & 7;
+
+    // Every load of a piece, unconditional (a piece index past the slice re-reads the slice's last piece and
+    // is neutralised by zero scales), register loads first, then the LDS-direct ones: kRegLoads + kLdsLoads per piece.
+    auto request = [&](int piece_raw, int slot) -> PieceRegs {
+        PieceRegs r;
+        const int piece = min(piece_raw, piece_end - 1);
+        const int blk0 = piece * 4;
+        {   // with 32 token slots a wave's fragment load is one contiguous kilobyte
+            auto la = [&](int bi) {
+                return *(const v4i*)(p.xq + ((size_t)(min(blk0 + bi, p.nb - 1) * 2 + half) * p.tslots + atok) * 16);
+            };
+            r.a0 = la(0); r.a1 = la(1); r.a2 = la(2); r.a3 = la(3);
+        }
+        const uint16_t* ws = p.wscales + (size_t)wrow * p.nb;
+        r.dx = *(const uint4*)(p.xd + ((size_t)piece * p.tslots + dx_tok) * 4);   // 16 contiguous bytes per token slot
+        if (vec_sc) {
+            r.dw = *(const uint2*)(ws + blk0);
+        } else {   // (the scalar form costs more loads; the waits below are then over-conservative, never too lax)
+            const int last = p.nb - 1;
+            r.dw.x = (unsigned)ws[min(blk0, last)] | ((unsigned)ws[min(blk0 + 1, last)] << 16);
+            r.dw.y = (unsigned)ws[min(blk0 + 2, last)] | ((unsigned)ws[min(blk0 + 3, last)] << 16);
+        }
+        if (Q4) {   // lane = [row:4][block:2]: 64 contiguous bytes of nibbles per row, landing as they are
+            const int b = min(blk0 + (lane & 3), p.nb - 1);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                load_to_lds16((const uint4*)p.wquants + (size_t)min(r0 + j * 16 + (lane >> 2), p.N - 1) * p.nb + b,
+                              mine_lds + slot * 2048 + j * 1024);
+        } else {
+            const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                load_to_lds16((const int8_t*)p.wquants + (size_t)min(r0 + j * 8 + g_rowlo, p.N - 1) * K + koff,
+                              mine_lds + slot * kPiece + j * 1024);
+        }
+        return r;
+    };
+
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    v16i cmagic;
+#pragma unroll
+    for (int i = 0; i < 16; i++) cmagic[i] = kMagicI;
+
+    // The ring is always full: kDepth - 1 younger pieces are in flight behind the one consumed.
+    auto consume = [&](const PieceRegs r, int piece_raw, int slot) {
+        const bool piece_live = piece_raw < piece_end;
+        const int piece = min(piece_raw, piece_end - 1);
+        // the piece's LDS-direct loads are complete once at most the younger pieces' loads are outstanding
+        static_assert(kDepth == 4, "the wait counts below are (kDepth - 1) * loads per piece");
+        if (Q4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");   // 3 * (6 + 2)
+        else asm volatile("s_waitcnt vmcnt(30)" ::: "memory");      // 3 * (6 + 4)
+        const char* buf;
+        if (Q4) {   // widen the raw nibbles (lane = [row:4][block:2]) into the operand-order area
+            char* wide = mine + kDepth * 2048;
+            const char* raw = mine + slot * 2048;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int row = j * 16 + (lane >> 2), bi = lane & 3;
+                const uint4 q = *(const uint4*)(raw + j * 1024 + lane * 16);
+                uint4 lo, hi;
+                lo.x = sub8s(q.x & 0x0f0f0f0fu); hi.x = sub8s((q.x >> 4) & 0x0f0f0f0fu);
+                lo.y = sub8s(q.y & 0x0f0f0f0fu); hi.y = sub8s((q.y >> 4) & 0x0f0f0f0fu);
+                lo.z = sub8s(q.z & 0x0f0f0f0fu); hi.z = sub8s((q.z >> 4) & 0x0f0f0f0fu);
+                lo.w = sub8s(q.w & 0x0f0f0f0fu); hi.w = sub8s((q.w >> 4) & 0x0f0f0f0fu);
+                *(uint4*)(wide + row * 128 + ((2 * bi + row) & 7) * 16) = lo;       // elements 0..15 of the block
+                *(uint4*)(wide + row * 128 + ((2 * bi + 1 + row) & 7) * 16) = hi;   // elements 16..31
+            }
+            // the wave's own LDS writes above are read back by other lanes of the same wave below
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            buf = wide;
+        } else {
+            buf = mine + slot * kPiece;
+        }
+        const int blk0 = piece * 4;
+        const unsigned dwh[4] = {r.dw.x & 0xffffu, r.dw.x >> 16, r.dw.y & 0xffffu, r.dw.y >> 16};
+        const unsigned dxs[4] = {r.dx.x, r.dx.y, r.dx.z, r.dx.w};
+#pragma unroll
+        for (int bi = 0; bi < 4; bi++) {
+            const v4i bfrag = *(const v4i*)(buf + col * 128 + ((2 * bi + half + col) & 7) * 16);
+            const v4i afrag = bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3));
+            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, bfrag, cmagic, 0, 0, 0);
+            const bool live = piece_live && blk0 + bi < p.nb;         // pieces past the slice, blocks past K: clamped loads, zero scale
+            const float dw = live ? h2f_s((uint16_t)dwh[bi]) : 0.f;
+            const float ndw = -dw * kMagicF;                          // exact: dw has 11 significant bits
+            const float dxv = __uint_as_float(dxs[bi]);
+            float t[16];
+#pragma unroll
+            for (int i = 0; i < 16; i++) t[i] = fmaf(dw, __int_as_float(d[i]), ndw);
+            SMX_SK_FMAC(0); SMX_SK_FMAC(1); SMX_SK_FMAC(2); SMX_SK_FMAC(3); SMX_SK_FMAC(4); SMX_SK_FMAC(5); SMX_SK_FMAC(6);
+            SMX_SK_FMAC(7); SMX_SK_FMAC(8); SMX_SK_FMAC(9); SMX_SK_FMAC(10); SMX_SK_FMAC(11); SMX_SK_FMAC(12);
+            SMX_SK_FMAC(13); SMX_SK_FMAC(14); SMX_SK_FMAC(15);
+            if (DUMP) {
+                const int row = r0 + col;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
+                    if (live && tok < p.m && row < p.N) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
+                }
+            }
+        }
+        // the landing area is requested into again right after: every lane's reads of it are done (their
+        // results were used above), and no LDS-direct write may overtake them
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // This wave's pieces: a run of consecutive ones (a wave's scale loads and its 128-byte weight lines then
+    // follow each other in memory); kDepth in flight (requests past the run re-read its last piece).
+    {
+        const int per_wave = (piece_end - piece0 + kWaves - 1) / kWaves;
+        int pc = piece0 + wave * per_wave;
+        const int my_end = min(pc + per_wave, piece_end);
+        auto req = [&](int piece, int slot) { return request(min(piece, my_end - 1), slot); };
+        if (pc < my_end) {   // wave-uniform
+            PieceRegs ra = req(pc, 0), rb = req(pc + 1, 1), rc = req(pc + 2, 2), rd = req(pc + 3, 3);
+            while (true) {
+                consume(ra, pc, 0);
+                if (++pc >= my_end) break;
+                ra = req(pc + 3, 0);
+                consume(rb, pc, 1);
+                if (++pc >= my_end) break;
+                rb = req(pc + 3, 1);
+                consume(rc, pc, 2);
+                if (++pc >= my_end) break;
+                rc = req(pc + 3, 2);
+                consume(rd, pc, 3);
+                if (++pc >= my_end) break;
+                rd = req(pc + 3, 3);
+            }
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no LDS-direct load is left in flight when the area is reused
+
+    // the waves' partial tiles, added in wave order
+    __syncthreads();
+    float* red = (float*)smem;   // [wave][16][64]
+#pragma unroll
+    for (int i = 0; i < 16; i++) red[(wave * 16 + i) * 64 + lane] = acc[i];
+    __syncthreads();
+#pragma unroll
+    for (int i = wave; i < 16; i += kWaves) {   // accumulator index; lane as above
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) s += red[(w * 16 + i) * 64 + lane];
+        const int tok = (i >> 2) * 8 + half * 4 + (i & 3), row = r0 + col;
+        if (tok < p.m && row < p.N) {
+            float* o = p.y + (size_t)tok * p.N + row;
+            if (p.ksplit == 1) *o = s;
+            else atomicAdd(o, s);   // two addends onto a zeroed output: the sum does not depend on their order
+        }
+    }
+}
+#undef SMX_SK_FMAC
+
+// The activation quantiser of this path (arithmetic of actquant_kernel: d = amax / 127, q = rint(x / d),
+// crates/strix-backend-rocm/src/kernels.rs:75-96, 1000-1013) writing the quants in MFMA fragment order:
+// for block b, k-half h, token slot t the 16 bytes xq[t][32 b + 16 h ..] form chunk (b * 2 + h) * tslots + t,
+// so a wave's operand load for a block is one contiguous piece, and so is every wave's store here: one
+// thread per chunk (16 values), its block partner tslots lanes away.  Slots past m are zero.  The block
+// scales go out as [piece = b / 4][token slot][b % 4].  The same launch zeroes the output when two K slices are going to add into it.
+__global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restrict__ x, int m, int nb, int tslots,
+                                                           uint4* __restrict__ xq, float* __restrict__ xd,
+                                                           float4* __restrict__ zero, size_t zero_n4) {
+    const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid < zero_n4) zero[gid] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const size_t nchunks = (size_t)nb * 2 * tslots;
+    const int t = (int)(gid % tslots), h = (int)((gid / tslots) & 1);
+    const size_t b = gid / (2 * (size_t)tslots);
+    const bool live = gid < nchunks && t < m;
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) v[i] = 0.f;
+    if (live) {
+        const float4* src = (const float4*)(x + ((size_t)t * nb + b) * 32 + h * 16);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float4 f = src[i];
+            v[4 * i] = f.x; v[4 * i + 1] = f.y; v[4 * i + 2] = f.z; v[4 * i + 3] = f.w;
+        }
+    }
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) a = fmaxf(a, fabsf(v[i]));
+    a = fmaxf(a, __shfl_xor(a, tslots));   // the other half of the block (tslots = 8, 16 or 32: inside the wave)
+    const float d = a / 127.f;
+    const float inv = d > 0.f ? 1.f / d : 0.f;
+    unsigned w[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        unsigned pk = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) pk |= (unsigned)(max(-127, min(127, (int)rintf(v[4 * i + k] * inv))) & 0xff) << (8 * k);
+        w[i] = pk;
+    }
+    if (gid < nchunks) xq[gid] = make_uint4(w[0], w[1], w[2], w[3]);
+    if (live && h == 0) xd[((b >> 2) * tslots + t) * 4 + (b & 3)] = d;
+}
+
+}  // namespace
+
+// Measured on MI355X (Q8_0 2560 x 9728 / Q4_0 9728 x 2560 / Q8_0 15360 x 3840, quantiser included): 16.1 / 16.8 /
+// 26.3 us at 9 rows and 18.3 / 21 / 32 us at 32 rows, against 23.5 / 22.2 / 25.3 and 24.5 / 24.2 / 27.4 us for the
+// tiled GEMM with split-K; up to 8 rows the dot4 GEMV is faster (13.8 us at 8 rows on the first shape).  With
+// one 32-row group per workgroup, weights of more than about 12000 rows no longer fit one round of workgroups
+// and the tiled GEMM wins.
+bool skinny_serves(const Weight& w, size_t m) {
+    return (w.type == kQ8_0 || w.type == kQ4_0) && m > SMX_GEMV_MAX_M && m <= SMX_SKINNY_MAX_M && w.K >= 128 && w.N <= 12288;
+}
+
+size_t skinny_xq_bytes(size_t m, size_t K) { return (K / 32) * 2 * (m <= 8 ? 8 : (m <= 16 ? 16 : 32)) * 16; }
+size_t skinny_xd_bytes(size_t m, size_t K) { return ((K / 32 + 3) / 4) * (m <= 8 ? 8 : (m <= 16 ? 16 : 32)) * 16; }
+
+// y[m][N] for m <= 32 fp32 rows x[m][K]: quantiser launch (fragment-ordered quants into sc.xq, skinny_xq_bytes(m, K)
+// bytes; scales into sc.xd) and the matmul launch.  dump (optional): out[m][N][K/32].
+int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump, const ActScratch& sc) {
+    if (!skinny_serves(w, m)) return fail(c, SMX_ERR_ARG, "small-batch matmul: weight type %d, %zu rows", (int)w.type, m);
+    if (w.N > (size_t(1) << 24) || w.K > (size_t(1) << 20) || w.N * w.K >= (size_t(1) << 40))
+        return fail(c, SMX_ERR_LIMIT, "small-batch matmul: shape N=%zu K=%zu exceeds the kernel's index range", w.N, w.K);
+    SkinnyArgs p = {};
+    p.wscales = w.scales;
+    p.wquants = w.quants;
+    p.xq = sc.xq;
+    p.xd = sc.xd;
+    p.y = y;
+    p.dump = dump;
+    p.m = (int)m;
+    p.N = (int)w.N;
+    p.nb = (int)(w.K / 32);
+    p.tslots = m <= 8 ? 8 : (m <= 16 ? 16 : 32);
+    const int nrg = (int)((w.N + 31) / 32);
+    const int npieces = (p.nb + 3) / 4;
+    // two K slices per row group when one would leave CUs without a workgroup (and every wave still gets a
+    // piece): the second workgroup costs no further launch
+    int ksplit = c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, 2) : ((nrg <= c->num_cu && npieces >= 2 * kWaves) ? 2 : 1);
+    if (dump || ((uintptr_t)y & 15) != 0 || (m * w.N) % 4 != 0) ksplit = 1;
+    p.ksplit = ksplit;
+    p.pieces_per_slice = (npieces + ksplit - 1) / ksplit;
+    {
+        const size_t threads = (size_t)p.nb * 2 * p.tslots, zero_n4 = ksplit > 1 ? m * w.N / 4 : 0;
+        const size_t grid = (std::max(threads, zero_n4) + 255) / 256;
+        ProfScope ps(c, "skinny_quant");
+        hipLaunchKernelGGL(skinny_quant_kernel, dim3((unsigned)grid), dim3(256), 0, c->stream, x, (int)m, p.nb, p.tslots,
+                           (uint4*)sc.xq, sc.xd, (float4*)y, zero_n4);
+        SMX_HIP(c, hipGetLastError());
+    }
+    const size_t lds = (size_t)kWaves * kWaveLds;   // 128 KB; the reduction reuses the first 32 KB
+    const dim3 grid((unsigned)(nrg * ksplit));
+    ProfScope ps(c, w.type == kQ4_0 ? "skinny_q4_0" : "skinny_q8_0");
+    auto go = [&](auto kern) -> int {
+        int rc = set_dyn_lds(c, kern, lds);
+        if (rc != SMX_OK) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * kWaves), lds, c->stream, p);
+        SMX_HIP(c, hipGetLastError());
+        return SMX_OK;
+    };
+    if (w.type == kQ4_0) return dump ? go(skinny_kernel<true, true>) : go(skinny_kernel<true, false>);
+    return dump ? go(skinny_kernel<false, true>) : go(skinny_kernel<false, false>);
+}
+
+}  // namespace smx

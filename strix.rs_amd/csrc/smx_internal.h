@@ -217,6 +217,10 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
                 const ActScratch* sc = nullptr);
 // y[N] = dequant(W) . x with fp32 activations (no quantiser): the arithmetic of the reference's per-weight gemv.
 int launch_gemv_f32(smx_ctx* c, const Weight& w, const float* x, float* y);
+// Quantise m device rows and run the kernel that serves this (weight, m): the dot4 GEMV, the small-batch MFMA
+// kernel or the tiled GEMM (force_gemm: never the GEMV).  sc: caller-provided room for the quantised rows.
+int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm, int32_t* dump,
+                   const ActScratch* sc);
 // Looks the library's static scratch array up on the context's device (called once by smx_create).
 int noalloc_init(smx_ctx* c);
 // n <= 8 single-row GEMVs of one format and row length in one launch (device pointers).
@@ -242,6 +246,15 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);
+
+// Small-batch matmul on the matrix cores (skinny.hip): m <= SMX_SKINNY_MAX_M fp32 rows against a Q8_0 / Q4_0
+// weight read once (its own quantiser launch + the matmul launch).  dump (optional): out[m][N][K/32] i32.
+#define SMX_SKINNY_MAX_M 32
+bool skinny_serves(const Weight& w, size_t m);
+// bytes of sc.xq the call needs (quants in MFMA fragment order, 8, 16 or 32 token slots)
+size_t skinny_xq_bytes(size_t m, size_t K);
+size_t skinny_xd_bytes(size_t m, size_t K);   // of sc.xd (block scales, piece-major)
+int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y, int32_t* dump, const ActScratch& sc);
 
 int launch_gemm_grouped(smx_ctx* c, QType type, const GemmArgs& args, int ntiles, int nops, const char* name);
 // the weight planes of w as a GEMM operand writing to out

@@ -57,3 +57,47 @@ def test_gemm_declines_and_errors(accel, synth, pkg):
     assert accel.upload_q8_0("t.e", raw, 256, 8)
     with pytest.raises(pkg.SmxError):   # wrong activation length
         accel.prefill_q8_gemm("t.e", np.zeros((16, 128), np.float32), 16, 8)
+
+
+# The small-batch kernel on the matrix cores serves 9..32 rows of a Q8_0 / Q4_0 weight of up to 12288 rows
+# (kernels.rs:830-857, 1016-1045, 1605-1632).  (type, N, K): one and two K slices per row group (two when the row
+# groups alone would leave CUs idle and K has at least 64 blocks), K not a multiple of the 4-block piece, ragged row
+# counts, fewer pieces than waves, the two decode shapes of the benchmark.
+SMALL_BATCH = [(8, 96, 256), (8, 130, 2560), (8, 37, 9728), (2, 130, 2560), (2, 33, 4128), (8, 64, 2592), (2, 1000, 160),
+               (8, 300, 128), (2, 7, 15360), (8, 2560, 9728), (2, 9728, 2560), (8, 12288, 512)]
+
+
+@pytest.mark.parametrize("ty,N,K", SMALL_BATCH)
+def test_small_batch_matches_oracle(accel, orc, synth, relerr, ty, N, K):
+    raw = synth.make_weight(ty, N, K, seed=N + K)
+    assert getattr(accel, UPLOAD[ty])("t.sb", raw, K, N)
+    for m in (9, 16, 17, 32):
+        xs = synth.make_acts(m, K, seed=m + N)
+        ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
+        y = accel.prefill_q8_gemm("t.sb", xs, m, N)               # WeightAccel::prefill_q8_gemm with a short chunk
+        assert y.shape == ref.shape and relerr(y, ref) <= TOL, m
+        assert np.array_equal(accel.gemv_rows("t.sb", xs, N), y)  # the verify-step entry point runs the same kernel
+        assert np.array_equal(accel.prefill_q8_gemm("t.sb", xs, m, N), y)   # two K slices add in either order: same bits
+        if N * K <= 400000:   # the integers behind it, dumped by the same kernel
+            xq, _, _ = orc.actquant(xs, K)
+            dots = accel.gemm_block_dots("t.sb", xs, m, N, K // 32)
+            for t in range(m):
+                assert np.array_equal(dots[t], orc.block_dots(ty, raw, K, N, xq[t])), (m, t)
+    accel.evict("t.sb")
+
+
+def test_small_batch_rows_equal_single_rows(accel, synth, relerr):
+    # row t of a 20-row call is the GEMV of xs[t] (same integers; fp32 association differs), for both kernels' ranges
+    N, K = 520, 4096
+    for ty in (8, 2):
+        raw = synth.make_weight(ty, N, K, seed=ty)
+        xs = synth.make_acts(20, K, seed=5)
+        assert getattr(accel, UPLOAD[ty])("t.sbr", raw, K, N)
+        y = accel.gemv_rows("t.sbr", xs, N)
+        y8 = accel.gemv_rows("t.sbr", xs[:8], N)                    # 8 rows: the dot4 GEMV
+        assert relerr(y[:8], y8) <= TOL
+        for t in (0, 9, 19):
+            assert relerr(y[t], accel.gemv("t.sbr", xs[t], N)) <= TOL
+    with pytest.raises(Exception):
+        accel.gemv_rows("t.sbr", synth.make_acts(33, K, seed=1), N)   # gemv_rows takes up to 32 rows
+    accel.evict("t.sbr")
