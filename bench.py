@@ -11,8 +11,14 @@ The same JSON line carries the other configurations of the metric (Q8_0 / Q6_K G
 MFMA prefill GEMM in TOPS, MoE) under "workloads", the roofline of the dominant kernel and the
 CPU baseline (the oracle's restatement of the reference's CPU matmul, timed on this host).
 
+The same line also carries what the machine allows at these sizes, measured in the same run by the
+measurement-only kernels of strix.rs_amd/libstrix_bench.so (not part of the product library): the cost of
+an empty launch, a kernel that only reads the weight bytes cache-cold (the floor of a GEMV of that size)
+and the int8 GEMM's compute phase alone (MFMA + the two FMAs per output of exact per-block rescaling).
+
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only name,...] [--no-cpu]
 """
+import ctypes
 import argparse
 import importlib.util
 import json
@@ -43,6 +49,72 @@ def _load(name, path, search=None):
     sys.modules[name] = mod
     spec.loader.exec_module(mod)
     return mod
+
+
+class Floors:
+    """ctypes view of libstrix_bench.so (measurement-only kernels)."""
+
+    def __init__(self):
+        path = os.path.join(ROOT, "strix.rs_amd", "libstrix_bench.so")
+        if not os.path.exists(path):
+            raise FileNotFoundError(f"{path} is missing: build it with `python strix.rs_amd/build.py`")
+        L = ctypes.CDLL(path)
+        dp = ctypes.POINTER(ctypes.c_double)
+        L.sbk_empty_launch.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, dp]
+        L.sbk_read_floor.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int, dp]
+        L.sbk_copy.argtypes = [ctypes.c_size_t, ctypes.c_int, dp]
+        L.sbk_mfma_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, dp, dp, dp]
+        self.L = L
+
+    def empty_launch(self, grid, block, launches=2000):
+        d = ctypes.c_double()
+        assert self.L.sbk_empty_launch(grid, block, launches, ctypes.byref(d)) == 1
+        return d.value
+
+    def read_floor(self, nbytes, cold=True, launches=400):
+        """us per launch of a kernel that only reads nbytes (256 x 1024 threads, four 16-byte loads in flight
+        per thread), from rotating buffers of > 1 GB in total (cold) or from one buffer (hot)."""
+        nbytes = nbytes // 16 * 16
+        nbuf = max(2, int(1.2e9 // nbytes)) if cold else 1
+        d = ctypes.c_double()
+        assert self.L.sbk_read_floor(nbytes, nbuf, 256, 1024, 4, launches, ctypes.byref(d)) == 1
+        return d.value
+
+    def copy(self, nbytes, launches=20):
+        d = ctypes.c_double()
+        assert self.L.sbk_copy(nbytes, launches, ctypes.byref(d)) == 1
+        return d.value
+
+    def mfma_valu(self, mode, row_tiles, waves_per_simd, nblocks=4000):
+        us, tops, cyc = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
+        assert self.L.sbk_mfma_valu(mode, row_tiles, waves_per_simd, nblocks, ctypes.byref(us), ctypes.byref(tops), ctypes.byref(cyc)) == 1
+        return {"us": us.value, "TOPS": tops.value, "cycles_per_mfma_per_wave": cyc.value,
+                "simd_cycles_per_mfma": cyc.value / waves_per_simd}
+
+
+def machine_floors(log):
+    """What the machine allows, measured with the measurement-only kernels in this run."""
+    f = Floors()
+    out = {"workload": "machine_floors",
+           "method": "HIP events around back-to-back launches on one stream, like every other workload here"}
+    out["empty_launch_us"] = {f"{g}x{b}": f.empty_launch(g, b) for g, b in ((1, 64), (256, 256), (256, 1024), (512, 256), (1024, 256))}
+    sizes = {"14MB_q4_0_9728x2560": 14008320, "26MB_q8_0_2560x9728": 26460160, "48MB_q6_k_15360x3840": 48384000,
+             "112MB_eight_q4_0_9728x2560": 8 * 14008320}
+    out["read_only_cold_us"] = {k: f.read_floor(v, True, 400 if v < 1e8 else 100) for k, v in sizes.items()}
+    out["read_only_cold_GBps"] = {k: sizes[k] / out["read_only_cold_us"][k] / 1e3 for k in sizes}
+    out["read_only_hot_us"] = {"14MB_q4_0_9728x2560": f.read_floor(14008320, False)}
+    us = f.copy(256 << 20)
+    out["copy_256MiB_GBps_read_plus_write"] = 2 * (256 << 20) / us / 1e3
+    # the int8 GEMM's compute phase alone: 32 x 128 wave tiles, two waves per SIMD (what its registers allow)
+    out["mfma_only"] = f.mfma_valu(0, 4, 2)
+    out["fma_only"] = f.mfma_valu(1, 4, 2)
+    out["mfma_plus_rescale_fma"] = f.mfma_valu(2, 4, 2)
+    out["mfma_plus_rescale_fma_plus_lds_fragment_reads"] = f.mfma_valu(3, 4, 2)
+    out["mfma_plus_rescale_fma_three_waves_per_simd"] = f.mfma_valu(2, 4, 3)
+    out["note"] = ("mfma_only runs at the clock the chip sustains under matrix load; with the two FMAs per output that exact "
+                   "per-block rescaling needs, the vector ALU bounds the rate: mfma_plus_rescale_fma is the ceiling of this arithmetic")
+    log(json.dumps(out))
+    return out
 
 
 def gemv_bytes(ty, N, K, m=1):
@@ -97,7 +169,9 @@ class Bench:
         return (ms / n * 1e3 if n else float("nan")), n
 
     # ------------------------------------------------------------------ GEMV
-    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None):
+    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False):
+        """m rows against rotating weight copies.  m <= 8: the dot4 GEMV (quantiser fused for m = 1); 9..32 rows: the
+        small-batch kernel on the matrix cores; f32: the fp32-activation GEMV (no quantiser)."""
         acc, sy = self.acc, self.synth
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
         algo, wbytes = gemv_bytes(ty, N, K, m)
@@ -117,10 +191,14 @@ class Bench:
         acc.h2d(xd, x)
 
         def step(i):
-            acc.gemv_dev(keys[i % ncopies], xd, m, yd)
+            if f32:
+                acc.gemv_f32_dev(keys[i % ncopies], xd, yd)
+            else:
+                acc.gemv_dev(keys[i % ncopies], xd, m, yd)
 
+        kname = ("gemv_f32_" + KERNEL[ty][5:]) if f32 else (KERNEL[ty] if m <= 8 or ty == Q6_K else "skinny_" + KERNEL[ty][5:])
         ms, wall_ms = self._timed(step, steps, warmup)
-        kus, nk = self._kernel_avg_us(step, steps, warmup, KERNEL[ty])
+        kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
         for k in keys:
             acc.evict(k)
         acc.dev_free(xd)
@@ -129,7 +207,7 @@ class Bench:
         # With one activation row the quantiser is fused: a step is exactly one launch of the GEMV
         # kernel, so the timed region's events give that kernel's average launch duration directly
         # (an event pair per launch adds about 2 us of its own and is reported separately).
-        single = m == 1
+        single = m == 1 or f32
         launch_us = ms / steps * 1e3 if single else kus
         kgbs = algo / (launch_us * 1e-6) / 1e9
         return {
@@ -137,7 +215,7 @@ class Bench:
             "algorithmic_bytes": algo, "weight_bytes": wbytes, "steps": steps, "ms_per_step": ms / steps,
             "wall_ms_per_step": wall_ms / steps, "GBps": gbs, "weight_only_GBps": wbytes * steps / (ms * 1e-3) / 1e9,
             "frac_hbm_peak": gbs / HBM_PEAK_GBS,
-            "kernel": KERNEL[ty], "kernel_avg_us": launch_us, "kernel_avg_us_event_pair": kus, "kernel_launches": nk,
+            "kernel": kname, "kernel_avg_us": launch_us, "kernel_avg_us_event_pair": kus, "kernel_launches": nk,
             "kernel_GBps": kgbs, "kernel_frac_hbm_peak": kgbs / HBM_PEAK_GBS,
             "kernel_timing": ("events around the timed region's back-to-back launches / launches" if single
                               else "event pair around each launch"),
@@ -308,6 +386,59 @@ class Bench:
             "split_k": "splitk_reduce" in names,
         }
 
+    # ------------------------------------------------------------------ decode chain as one graph
+    def decode_chain_graph(self, name, layers=4, hidden=2048, ffn=8192, ne=64, eff=768, k=8, steps=None, warmup=None):
+        """`layers` decoder FFN halves captured once as ONE HIP graph and replayed per token, everything resident and
+        routed on the device: per layer rmsnorm + gate/up GEMVs (one launch), SwiGLU + down GEMV, router logits GEMV,
+        top-k router, the k routed experts' FFN (gate/up, down).  Attention is outside this path.  Q4_0 dense
+        weights, Q8_0 experts and router."""
+        acc, sy = self.acc, self.synth
+        steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
+        base = 50
+        for l in range(layers):
+            assert acc.upload_q4_0(f"{name}.g{l}", sy.make_weight(Q4_0, ffn, hidden, seed=4000 + l), hidden, ffn)
+            assert acc.upload_q4_0(f"{name}.u{l}", sy.make_weight(Q4_0, ffn, hidden, seed=4100 + l), hidden, ffn)
+            assert acc.upload_q4_0(f"{name}.d{l}", sy.make_weight(Q4_0, hidden, ffn, seed=4200 + l), ffn, hidden)
+            assert acc.upload_q8_0(f"{name}.r{l}", sy.make_weight(Q8_0, ne, hidden, seed=4300 + l), hidden, ne)
+            gate, up, down = sy.make_moe_q8(ne, hidden, eff, seed=4400 + l)
+            assert acc.upload_moe_q8(base + l, gate, up, down, hidden, eff, ne)
+        x = sy.make_acts(1, hidden, seed=11)
+        xd, nw, gd, ud, hd, ld, yd = (acc.dev_alloc(n * 4) for n in (hidden, hidden, ffn, ffn, hidden, ne, hidden))
+        idd, wd = acc.dev_alloc(k * 4), acc.dev_alloc(k * 4)
+        acc.h2d(xd, x)
+        acc.h2d(nw, np.ones(hidden, np.float32))
+
+        def chain():
+            cur = xd
+            for l in range(layers):
+                acc.gemv_fused_dev([f"{name}.g{l}", f"{name}.u{l}"], 1, cur, nw, [gd, ud], 1e-6)
+                acc.gemv_fused_dev([f"{name}.d{l}"], 2, gd, ud, [hd])
+                acc.gemv_dev(f"{name}.r{l}", hd, 1, ld)
+                acc.moe_route_dev(ld, ne, k, idd, wd)
+                acc.moe_ffn_routed_dev(base + l, idd, wd, k, hd, yd)
+                cur = yd
+
+        chain()
+        acc.sync()
+        acc.graph_begin()
+        chain()
+        g = acc.graph_end()
+        eager_ms, _ = self._timed(lambda i: chain(), steps, warmup)
+        graph_ms, _ = self._timed(lambda i: acc.graph_launch(g), steps, warmup)
+        acc.graph_destroy(g)
+        for l in range(layers):
+            for t in "gudr":
+                acc.evict(f"{name}.{t}{l}")
+        for p in (xd, nw, gd, ud, hd, ld, yd, idd, wd):
+            acc.dev_free(p)
+        wbytes = layers * (3 * gemv_bytes(Q4_0, ffn, hidden)[1] + gemv_bytes(Q8_0, ne, hidden)[1] + k * 3 * eff * (hidden // 32) * 34)
+        return {"workload": name, "shape": {"layers": layers, "hidden": hidden, "ffn": ffn, "experts": ne, "eff": eff, "top_k": k,
+                                            "launches_per_token": layers * 7},
+                "weight_bytes_per_token": wbytes, "steps": steps, "graph_us_per_token": graph_ms / steps * 1e3,
+                "eager_us_per_token": eager_ms / steps * 1e3, "GBps": wbytes * steps / (graph_ms * 1e-3) / 1e9,
+                "frac_hbm_peak": wbytes * steps / (graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "note": "weights (304 MB) stay in the 256 MB Infinity Cache in part: not a cache-cold figure"}
+
     # ------------------------------------------------------------------ MoE
     def moe(self, name, ne, hidden, eff, k, m, layers, steps=None, warmup=None, ty=Q8_0):
         """Decode (m == 1): rotate over `layers` resident layers (320 MB each) so expert reads are
@@ -380,13 +511,21 @@ class Bench:
         return out
 
 
-def cpu_baseline(seconds=12.0):
-    """The reference's CPU matmul (dequantise a row, f32 dot, rows split over the host's cores:
-    crates/strix-backend-cpu/src/mellum.rs:219-237) as restated by the oracle, on the headline shape."""
+def cpu_baseline(seconds=10.0, gemm_seconds=8.0):
+    """The reference's CPU matmul (dequantise a row, f32 dot, rows split over the host's cores with rayon:
+    crates/strix-backend-cpu/src/mellum.rs:219-237, gemma.rs:318) as restated by the oracle: the headline GEMV, and the
+    batched form (mellum.rs:244-271: a row dequantised once, dotted with every token) on a row sample of the
+    ffn_up GEMM.  Threads: every core this process may run on (the GPU box gives a one-GPU job 16 of its
+    logical cores; both counts are reported)."""
     orc = _load("strix_oracle", os.path.join(ROOT, "oracle", "strix_oracle.py"))
     synth = sys.modules["strix_rs_amd_synth"]
     N, K = 9728, 2560
-    cores = min(os.cpu_count() or 1, 16)
+    logical = os.cpu_count() or 1
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = logical
+    cores = max(1, min(usable, int(os.environ.get("OMP_NUM_THREADS", usable))))
     raws = [synth.make_weight(Q4_0, N, K, seed=1000 + i) for i in range(4)]
     x = synth.make_acts(1, K, seed=7)
     orc.matmul_f32(Q4_0, raws[0], K, N, x, 1, cores)
@@ -396,9 +535,23 @@ def cpu_baseline(seconds=12.0):
         n += 1
     dt = time.perf_counter() - t0
     algo, _ = gemv_bytes(Q4_0, N, K, 1)
-    return {"value": algo * n / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{n} f32 GEMVs of the 9728x2560 Q4_0 weight over {dt:.1f} s, 4 rotating copies, "
-                      f"row-parallel dequantise+dot on {cores} threads", "ms_per_gemv": dt / n * 1e3}
+    out = {"value": algo * n / dt / 1e9, "unit": "GB/s", "cores": cores, "host_logical_cores": logical, "kind": "port",
+           "sample": f"{n} f32 GEMVs of the 9728x2560 Q4_0 weight over {dt:.1f} s, 4 rotating copies, "
+                     f"row-parallel dequantise+dot on {cores} threads", "ms_per_gemv": dt / n * 1e3}
+    # the prefill GEMM on the CPU: 2048 tokens x 3840, a sample of 256 of the 15360 Q8_0 weight rows per pass
+    M, Kg, rows = 2048, 3840, 256
+    rawg = synth.make_weight(Q8_0, rows, Kg, seed=2008)
+    xs = synth.make_acts(M, Kg, seed=8)
+    orc.matmul_f32(Q8_0, rawg, Kg, rows, xs, 1, cores)
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < gemm_seconds:
+        orc.matmul_f32(Q8_0, rawg, Kg, rows, xs, 1, cores)
+        n += 1
+    dt = time.perf_counter() - t0
+    out["gemm"] = {"value": 2.0 * M * rows * Kg * n / dt / 1e9, "unit": "GOP/s", "cores": cores, "kind": "port",
+                   "sample": f"{n} passes of 2048 tokens x 3840 against {rows} of the 15360 Q8_0 rows of ffn_up over {dt:.1f} s "
+                             f"(a row dequantised once, f32 dot with every token), {cores} threads"}
+    return out
 
 
 def main():
@@ -408,6 +561,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-floors", action="store_true", help="skip the measurement-only kernels (empty launch, read floor, MFMA+FMA ceiling)")
     ap.add_argument("--no-headline", action="store_true", help="skip the headline GEMV when --only names other workloads")
     ap.add_argument("--tune", default="", help="launch-geometry overrides for sweeps, e.g. gemm_nw=4,gemm_splitk=2")
     a = ap.parse_args()
@@ -423,6 +577,10 @@ def main():
         b.acc.tune(knob, int(value))
     GB = 1 << 30
     work = {}
+    floors = None
+    if want("machine_floors") and not a.no_floors:   # first: it also brings the clocks up before the headline's few steps
+        floors = machine_floors(b.log)
+        work["machine_floors"] = floors
     if a.no_headline and only:
         head = None
     else:
@@ -437,6 +595,9 @@ def main():
         ("q4_0_ffn_decode_block_2560x9728", lambda: b.ffn_block("q4_0_ffn_decode_block_2560x9728", Q4_0, 2560, 9728, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
+        ("q8_0_small_batch_2560x9728_m16", lambda: b.gemv("q8_0_small_batch_2560x9728_m16", Q8_0, 2560, 9728, 16, int(1.1 * GB))),
+        ("q8_0_small_batch_2560x9728_m32", lambda: b.gemv("q8_0_small_batch_2560x9728_m32", Q8_0, 2560, 9728, 32, int(1.1 * GB))),
+        ("q4_0_gemv_f32_9728x2560", lambda: b.gemv("q4_0_gemv_f32_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB), f32=True)),
         ("q6_k_gemv_15360x3840", lambda: b.gemv("q6_k_gemv_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB))),
         ("q6_k_lm_head_262144x3840", lambda: b.gemv("q6_k_lm_head_262144x3840", Q6_K, 262144, 3840, 1, int(1.6 * GB),
                                                      steps=max(10, a.steps // 10), warmup=2)),
@@ -447,6 +608,7 @@ def main():
         ("q8_0_ffn_prefill_block_m2048", lambda: b.ffn_prefill_block("q8_0_ffn_prefill_block_m2048", Q8_0, 3840, 15360, 2048)),
         ("gemm_q6_k_ffn_up", lambda: b.gemm("gemm_q6_k_ffn_up", Q6_K, 2048, 15360, 3840)),
         ("gemm_q6_k_ffn_down", lambda: b.gemm("gemm_q6_k_ffn_down", Q6_K, 2048, 3840, 15360)),
+        ("decode_chain_4layers_graph", lambda: b.decode_chain_graph("decode_chain_4layers_graph")),
         ("moe_decode", lambda: b.moe("moe_decode", 64, 2048, 768, 8, 1, layers=4)),
         ("moe_prefill_m512", lambda: b.moe("moe_prefill_m512", 64, 2048, 768, 8, 512, layers=1)),
         ("moe_decode_q6_k", lambda: b.moe("moe_decode_q6_k", 64, 2048, 768, 8, 1, layers=4, ty=Q6_K)),
@@ -466,13 +628,16 @@ def main():
         "metric": "Q4_0 GEMV GB/s (% HBM peak); int8 prefill GEMM TOPS (% MFMA peak)",
         "value": head["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": head["steps"], "warmup": a.warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "u8", "data": "synthetic",
+        "dtype": "int8", "data": "synthetic",
         "config": {"workload": "Q4_0 decode GEMV, weight 9728x2560, 1 token, Q8 activations, cache-cold: "
                                f"{head['weight_copies']} rotating resident weight copies "
                                f"({head['weight_copies'] * head['weight_bytes'] / 1e9:.2f} GB); "
                                "step = activation quantiser + GEMV", "frac_hbm_peak": head["frac_hbm_peak"]},
         "roofline": {"bound": "hbm", "achieved": head["kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": head["kernel_frac_hbm_peak"], "traffic": HEADLINE_TRAFFIC_BYTES, "kernel": head["kernel"],
+                     "frac": head["kernel_frac_hbm_peak"], "traffic": HEADLINE_TRAFFIC_BYTES,
+                     "traffic_source": "constant from profiles/gemv_q4_0_9728x2560_hbm_traffic.md (rocprofv3 FETCH_SIZE + WRITE_SIZE "
+                                       "scaled by a 256 MiB copy), not measured by this run",
+                     "kernel": head["kernel"],
                      "kernel_avg_us": head["kernel_avg_us"], "kernel_avg_us_event_pair": head["kernel_avg_us_event_pair"],
                      "algorithmic_bytes_per_launch": head["algorithmic_bytes"],
                      "method": "HIP events on the launch stream around the K back-to-back launches of the timed "
@@ -482,9 +647,20 @@ def main():
             "frac_int8_mfma_peak": best_gemm["frac_int8_peak"],
             "roofline": {"bound": "mfma", "achieved": best_gemm["kernel_TOPS"], "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                          "frac": best_gemm["kernel_frac_int8_peak"],
-                         "traffic": GEMM_TRAFFIC_BYTES.get(best_gemm["workload"]), "kernel": best_gemm["kernel"]}},
+                         "traffic": GEMM_TRAFFIC_BYTES.get(best_gemm["workload"]),
+                         "traffic_source": "constant from profiles/gemm_i8_q8_0_ffn_up_counters.md, not measured by this run",
+                         "kernel": best_gemm["kernel"]}},
         "workloads": work,
     }
+    if floors:
+        floor_us = floors["read_only_cold_us"]["14MB_q4_0_9728x2560"]
+        line["roofline"]["read_only_floor_us"] = floor_us
+        line["roofline"]["kernel_over_floor"] = head["kernel_avg_us"] / floor_us
+        line["roofline"]["empty_launch_us"] = floors["empty_launch_us"]["256x1024"]
+        if best_gemm:
+            ceil = floors["mfma_plus_rescale_fma"]["TOPS"]
+            line["gemm"]["roofline"]["rescale_ceiling_TOPS"] = ceil
+            line["gemm"]["roofline"]["kernel_over_ceiling"] = best_gemm["kernel_TOPS"] / ceil
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline()
     b.acc.close()
