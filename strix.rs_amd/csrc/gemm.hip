@@ -20,16 +20,12 @@
 //   * split-K: grid.z slices of whole stages write fp32 partials that a second kernel sums in slice
 //     order (deterministic, unlike the reference's atomicAdd, kernels.rs:597).
 // Bound: dense int8 MFMA, 2*M*N*K operations.
-#include <hip/hip_fp16.h>
-
 #include <algorithm>
 
+#include "mfma_dev.h"
 #include "smx_internal.h"
 
 namespace smx {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int BN = 128, KB = 4;
 constexpr int GRP = 1024;                   // 8 rows x 128 B of one stage: row r at r * 128, its 16-byte chunk c at slot (c + r) % 8
@@ -39,29 +35,9 @@ constexpr int B_BYTES = 16 * GRP;           // 128 weight rows
 // operation through L2, which is what bounds the kernel after the epilogue FMAs.
 constexpr int a_bytes(int NW) { return 4 * NW * GRP; }
 constexpr int stage_bytes(int NW, bool q6 = false) { return a_bytes(NW) + B_BYTES + (q6 ? 2 : 1) * KB * 128 * 4 + KB * 32 * NW * 4; }
-constexpr float MAGIC_F = 12582912.f;       // 1.5 * 2^23
-constexpr int MAGIC_I = 0x4B400000;
-
-__device__ __forceinline__ float h2f_(uint16_t h) { return __half2float(__ushort_as_half(h)); }
-__device__ __forceinline__ unsigned sub8(unsigned x) { return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
 // four 6-bit quants (low nibbles in lo4, the two high bits in hi2) -> four signed bytes q - 32
 __device__ __forceinline__ unsigned q6_bytes(unsigned lo4, unsigned hi2) {
     return (((lo4 & 0x0f0f0f0fu) | ((hi2 & 0x03030303u) << 4) | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
-}
-
-// 64 lanes x 16 bytes from global memory straight into LDS (no register round trip): lane i's
-// bytes land at LDS byte address lds_base + 16 * i; lds_base is wave-uniform (M0).  Completion is
-// counted by vmcnt.  Written as inline assembly so that the compiler's wait-count insertion does
-// not put vmcnt(0) in front of every later LDS read (it cannot tell the two stage buffers apart);
-// the kernel waits for vmcnt(0) itself before the barrier that publishes a stage.
-__device__ __forceinline__ void load_to_lds16(const void* g, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :
-                 : "s"(lds_base), "v"(g)
-                 : "memory", "m0");
-}
-__device__ __forceinline__ unsigned lds_addr(const void* p) {
-    return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
 }
 
 // Operand fragments of one 32-block.  SUB = 1: one K = 32 MFMA per row tile, a lane holds 16 k of
@@ -77,27 +53,6 @@ struct GemmFrag {
 
 constexpr int FMT_Q8 = 0, FMT_Q4 = 1, FMT_Q6 = 2;
 
-// acc[I] += dx(token of accumulator I) * t[I].  The 16 activation scales a lane needs differ between
-// the two lane halves (MFMA 32x32 output: accumulator i of lane half h is token (i/4)*8 + h*4 + i%4),
-// so the Q6_K variant keeps them ONE per lane -- lane n of every 16-lane row holds the scale of
-// accumulator n for that row's half -- and the multiply-add reads it through a row broadcast (DPP
-// row_newbcast:n): one LDS dword and one register per lane and block instead of 16.  Measured: the
-// Q6_K kernel gains 9 % (its 16 spilled registers are gone); the Q8_0 / Q4_0 kernels, which fit
-// their registers either way, lose 4 % to the broadcast form and keep the 16 scales in registers.
-#define SMX_FMAC_BC(I)                                                                      \
-    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I " row_mask:0xf bank_mask:0xf"        \
-        : "+v"(accv[I])                                                                     \
-        : "v"(dxv), "v"(t[I]))
-__device__ __forceinline__ void scale_accumulate(float (&accv)[16], const v16i& dn, float dw, float ndw, float dxv) {
-    float t[16];
-#pragma unroll
-    for (int i = 0; i < 16; i++) t[i] = fmaf(dw, __int_as_float(dn[i]), ndw);
-    SMX_FMAC_BC(0); SMX_FMAC_BC(1); SMX_FMAC_BC(2); SMX_FMAC_BC(3); SMX_FMAC_BC(4); SMX_FMAC_BC(5); SMX_FMAC_BC(6);
-    SMX_FMAC_BC(7); SMX_FMAC_BC(8); SMX_FMAC_BC(9); SMX_FMAC_BC(10); SMX_FMAC_BC(11); SMX_FMAC_BC(12);
-    SMX_FMAC_BC(13); SMX_FMAC_BC(14); SMX_FMAC_BC(15);
-}
-#undef SMX_FMAC_BC
-
 template <int FMT, bool DUMP, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmArgs p) {
     constexpr bool Q4 = FMT == FMT_Q4, Q6 = FMT == FMT_Q6;
@@ -106,7 +61,8 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     constexpr int BM = 32 * NW, A_BYTES = a_bytes(NW), STAGE_BYTES = stage_bytes(NW, Q6);
     constexpr int BG = 16 / NW;  // 8-row groups of B each wave stages
     extern __shared__ __align__(16) char smem[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int K = p.nb * 32;
     const unsigned smem_base = lds_addr(smem);
 
@@ -186,11 +142,8 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const unsigned sB = sA + A_BYTES;
         const int blk0 = s * KB;
         const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
-        // 8-row groups wholly past the tile's end (ragged expert groups) are not fetched: nothing reads
-        // their LDS rows but lanes whose results are dropped
 #pragma unroll
-        for (int ps = 0; ps < 4; ps++)
-            if (tok0 + (ps * NW + wave) * 8 < M_end) load_to_lds16(p.xq + a_off[ps] + koff, sA + ps * NW * GRP);
+        for (int ps = 0; ps < 4; ps++) load_to_lds16(p.xq, a_off[ps] + koff, sA + ps * NW * GRP);
         if (Q6) {
             const size_t sbi = (size_t)b_off[0] + (s >> 1);
             const char* ql = (const char*)op.wquants + sbi * 128 + (s & 1) * 64 + q6_p * 16;
@@ -200,7 +153,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         } else if (!Q4) {
 #pragma unroll
             for (int ps = 0; ps < BG; ps++)
-                load_to_lds16((const int8_t*)op.wquants + b_off[ps] + koff, sB + ps * NW * GRP);
+                load_to_lds16(op.wquants, b_off[ps] + koff, sB + ps * NW * GRP);
         } else {
             const int bq = min(blk0 + q_bi, p.nb - 1);
 #pragma unroll
@@ -500,9 +453,12 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     p.N = (int)w.N;
     p.ldo = (int)w.N;
     p.nb = (int)(w.K / 32);
-    // 128 x 128 tiles, two workgroups per CU (256 x 128 with one 8-wave workgroup per CU measured 7 % slower)
-    constexpr int nw = 4;
-    const int bm = 32 * nw;
+    // 128 x 128 tiles, two 4-wave workgroups per CU.  Measured alternatives, all slower on every shape tried
+    // (M 512..4096 of both FFN shapes, grouped MoE tiles): 256 x 128 tiles with one 8-wave workgroup per CU
+    // (-7 %); three workgroups per CU with 2-block stages, every operand and scale staged LDS-direct and the
+    // LDS reads software-pipelined (-5..-10 %: the third wave per SIMD raises the instruction issue rate,
+    // and the clock the chip sustains drops by as much).
+    const int bm = 128;
     p.tiles_m = (p.M + bm - 1) / bm;
     p.tiles_n = (p.N + BN - 1) / BN;
     const int T = p.tiles_m * p.tiles_n;
@@ -547,8 +503,10 @@ int launch_gemm_grouped(smx_ctx* c, QType type, const GemmArgs& args, int ntiles
     if (ntiles <= 0) return SMX_OK;
     ProfScope ps(c, name);
     const dim3 grid((unsigned)ntiles, (unsigned)nops, 1);
-    if (type == kQ6_K) return launch_gemm_variant<FMT_Q6, false, 4>(c, args, grid);
-    if (type == kQ8_0) return launch_gemm_variant<FMT_Q8, false, 4>(c, args, grid);
+    GemmArgs p = args;   // one K slice: every stage
+    p.stages_per_slice = (p.nb + KB - 1) / KB;
+    if (type == kQ6_K) return launch_gemm_variant<FMT_Q6, false, 4>(c, p, grid);
+    if (type == kQ8_0) return launch_gemm_variant<FMT_Q8, false, 4>(c, p, grid);
     return fail(c, SMX_ERR_ARG, "grouped gemm: weight type %d not supported", (int)type);
 }
 
