@@ -80,6 +80,14 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         tok0 = tm * BM; row0 = tn * BN; col0 = row0; M_end = p.M; N_end = p.N;
     }
     const GemmOperand op = p.op[blockIdx.y];
+    // Wave roles.  A full tile gives each wave 32 tokens x 128 rows (4 row tiles).  A tile with few live
+    // tokens (the tail of M, a small expert group) would leave three of the four waves idle, so its waves
+    // share the token sub-tiles that are live and split the rows: <= 32 tokens: every wave takes the first
+    // 32 tokens and ONE row tile; <= 64 tokens: two waves per token half, two row tiles each.
+    const int live_tok = M_end - tok0;
+    const int tw = NW == 4 ? (live_tok <= 32 ? 0 : live_tok <= 64 ? (wave & 1) : wave) : wave;   // token sub-tile
+    const int nt_cnt = NW == 4 ? (live_tok <= 32 ? 1 : live_tok <= 64 ? 2 : 4) : 4;              // row tiles of this wave
+    const int nt_base = NW == 4 ? (live_tok <= 32 ? wave : live_tok <= 64 ? (wave >> 1) * 2 : 0) : 0;
 
     const int nstage_total = (p.nb + KB - 1) / KB;
     const int s_begin = blockIdx.z * p.stages_per_slice;
@@ -142,8 +150,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const unsigned sB = sA + A_BYTES;
         const int blk0 = s * KB;
         const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
+        // 8-token groups wholly past the tile's end are not fetched (nothing reads their LDS rows)
 #pragma unroll
-        for (int ps = 0; ps < 4; ps++) load_to_lds16(p.xq, a_off[ps] + koff, sA + ps * NW * GRP);
+        for (int ps = 0; ps < 4; ps++)
+            if ((ps * NW + wave) * 8 < live_tok) load_to_lds16(p.xq, a_off[ps] + koff, sA + ps * NW * GRP);
         if (Q6) {
             const size_t sbi = (size_t)b_off[0] + (s >> 1);
             const char* ql = (const char*)op.wquants + sbi * 128 + (s & 1) * 64 + q6_p * 16;
@@ -263,28 +273,32 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const float* sdw = (const float*)(sB + B_BYTES);
         const float* sdx = sdw + SUB * KB * 128;
         if (Q6) {
-            f.dxv = sdx[bi * BM + wave * 32 + dx_tok];
+            f.dxv = sdx[bi * BM + tw * 32 + dx_tok];
         } else {
 #pragma unroll
-            for (int g = 0; g < 4; g++) f.dx[g] = *(const float4*)(sdx + bi * BM + wave * 32 + g * 8 + half * 4);
+            for (int g = 0; g < 4; g++) f.dx[g] = *(const float4*)(sdx + bi * BM + tw * 32 + g * 8 + half * 4);
         }
+        const char* sBw = sB + nt_base * 4 * GRP;   // this wave's row tiles
+        const float* sdww = sdw + nt_base * 32;
         if (Q6) {
             const int o0 = frag6 + ((2 * bi + col) & 7) * 16, o1 = frag6 + ((2 * bi + 1 + col) & 7) * 16;
-            const int2 a0 = *(const int2*)(sA + wave * 4 * GRP + o0), a1 = *(const int2*)(sA + wave * 4 * GRP + o1);
+            const int2 a0 = *(const int2*)(sA + tw * 4 * GRP + o0), a1 = *(const int2*)(sA + tw * 4 * GRP + o1);
             f.a = v4i{a0.x, a0.y, a1.x, a1.y};
 #pragma unroll
             for (int nt = 0; nt < 4; nt++) {
-                const int2 b0 = *(const int2*)(sB + nt * 4 * GRP + o0), b1 = *(const int2*)(sB + nt * 4 * GRP + o1);
+                if (nt >= nt_cnt) break;
+                const int2 b0 = *(const int2*)(sBw + nt * 4 * GRP + o0), b1 = *(const int2*)(sBw + nt * 4 * GRP + o1);
                 f.b[nt] = v4i{b0.x, b0.y, b1.x, b1.y};
 #pragma unroll
-                for (int jj = 0; jj < SUB; jj++) f.dw[nt][jj] = sdw[(2 * bi + jj) * 128 + nt * 32 + col];
+                for (int jj = 0; jj < SUB; jj++) f.dw[nt][jj] = sdww[(2 * bi + jj) * 128 + nt * 32 + col];
             }
         } else {
-            f.a = *(const v4i*)(sA + wave * 4 * GRP + frag_lane[bi]);
+            f.a = *(const v4i*)(sA + tw * 4 * GRP + frag_lane[bi]);
 #pragma unroll
             for (int nt = 0; nt < 4; nt++) {
-                f.b[nt] = *(const v4i*)(sB + nt * 4 * GRP + frag_lane[bi]);
-                f.dw[nt][0] = sdw[bi * 128 + nt * 32 + col];
+                if (nt >= nt_cnt) break;
+                f.b[nt] = *(const v4i*)(sBw + nt * 4 * GRP + frag_lane[bi]);
+                f.dw[nt][0] = sdww[bi * 128 + nt * 32 + col];
             }
         }
     };
@@ -311,7 +325,8 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
 #pragma unroll
         for (int u = 0; u < 4 * SUB; u++) {
             const int nt = u / SUB, jj = u % SUB;
-            if (u + 1 < 4 * SUB) {
+            if (nt >= nt_cnt) break;
+            if (u + 1 < 4 * SUB && (u + 1) / SUB < nt_cnt) {
                 d[(u + 1) & 1] = mfma_unit(f, u + 1);
                 asm volatile("" : "+v"(d[(u + 1) & 1]));
             }
@@ -329,10 +344,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
                               "+v"(acc[nt][10]), "+v"(acc[nt][11]), "+v"(acc[nt][12]), "+v"(acc[nt][13]),
                               "+v"(acc[nt][14]), "+v"(acc[nt][15]));
             if (DUMP) {
-                const int row = row0 + nt * 32 + col;
+                const int row = row0 + (nt_base + nt) * 32 + col;
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int tok = tok0 + wave * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                    const int tok = tok0 + tw * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
                     if (tok < M_end && row < N_end && blk < p.nb)
                         p.dump[((size_t)tok * p.N + row) * (SUB * p.nb) + SUB * blk + jj] = dn[i] - MAGIC_I;
                 }
@@ -348,7 +363,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     __syncthreads();
     // a wave whose 32 tokens all lie past the tile's end (ragged expert groups, M tails) only helps
     // with the staging: its SIMD time goes to the other workgroup on the CU
-    const bool wave_live = tok0 + wave * 32 < M_end;
+    const bool wave_live = tw * 32 < live_tok;
     // The waves of a workgroup leave the barrier together, and 8 KB of loads per wave queue up in the
     // CU's one address unit (20 cycles per 1 KB load alone, 64 behind three other waves): even waves
     // issue the next stage's loads before block 0, odd waves after it (measured +4 %; spreading them
@@ -385,11 +400,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     float* out = op.out + (size_t)blockIdx.z * p.M * p.ldo;
 #pragma unroll
     for (int nt = 0; nt < 4; nt++) {
-        const int row = row0 + nt * 32 + col;
+        if (nt >= nt_cnt) break;
+        const int row = row0 + (nt_base + nt) * 32 + col;
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            const int tok = tok0 + wave * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
-            if (tok < M_end && row < N_end) out[(size_t)tok * p.ldo + col0 + nt * 32 + col] = acc[nt][i];
+            const int tok = tok0 + tw * 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+            if (tok < M_end && row < N_end) out[(size_t)tok * p.ldo + col0 + (nt_base + nt) * 32 + col] = acc[nt][i];
         }
     }
 }

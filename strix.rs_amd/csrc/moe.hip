@@ -690,6 +690,11 @@ static void build_tiles(const size_t* plan, size_t nplan, size_t rows_per_expert
                 tiles->push_back(t);
             }
     }
+    // Longest first: a tile's time follows the row tiles each of its waves computes (4 with more than 64 live
+    // tokens, 2 up to 64, 1 up to 32), and workgroups start in table order, so the long tiles must not be
+    // the last to start.  Equal-cost tiles keep their order (tiles of one weight strip stay adjacent).
+    auto cost = [](const GemmTile& t) { const int live = t.tok_end - t.tok0; return live > 64 ? 4 : live > 32 ? 2 : 1; };
+    std::stable_sort(tiles->begin(), tiles->end(), [&](const GemmTile& a, const GemmTile& b) { return cost(a) > cost(b); });
 }
 
 }  // namespace smx
