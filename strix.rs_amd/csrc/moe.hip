@@ -87,11 +87,14 @@ __device__ __forceinline__ float route_w(const MoeRoute& r, int i) { return r.w_
 // first, the order of the reference's stable sort), weights renormalised over the chosen k.  Experts more
 // than 87 below the largest logit all get the probability exp(-87) (the fixed-sequence exp clamps its
 // argument) and tie to the lowest index; their weight is below 2e-38 either way.  One wave;
-// lane l holds experts l, l + 64, ...  The softmax denominator is summed in double in a fixed order.
+// lane l holds experts l, l + 64, ... (PL of them: 1 for up to 64 experts, which keeps the k selection
+// rounds at one compare each).  The softmax denominator is summed in double in a fixed order.
 constexpr int kRouterPerLane = 16;   // ne <= 1024
+template <int PL>
 __global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict__ logits, int ne, int k,
                                                          int* __restrict__ ids, float* __restrict__ w) {
 #pragma clang fp contract(off)
+    constexpr int kRouterPerLane = PL;
     const int lane = threadIdx.x;
     float v[kRouterPerLane];
     float mx = -3.40282347e+38f;
@@ -730,7 +733,8 @@ int smx_moe_route_dev(smx_ctx* c, const float* logits_dev, size_t ne, size_t k, 
     if (ne == 0 || ne > 64 * kRouterPerLane || k == 0 || k > 64 || k > ne)
         return fail(c, SMX_ERR_LIMIT, "moe_route_dev: %zu experts, top %zu (up to %d experts, top 64)", ne, k, 64 * kRouterPerLane);
     ProfScope ps(c, "topk_router");
-    hipLaunchKernelGGL(topk_router_kernel, dim3(1), dim3(64), 0, c->stream, logits_dev, (int)ne, (int)k, ids_dev, w_dev);
+    auto kern = ne <= 64 ? topk_router_kernel<1> : ne <= 256 ? topk_router_kernel<4> : topk_router_kernel<kRouterPerLane>;
+    hipLaunchKernelGGL(kern, dim3(1), dim3(64), 0, c->stream, logits_dev, (int)ne, (int)k, ids_dev, w_dev);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
