@@ -96,6 +96,37 @@ __global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict
 #pragma clang fp contract(off)
     constexpr int kRouterPerLane = PL;
     const int lane = threadIdx.x;
+    if (PL == 1) {
+        // Up to 64 experts, one per lane: every cross-lane step is a lane read into a scalar register (no
+        // LDS round trips, which dominate the time of this one-wave kernel).  A lane's rank = the number
+        // of experts that precede it in (probability descending, index ascending) order; rank r < k is pick r.
+        const bool live = lane < ne;
+        const float x = live ? logits[lane] : -3.40282347e+38f;
+        float mx = -3.40282347e+38f;
+#pragma unroll
+        for (int j = 0; j < 64; j++) mx = fmaxf(mx, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j)));
+        const float e = live ? det_expf(x - mx) : 0.f;
+        double sum = 0.0;   // ascending expert index
+#pragma unroll
+        for (int j = 0; j < 64; j++) sum += (double)__int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), j));
+        const float p = live ? e / (float)sum : -1.f;
+        int rank = 0;
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), j));
+            rank += (pj > p || (pj == p && j < lane)) ? 1 : 0;
+        }
+        __shared__ float sel[64];
+        if (live && rank < k) {
+            sel[rank] = p;
+            ids[rank] = lane;
+        }
+        __syncthreads();
+        float wsum = 0.f;   // in pick order, as the reference sums the chosen probabilities
+        for (int i = 0; i < k; i++) wsum += sel[i];
+        if (lane < k) w[lane] = sel[lane] / wsum;
+        return;
+    }
     float v[kRouterPerLane];
     float mx = -3.40282347e+38f;
 #pragma unroll
