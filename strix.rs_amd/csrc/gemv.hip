@@ -29,41 +29,43 @@ struct GemvJob {
     int N;
 };
 struct GemvJobs {
-    GemvJob job[SMX_GEMV_GROUP_MAX];
     // expert indirection (MoE decode routed on the device): job j reads expert ids[slot[j]] of a stacked tensor
     const int* ids;
     int ne;
     unsigned long long blocks_per_expert;
     int slot[SMX_GEMV_GROUP_MAX];
+    GemvJob job[SMX_GEMV_GROUP_MAX];
 };
 
-// The planes of a job's weight, moved to the expert the device-side routing names.
-template <class Ops>
+// The planes of a job's weight; IND: moved to the expert the device-side routing names.  The indirection is
+// compiled only into the kernels that a routed launch uses: with it the plane pointers are no longer
+// known to be wave-uniform, which costs every other GEMV 0.2-0.3 us per launch.
+template <class Ops, bool IND>
 __device__ __forceinline__ GemvW job_weight(const GemvJobs& J, int j) {
     GemvW W = J.job[j].W;
-    if (J.ids) {
+    if (IND) {
         const size_t b0 = (size_t)min(max(J.ids[J.slot[j]], 0), J.ne - 1) * J.blocks_per_expert;
         Ops::advance(W, b0);
     }
     return W;
 }
 
-template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT>
+template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT, bool IND = false>
 __global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, int m, int* __restrict__ dump,
                                                   int dump_per_row) {
     const int nw = NT / 64;
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(job_weight<Ops>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
+    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
                                                        blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
 // Flat form (one activation row): blockIdx.x of gridDim.x workgroups share a job's rows.
 // DUMP: the per-block i32 dots of job 0 are also written to dump[row * dump_per_row + ...].
-template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP>
+template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP, bool IND = false>
 __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, int m, unsigned magic_u,
                                                          int* __restrict__ dump, int dump_per_row) {
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(job_weight<Ops>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u,
+    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u,
                                                dump, dump_per_row);
 }
 
@@ -86,6 +88,10 @@ struct Geom {
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT>
 int launch_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump, int dump_per_row) {
     auto k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP, NT>;
+    if (J.ids) {   // experts chosen on the device: one fp32 activation row per job, no dump
+        if constexpr (MT == 1 && FQ != 0 && !DUMP) k = gemv_kernel<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP, NT, true>;
+        else return fail(c, SMX_ERR_ARG, "gemv: device-routed experts take one fp32 activation row per job");
+    }
     int rc = set_dyn_lds(c, k, g.lds);
     if (rc != SMX_OK) return rc;
     hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(NT), g.lds, c->stream, J, nblk, m, dump, dump_per_row);
@@ -108,6 +114,10 @@ template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP = false>
 int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk, int m, int* dump = nullptr,
                    int dump_per_row = 0) {
     auto k = gemv_flat_kernel<Ops, MT, PRE, GL, FQ, DUMP>;
+    if (J.ids) {   // experts chosen on the device: one fp32 activation row per job, no dump
+        if constexpr (MT == 1 && FQ != 0 && !DUMP) k = gemv_flat_kernel<Ops, MT, PRE, GL, FQ, DUMP, true>;
+        else return fail(c, SMX_ERR_ARG, "gemv: device-routed experts take one fp32 activation row per job");
+    }
     int rc = set_dyn_lds(c, k, g.lds);
     if (rc != SMX_OK) return rc;
     const unsigned upb = std::is_same<Ops, OpsQ6_K>::value ? 4u : (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u);

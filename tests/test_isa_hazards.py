@@ -63,7 +63,7 @@ def test_flat_gemv_waits_for_the_activation_only(tmp_path):
     cmd = [HIPCC if os.path.exists(HIPCC) else "hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
            "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only", os.path.join(ROOT, "strix.rs_amd", "csrc", "gemv.hip"), "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True, timeout=900)
-    ins = _kernel_lines(out.read_text(), "_ZN3smx16gemv_flat_kernelINS_7OpsQ4_0ELi1ELi3ELi16ELi1ELb0EEE")
+    ins = _kernel_lines(out.read_text(), "_ZN3smx16gemv_flat_kernelINS_7OpsQ4_0ELi1ELi3ELi16ELi1ELb0ELb0EEE")
     barrier = next(i for i, l in enumerate(ins) if l.startswith("s_barrier"))
     loads = [i for i, l in enumerate(ins[:barrier]) if l.startswith("global_load")]
     weight_loads = [i for i in loads if ins[i].startswith(("global_load_ushort", "global_load_dwordx4 v")) and "off" in ins[i]]
