@@ -100,8 +100,9 @@ int smx_gemv_f32(smx_ctx* ctx, const char* key, const float* x, size_t in_len, f
 int smx_gemv_f32_dev(smx_ctx* ctx, const char* key, const float* x_dev, float* y_dev);
 /* Small batches, m <= SMX_GEMV_ROWS_MAX rows against one weight read once (kernels.rs:1605-1632 q8_gemm_rows,
  * :830-857 q8_gemm_rows32, :1016-1045 q8i_gemm_rows32; the n-gram verify step and short prefill chunks):
- * xs[m][in_dim] -> y[m][out_dim].  Up to SMX_GEMV_MAX_M rows of a Q6_K weight and the first few rows of the
- * others run in the dot4 GEMV, more rows of a Q8_0 / Q4_0 weight in the small-batch kernel on the matrix cores. */
+ * xs[m][in_dim] -> y[m][out_dim].  Up to SMX_GEMV_MAX_M rows (4 of a Q6_K weight) run in the dot4 GEMV, 9..32 rows
+ * of a Q8_0 / Q4_0 weight of up to 12288 rows in the small-batch kernel on the matrix cores, every other case in the
+ * tiled GEMM; the result does not depend on which. */
 #define SMX_GEMV_MAX_M 8
 #define SMX_GEMV_ROWS_MAX 32
 int smx_gemv_rows(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim,

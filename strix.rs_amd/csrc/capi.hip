@@ -70,7 +70,11 @@ namespace smx {
 int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm,
                    int32_t* dump, const ActScratch* sc) {
     const bool skinny = skinny_serves(w, m);
-    if (!skinny && m <= SMX_GEMV_MAX_M && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump, sc);  // quantiser fused
+    // Q6_K with 5..8 rows: the dot4 GEMV runs its 8-row variant there (35 us on 15360 x 3840, 440 us on a 262144-row
+    // head, LDS- and VALU-bound), the tiled GEMM, whose sparse tiles share their rows out over the waves, 29 / 290 us
+    // for any row count up to 32.  (A caller that brings its own scratch keeps the GEMV: the GEMM sizes its scratch itself.)
+    const bool gemv_rows = m <= SMX_GEMV_MAX_M && (w.type != kQ6_K || m <= 4 || sc != nullptr);
+    if (!skinny && gemv_rows && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump, sc);  // quantiser fused
     if (sc && !skinny) return fail(c, SMX_ERR_LIMIT, "%zu rows of this weight need the tiled GEMM, which sizes its scratch from the call", m);
     ActScratch a;
     int rc;
@@ -239,17 +243,7 @@ int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t
     if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->tab, m * 4)) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
-    if (w->type == kQ6_K && m > SMX_GEMV_MAX_M) {
-        // a Q6_K head is HBM-bound at these row counts: GEMV-sized groups re-read the weights once per
-        // 8 rows, which costs less than a GEMM whose 128-token tiles would be mostly empty
-        rc = SMX_OK;
-        for (size_t t = 0; t < m && rc == SMX_OK; t += SMX_GEMV_MAX_M) {
-            const size_t mm = std::min<size_t>(SMX_GEMV_MAX_M, m - t);
-            rc = launch_gemv(c, *w, (const float*)c->xf32.p + t * w->K, mm, (float*)c->yf32.p + t * w->N, nullptr);
-        }
-    } else {
-        rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr, nullptr);
-    }
+    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr, nullptr);
     if (rc != SMX_OK) return rc;
     {
         ProfScope ps(c, "argmax_rows");

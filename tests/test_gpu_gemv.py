@@ -135,6 +135,21 @@ def test_gemv_rows_batched(accel, orc, synth, relerr, ty, m):
     assert relerr(y[m - 1], y0) <= TOL
 
 
+@pytest.mark.parametrize("m", [2, 4, 5, 8, 20, 32])
+def test_gemv_rows_q6k(accel, orc, synth, relerr, m):
+    # Q6_K: up to 4 rows in the dot4 GEMV, more in the tiled GEMM (whose sparse tiles share their row tiles
+    # out over the waves); the lm_head argmax entry point takes the same route
+    N, K = 300, 2560
+    raw = synth.make_weight(14, N, K, seed=40 + m)
+    xs = synth.make_acts(m, K, seed=50 + m)
+    _up(accel, 14, "t.q6rows", raw, K, N)
+    y = accel.gemv_rows("t.q6rows", xs, N)
+    ref = orc.matmul_q8_from_f32(14, raw, K, N, xs)
+    assert y.shape == ref.shape and relerr(y, ref) <= TOL
+    assert [int(v) for v in accel.lm_head_argmax_rows("t.q6rows", xs, m)] == [int(np.argmax(r)) for r in y]
+    accel.evict("t.q6rows")
+
+
 def test_gemv_rows_long_k_batched(accel, orc, synth, relerr):
     # the batched verify shape: Q8_0 2560 x 9728, M = 8 (large LDS staging, 16-wave groups)
     N, K, m = 2560, 9728, 8

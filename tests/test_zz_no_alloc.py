@@ -1,5 +1,7 @@
 """The allocation-free GEMV entry point (static device scratch) against the ordinary device entry
-point, through the C ABI: same kernels, so the results must be identical bit for bit."""
+point, through the C ABI: where both run the same kernels the results must be identical bit for bit;
+for 5..8 rows of a Q6_K weight the ordinary entry point takes the tiled GEMM (whose scratch grows with
+the call) while this one keeps the GEMV, so there the two agree to the fp32 bar of every other test."""
 import numpy as np
 import pytest
 
@@ -37,13 +39,18 @@ def test_noalloc_gemv_equals_gemv_dev_two_calls_in_a_row(accel, orc, synth, rele
 
 
 @pytest.mark.parametrize("ty,N,K,m", [(14, 70, 3840, 7), (8, 37, 9728, 2), (2, 1000, 2592, 5), (2, 64, 256, 1)])
-def test_noalloc_gemv_other_shapes(accel, synth, ty, N, K, m):
+def test_noalloc_gemv_other_shapes(accel, orc, synth, relerr, ty, N, K, m):
     # Q6_K with more than four rows (two passes over the scratch), a row-per-wave shape, one fused row
     raw = synth.make_weight(ty, N, K, seed=3 * N + m)
     up = {2: accel.upload_q4_0, 8: accel.upload_q8_0, 14: accel.upload_q6_k}[ty]
     assert up("t.nb", raw, K, N)
     xs = synth.make_acts(m, K, seed=90 + m)
-    assert np.array_equal(_run(accel, "t.nb", xs, N, accel.gemv_noalloc_dev), _run(accel, "t.nb", xs, N, accel.gemv_dev))
+    got, want = _run(accel, "t.nb", xs, N, accel.gemv_noalloc_dev), _run(accel, "t.nb", xs, N, accel.gemv_dev)
+    if ty == 14 and m > 4:   # different kernels: same integers, another fp32 summation order
+        assert relerr(got, want) <= 1e-5
+    else:
+        assert np.array_equal(got, want)
+    assert relerr(got, orc.matmul_q8_from_f32(ty, raw, K, N, xs)) <= 1e-5
 
 
 def test_noalloc_gemv_limits_and_declines(accel, synth, pkg):
