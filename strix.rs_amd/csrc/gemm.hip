@@ -70,7 +70,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     // gets a contiguous range of logical tiles so its L2 holds few strips
     int t = blockIdx.x;
     int tok0, row0, col0, M_end, N_end;
+    int op_i = blockIdx.y;
     if (p.tiles) {  // grouped (MoE): tile table, A rows are slots of one expert, B rows that expert's rows
+        // the operands (gate, up) of a tile are neighbours in the launch order, so that the table's order
+        // (longest tiles first) holds for all of them
+        op_i = t % p.nops;
+        t /= p.nops;
         const GemmTile tl = p.tiles[t];
         tok0 = tl.tok0; M_end = tl.tok_end; row0 = tl.row0; N_end = tl.row_end; col0 = tl.col0;
     } else {
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const int tm = t % p.tiles_m, tn = t / p.tiles_m;
         tok0 = tm * BM; row0 = tn * BN; col0 = row0; M_end = p.M; N_end = p.N;
     }
-    const GemmOperand op = p.op[blockIdx.y];
+    const GemmOperand op = p.op[op_i];
     // Wave roles.  A full tile gives each wave 32 tokens x 128 rows (4 row tiles).  A tile with few live
     // tokens (the tail of M, a small expert group) would leave three of the four waves idle, so its waves
     // share the token sub-tiles that are live and split the rows: <= 32 tokens: every wave takes the first
@@ -518,8 +523,9 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
 int launch_gemm_grouped(smx_ctx* c, QType type, const GemmArgs& args, int ntiles, int nops, const char* name) {
     if (ntiles <= 0) return SMX_OK;
     ProfScope ps(c, name);
-    const dim3 grid((unsigned)ntiles, (unsigned)nops, 1);
+    const dim3 grid((unsigned)(ntiles * nops), 1, 1);
     GemmArgs p = args;   // one K slice: every stage
+    p.nops = nops;
     p.stages_per_slice = (p.nb + KB - 1) / KB;
     if (type == kQ6_K) return launch_gemm_variant<FMT_Q6, false, 4>(c, p, grid);
     if (type == kQ8_0) return launch_gemm_variant<FMT_Q8, false, 4>(c, p, grid);

@@ -192,6 +192,7 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int stages_per_slice;   // stages (of 4 blocks) each grid.z slice covers
     int xcd_remap;
+    int nops;               // grouped launches: operands per tile (workgroup x serves tile x / nops, operand x % nops)
 };
 
 // ---- launchers (all enqueue on c->stream; return SMX_OK or an error) ----

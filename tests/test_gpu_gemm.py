@@ -10,6 +10,8 @@ UPLOAD = {2: "upload_q4_0", 8: "upload_q8_0", 14: "upload_q6_k"}
 # long K that triggers split-K, single token
 SHAPES = [
     (8, 128, 128, 128), (2, 128, 128, 128), (8, 37, 96, 256), (2, 37, 96, 256), (8, 1, 300, 32),
+    # at most 32 live tokens in a tile (every wave one row tile): ragged rows, K of 1, 2, 3 and many stages, a 160-token M whose last tile holds 32
+    (8, 32, 13000, 2560), (8, 9, 12500, 9728), (8, 17, 300, 96), (8, 30, 257, 288), (8, 160, 200, 2560),
     (2, 200, 130, 160), (8, 256, 384, 2560), (2, 130, 257, 3840), (8, 64, 128, 15360), (2, 96, 256, 15360),
     # Q6_K (16-element sub-block scales, two K = 16 MFMAs per 32-block): one superblock, ragged, long K with split-K
     (14, 128, 128, 256), (14, 37, 96, 512), (14, 9, 300, 256), (14, 200, 130, 2560), (14, 96, 256, 15360),
@@ -28,6 +30,8 @@ def test_gemm_matches_q8_oracle(accel, orc, synth, relerr, ty, M, N, K):
 
 
 @pytest.mark.parametrize("ty,M,N,K", [(8, 37, 96, 256), (2, 37, 96, 256), (8, 130, 40, 160), (2, 64, 130, 2560),
+                                      (8, 20, 13000, 160), (8, 5, 12400, 96),   # tiles of at most 32 live tokens: one row tile per wave
+
                                       (14, 37, 96, 256), (14, 130, 40, 768), (14, 64, 130, 2560)])
 def test_gemm_block_dots_bit_exact(accel, orc, synth, ty, M, N, K):
     raw = synth.make_weight(ty, N, K, seed=M + N + K)
