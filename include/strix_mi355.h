@@ -160,7 +160,9 @@ int smx_dev_copy(smx_ctx* ctx, void* dst_dev, const void* src_dev, size_t nbytes
 int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 /* smx_gemv_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same kernels and results
- * as smx_gemv_dev; the rows quantised for m >= 2 live in a static device array of the library (160 KB per
+ * as smx_gemv_dev (for 5..8 rows of a Q6_K weight smx_gemv_dev takes the tiled GEMM, whose scratch grows with the
+ * call, and this entry point keeps the dot4 GEMV: same integers, fp32 sums within 1e-5); the rows quantised
+ * for m >= 2 live in a static device array of the library (160 KB per
  * GPU, held until the process ends) instead of the context's growable scratch, so the call never
  * allocates or frees device or host memory.  Limits: m <= SMX_NOALLOC_MAX_ROWS, in_dim <= SMX_NOALLOC_MAX_IN_DIM
  * (SMX_ERR_LIMIT beyond).  All contexts of one GPU share the array: calls that overlap on one GPU race. */
