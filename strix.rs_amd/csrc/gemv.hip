@@ -12,6 +12,7 @@
 // number of unit groups, and the persistent row-per-wave form for the rest.
 // HBM-bound: algorithmic bytes per row are K/32 * {18, 34} (Q4_0, Q8_0) or K/256 * 210 (Q6_K).
 #include <algorithm>
+#include <cstddef>
 #include <type_traits>
 
 #include "gemv_body.h"
@@ -22,19 +23,37 @@ namespace smx {
 // One launch serves up to 8 independent GEMVs of the same format and row length (blockIdx.y picks
 // the job): the gate/up pair or the q/k/v triple of a decode step, or a caller's batch of (key, x)
 // pairs, share one kernel start-up.
-struct GemvJob {
+// A job's launch scalars.  Its first 64 bytes are one line of the kernel-argument segment and hold everything the
+// one-row kernels need before their first weight load, so that a wave's start costs ONE scalar-cache miss: with
+// the fields spread over the segment (and the grid size taken from the hidden arguments) a workgroup paid two
+// misses one after the other before it could request a weight, and a third one in its tail.
+struct alignas(128) GemvJob {
     GemvW W;
-    GemvX X;
+    const float* x;     // fp32 activation row(s), null when they arrive quantised
     float* y;
     int N;
+    int nblk;
+    int n_wgs;          // flat form: workgroups that share the job's rows (the launch's gridDim.x)
+    unsigned magic_u;   // flat form: ceil(2^32 / units per row)
+    // second line: what only some variants read
+    const int8_t* xq;   // quantised rows [m][K], their scales and packed 16-element sums
+    const float* xd;
+    const int* xs;
+    const float* x2;    // activation producer: second operand
+    int prod;           // SMX_ACT_*
+    float eps;
+    int m;              // activation rows
+    __host__ __device__ GemvX X() const { return GemvX{x, xq, xd, xs, x2, prod, eps}; }
+    void set_x(const GemvX& a) { x = a.x; xq = a.xq; xd = a.xd; xs = a.xs; x2 = a.x2; prod = a.prod; eps = a.eps; }
 };
+static_assert(offsetof(GemvJob, xq) == 64, "the first line ends with magic_u");
 struct GemvJobs {
+    GemvJob job[SMX_GEMV_GROUP_MAX];
     // expert indirection (MoE decode routed on the device): job j reads expert ids[slot[j]] of a stacked tensor
     const int* ids;
     int ne;
     unsigned long long blocks_per_expert;
     int slot[SMX_GEMV_GROUP_MAX];
-    GemvJob job[SMX_GEMV_GROUP_MAX];
 };
 
 // The planes of a job's weight; IND: moved to the expert the device-side routing names.  The indirection is
@@ -51,22 +70,20 @@ __device__ __forceinline__ GemvW job_weight(const GemvJobs& J, int j) {
 }
 
 template <class Ops, int MT, int RPW, int PRE, int KS, int LPR, int FQ, bool DUMP, int NT, bool IND = false>
-__global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int nblk, int m, int* __restrict__ dump,
-                                                  int dump_per_row) {
+__global__ __launch_bounds__(NT) void gemv_kernel(const GemvJobs J, int* __restrict__ dump, int dump_per_row) {
     const int nw = NT / 64;
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, dump, dump_per_row,
-                                                       blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
+    gemv_body<Ops, MT, RPW, PRE, KS, LPR, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X(), jb.y, jb.N, jb.nblk, jb.N, MT == 1 ? 1 : jb.m,
+                                                       dump, dump_per_row, blockIdx.x * nw + (threadIdx.x >> 6), gridDim.x * nw);
 }
 
-// Flat form (one activation row): blockIdx.x of gridDim.x workgroups share a job's rows.
+// Flat form (one activation row): blockIdx.x of the job's n_wgs workgroups share its rows.
 // DUMP: the per-block i32 dots of job 0 are also written to dump[row * dump_per_row + ...].
 template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP, bool IND = false>
-__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int nblk, int m, unsigned magic_u,
-                                                         int* __restrict__ dump, int dump_per_row) {
+__global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int* __restrict__ dump, int dump_per_row) {
     const GemvJob& jb = J.job[blockIdx.y];
-    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X, jb.y, jb.N, nblk, jb.N, m, blockIdx.x, gridDim.x, magic_u,
-                                               dump, dump_per_row);
+    gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X(), jb.y, jb.N, jb.nblk, jb.N, MT == 1 ? 1 : jb.m,
+                                               blockIdx.x, jb.n_wgs, jb.magic_u, dump, dump_per_row);
 }
 
 namespace {
@@ -94,7 +111,9 @@ int launch_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nblk,
     }
     int rc = set_dyn_lds(c, k, g.lds);
     if (rc != SMX_OK) return rc;
-    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(NT), g.lds, c->stream, J, nblk, m, dump, dump_per_row);
+    GemvJobs JJ = J;
+    for (int i = 0; i < njobs; i++) { JJ.job[i].nblk = nblk; JJ.job[i].m = m; JJ.job[i].n_wgs = (int)g.grid; JJ.job[i].magic_u = 0; }
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(NT), g.lds, c->stream, JJ, dump, dump_per_row);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
@@ -123,7 +142,9 @@ int launch_flat_fq(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int 
     const unsigned upb = std::is_same<Ops, OpsQ6_K>::value ? 4u : (std::is_same<Ops, OpsQ8_0>::value ? 2u : 1u);
     const unsigned units = (unsigned)nblk * upb;                             // units per row
     const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);   // floor(f * magic / 2^32) = f / units for f < 2^16
-    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, J, nblk, m, magic, dump, dump_per_row);
+    GemvJobs JJ = J;
+    for (int i = 0; i < njobs; i++) { JJ.job[i].nblk = nblk; JJ.job[i].m = m; JJ.job[i].n_wgs = (int)g.grid; JJ.job[i].magic_u = magic; }
+    hipLaunchKernelGGL(k, dim3(g.grid, (unsigned)njobs), dim3(1024), g.lds, c->stream, JJ, dump, dump_per_row);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
 }
@@ -336,7 +357,7 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
         return fail(c, SMX_ERR_LIMIT, "gemv: %zu activation rows of %zu need %zu bytes of LDS (limit 163840)", m, w.K, g.lds);
     GemvJobs J = {};
     J.job[0].W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
-    J.job[0].X = {x, nullptr, nullptr, nullptr};
+    J.job[0].x = x;
     J.job[0].y = y;
     J.job[0].N = (int)w.N;
     if (mt > 1) {
@@ -353,7 +374,7 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
         }
         rc = launch_actquant(c, x, m, w.K, a.xq, a.xd, a.xs);
         if (rc != SMX_OK) return rc;
-        J.job[0].X = {nullptr, a.xq, a.xd, (const int*)a.xs};
+        J.job[0].set_x(GemvX{nullptr, a.xq, a.xd, (const int*)a.xs});
     }
     return launch_jobs(c, w.type, g, J, 1, (int)w.nblk, (int)m, mt, dump, (int)(w.type == kQ6_K ? w.K / 16 : w.K / 32));
 }
@@ -377,11 +398,11 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
             return fail(c, SMX_ERR_LIMIT, "gemv: shape %zu x %zu exceeds the kernel's index range", w.N, w.K);
         maxN = std::max(maxN, w.N);
         J.job[i].W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
-        J.job[i].X = {xs[i], nullptr, nullptr, nullptr};
+        J.job[i].x = xs[i];
         if (prod) {
-            J.job[i].X.x2 = x2s ? x2s[i] : prod->b;
-            J.job[i].X.prod = prod->kind;
-            J.job[i].X.eps = prod->eps;
+            J.job[i].x2 = x2s ? x2s[i] : prod->b;
+            J.job[i].prod = prod->kind;
+            J.job[i].eps = prod->eps;
         }
         J.job[i].y = ys[i];
         J.job[i].N = (int)w.N;
@@ -394,7 +415,7 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
     // quantiser kernel of their own, and the GEMV stages the quantised row.
     if (g.prod && (prod->kind == SMX_ACT_SILU_MUL || prod->kind == SMX_ACT_GEGLU) && w0.K >= kProducerSplitK) {
         const float* bs[SMX_GEMV_GROUP_MAX];
-        for (int i = 0; i < n; i++) bs[i] = J.job[i].X.x2;
+        for (int i = 0; i < n; i++) bs[i] = J.job[i].x2;
         const size_t nb = w0.K / 32;
         int rc;
         if ((rc = ensure(c, c->xq, (size_t)n * w0.K)) != SMX_OK) return rc;
@@ -403,8 +424,8 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
         rc = launch_actprod_quant(c, prod->kind, xs, bs, n, w0.K, (int8_t*)c->xq.p, (float*)c->xd.p, (int32_t*)c->xs.p);
         if (rc != SMX_OK) return rc;
         for (int i = 0; i < n; i++)
-            J.job[i].X = {nullptr, (const int8_t*)c->xq.p + (size_t)i * w0.K, (const float*)c->xd.p + (size_t)i * nb,
-                          (const int*)c->xs.p + (size_t)i * nb};
+            J.job[i].set_x(GemvX{nullptr, (const int8_t*)c->xq.p + (size_t)i * w0.K, (const float*)c->xd.p + (size_t)i * nb,
+                                 (const int*)c->xs.p + (size_t)i * nb});
         g.prod = false;
         g.preq = true;
     }

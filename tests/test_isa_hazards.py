@@ -66,7 +66,7 @@ def test_flat_gemv_waits_for_the_activation_only(tmp_path):
     ins = _kernel_lines(out.read_text(), "_ZN3smx16gemv_flat_kernelINS_7OpsQ4_0ELi1ELi3ELi16ELi1ELb0ELb0EEE")
     barrier = next(i for i, l in enumerate(ins) if l.startswith("s_barrier"))
     loads = [i for i, l in enumerate(ins[:barrier]) if l.startswith("global_load")]
-    weight_loads = [i for i in loads if ins[i].startswith(("global_load_ushort", "global_load_dwordx4 v")) and "off" in ins[i]]
+    weight_loads = [i for i in loads if ins[i].startswith(("global_load_ushort", "global_load_dwordx4 v")) and ins[i].split()[-1] == "off"]      # the activation's loads use the scalar base form
     assert len(weight_loads) == 6                      # three units: 16 bytes of quants + one f16 scale each
     last_weight = weight_loads[-1]
     assert any(i < weight_loads[0] for i in loads)     # the activation is requested first
