@@ -6,20 +6,22 @@
 // The dot4 GEMV pays its integer dots and LDS reads once per activation row, the tiled GEMM reads
 // 128-byte row pieces of mostly empty 128-token tiles; this kernel has the GEMV's memory side and the
 // GEMM's arithmetic:
-//   * a workgroup (8 waves, one per CU) owns 32 consecutive weight rows and a slice of K; wave w takes
-//     the 4-block (128 elements per row) pieces w, w + 8, ... of the slice, so the workgroup as a whole
-//     reads 32 contiguous row segments;
-//   * a wave's piece (32 rows x 128 B) goes global -> LDS directly into the wave's own corner of LDS (no
-//     registers, no workgroup barrier), four pieces in flight per wave (128 KB per CU); LDS turns "lane = 16 bytes of one
-//     row" into the MFMA operand "lane = row, k-half", chunk-rotated so the transposed reads spread over
-//     the banks (Q4_0 nibbles land raw and are widened to int8 in a second step);
+//   * a workgroup (8 or 16 waves) owns up to 32 consecutive weight rows and a slice of K; every wave takes a run
+//     of consecutive 4-block (128 elements per row) pieces of the slice;
+//   * a wave's piece (rows x 128 B) goes global -> LDS directly into the wave's own corner of LDS (no
+//     registers, no workgroup barrier); LDS turns "lane = 16 bytes of one row" into the MFMA operand
+//     "lane = row, k-half", chunk-rotated so the transposed reads spread over the banks (Q4_0 nibbles land
+//     raw and are widened to int8 in a second step).  One piece per wave is in flight: the kernel is bound by
+//     the number of vector-memory instructions a CU can take, not by bytes, and a ring of several pieces per wave
+//     costs re-requested pieces at the end of every run (measured: four in flight 16.4 us, two 14.3, one 13.8 on
+//     Q8_0 2560 x 9728 at 16 rows); the other waves of the CU cover a wave's wait;
 //   * v_mfma_i32_32x32x32_i8 with the (up to 32) activation rows as the other operand gives the exact
 //     i32 block dots of 32 tokens x 32 rows; per block acc += dx * (dw * I) as in the prefill GEMM
 //     (magic-constant conversion, activation scale through a DPP row broadcast);
-//   * the 8 waves' partial tiles meet in LDS and are added in wave order (deterministic).  With two K
+//   * the waves' partial tiles meet in LDS and are added in wave order (deterministic).  With two K
 //     slices per row group the two workgroups add onto an output the quantiser launch has zeroed:
 //     0 + a + b does not depend on which arrives first.
-// HBM-bound: weight bytes once + m * K activation bytes per workgroup from L2.
+// HBM-bound by bytes: weight bytes once + m * K activation bytes per workgroup from L2.
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
@@ -36,9 +38,9 @@ namespace {
 constexpr int kMagicI = 0x4B400000;       // float 12582912 = 1.5 * 2^23: adding an i32 |I| < 2^22 to its bits adds I to its value
 constexpr float kMagicF = 12582912.f;
 constexpr int kPiece = 32 * 128;          // LDS bytes of one piece: 32 rows x 4 blocks of int8
-constexpr int kWaves = 8;            // one workgroup per CU, two waves per SIMD: 256 registers per lane
-constexpr int kDepth = 4;            // pieces in flight per wave
-constexpr int kWaveLds = 16384;      // LDS bytes per wave
+// LDS bytes per wave: the landing area of its piece (Q8_0: 4 KB, already in operand order; Q4_0: 2 KB of raw
+// nibbles and the 4 KB area the widened piece is built in)
+constexpr int wave_lds(bool q4) { return q4 ? 2048 + kPiece : kPiece; }
 
 struct SkinnyArgs {
     const uint16_t* wscales;  // f16 [N][nb]
@@ -51,6 +53,7 @@ struct SkinnyArgs {
     int tslots;               // token slots of the fragment-ordered activations: 8, 16 or 32
     int ksplit;               // K slices per row group (1 or 2)
     int pieces_per_slice;     // 4-block pieces in a slice
+    int rows_per_group;       // weight rows a workgroup owns (<= 32): chosen so that the workgroups fill whole rounds of CUs
 };
 
 __device__ __forceinline__ float h2f_s(uint16_t h) { return __half2float(__ushort_as_half(h)); }
@@ -79,39 +82,42 @@ struct PieceRegs {
     uint2 dw;              // four f16 scales of this lane's weight row
     uint4 dx;              // four f32 scales (one per block) of the token whose accumulators this lane feeds by row broadcast
 };
-// vector-memory loads per piece: 6 that return into registers (issued first), then 4 (Q8_0: 8 rows x 128 B each)
+// vector-memory loads per piece: 6 that return into registers, then up to 4 (Q8_0: 8 rows x 128 B each)
 // or 2 (Q4_0: 16 rows x 64 B of nibbles each) LDS-direct ones
 
-template <bool Q4, bool DUMP>
-__global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p) {
+// NW waves per workgroup: 16 when the launch has at most one workgroup per CU (otherwise a CU would hold 8 waves
+// with one piece in flight each), 8 when two workgroups share a CU.
+template <bool Q4, bool DUMP, int NW>
+__global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
+    constexpr int kWaves = NW;
+    constexpr int kWaveLds = wave_lds(Q4);
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 31, half = lane >> 5;
     const int K = p.nb * 32;
     const int rg = blockIdx.x / p.ksplit, slice = blockIdx.x - rg * p.ksplit;
-    const int r0 = rg * 32;
+    const int R = p.rows_per_group;
+    const int r0 = rg * R;
+    const int r_last = min(r0 + R, p.N) - 1;   // rows of the tile past the group re-read its last row (and are not stored)
     const int piece0 = slice * p.pieces_per_slice;
     const int npieces_total = (p.nb + 3) >> 2;
     const int piece_end = min(piece0 + p.pieces_per_slice, npieces_total);
-    // per wave: kDepth landing areas for pieces in flight (Q8_0: 4 KB each, already in operand order; Q4_0: 2 KB of
-    // raw nibbles each) and, for Q4_0, one 4 KB area the widened piece is built in
     char* mine = smem + wave * kWaveLds;
     const unsigned mine_lds = __builtin_amdgcn_readfirstlane(lds_addr(mine));
 
     // loop-invariant lane roles
-    const int wrow = min(r0 + col, p.N - 1);                        // this lane's weight row (MFMA operand and scales)
+    const int wrow = min(r0 + col, r_last);                         // this lane's weight row (MFMA operand and scales)
     const int atok = min(col, p.m - 1);                             // this lane's token as the other MFMA operand
+    const int nrows = r_last - r0 + 1;                              // rows of this group: load instructions past them are not issued
     const int dx_tok = min(((lane & 15) >> 2) * 8 + half * 4 + (lane & 3), p.m - 1);   // token of accumulator lane % 16 in this lane half
     const bool vec_sc = (p.nb & 3) == 0;
     // Q8_0 landing: lane = [row:3][slot:3] of an 8-row group; the lane fetches chunk (slot - row) % 8 of its row, so
     // chunk c of row r sits in slot (c + r) % 8 and the transposed fragment reads spread over the banks
     const int g_rowlo = lane >> 3, g_chunk = ((lane & 7) - g_rowlo) & 7;
 
-    // Every load of a piece, unconditional (a piece index past the slice re-reads the slice's last piece and
-    // is neutralised by zero scales), register loads first, then the LDS-direct ones: kRegLoads + kLdsLoads per piece.
-    auto request = [&](int piece_raw, int slot) -> PieceRegs {
+    // Every load of a piece: the register loads, then the LDS-direct ones.
+    auto request = [&](int piece) -> PieceRegs {
         PieceRegs r;
-        const int piece = min(piece_raw, piece_end - 1);
         const int blk0 = piece * 4;
         {   // with 32 token slots a wave's fragment load is one contiguous kilobyte
             auto la = [&](int bi) {
@@ -132,14 +138,16 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
             const int b = min(blk0 + (lane & 3), p.nb - 1);
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                load_to_lds16((const uint4*)p.wquants + (size_t)min(r0 + j * 16 + (lane >> 2), p.N - 1) * p.nb + b,
-                              mine_lds + slot * 2048 + j * 1024);
+                if (j * 16 < nrows)   // wave-uniform
+                    load_to_lds16((const uint4*)p.wquants + (size_t)min(r0 + j * 16 + (lane >> 2), r_last) * p.nb + b,
+                                  mine_lds + j * 1024);
         } else {
             const int koff = min(blk0 * 32 + g_chunk * 16, K - 16);
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                load_to_lds16((const int8_t*)p.wquants + (size_t)min(r0 + j * 8 + g_rowlo, p.N - 1) * K + koff,
-                              mine_lds + slot * kPiece + j * 1024);
+                if (j * 8 < nrows)   // wave-uniform
+                    load_to_lds16((const int8_t*)p.wquants + (size_t)min(r0 + j * 8 + g_rowlo, r_last) * K + koff,
+                                  mine_lds + j * 1024);
         }
         return r;
     };
@@ -151,18 +159,12 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
 #pragma unroll
     for (int i = 0; i < 16; i++) cmagic[i] = kMagicI;
 
-    // The ring is always full: kDepth - 1 younger pieces are in flight behind the one consumed.
-    auto consume = [&](const PieceRegs r, int piece_raw, int slot) {
-        const bool piece_live = piece_raw < piece_end;
-        const int piece = min(piece_raw, piece_end - 1);
-        // the piece's LDS-direct loads are complete once at most the younger pieces' loads are outstanding
-        static_assert(kDepth == 4, "the wait counts below are (kDepth - 1) * loads per piece");
-        if (Q4) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");   // 3 * (6 + 2)
-        else asm volatile("s_waitcnt vmcnt(30)" ::: "memory");      // 3 * (6 + 4)
+    auto consume = [&](const PieceRegs r, int piece) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the piece's LDS-direct loads (the compiler does not see them)
         const char* buf;
         if (Q4) {   // widen the raw nibbles (lane = [row:4][block:2]) into the operand-order area
-            char* wide = mine + kDepth * 2048;
-            const char* raw = mine + slot * 2048;
+            char* wide = mine + 2048;
+            const char* raw = mine;
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const int row = j * 16 + (lane >> 2), bi = lane & 3;
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             buf = wide;
         } else {
-            buf = mine + slot * kPiece;
+            buf = mine;
         }
         const int blk0 = piece * 4;
         const unsigned dwh[4] = {r.dw.x & 0xffffu, r.dw.x >> 16, r.dw.y & 0xffffu, r.dw.y >> 16};
@@ -191,7 +193,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
             const v4i bfrag = *(const v4i*)(buf + col * 128 + ((2 * bi + half + col) & 7) * 16);
             const v4i afrag = bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3));
             const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, bfrag, cmagic, 0, 0, 0);
-            const bool live = piece_live && blk0 + bi < p.nb;         // pieces past the slice, blocks past K: clamped loads, zero scale
+            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero scale
             const float dw = live ? h2f_s((uint16_t)dwh[bi]) : 0.f;
             const float ndw = -dw * kMagicF;                          // exact: dw has 11 significant bits
             const float dxv = __uint_as_float(dxs[bi]);
@@ -206,7 +208,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
                     const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
-                    if (live && tok < p.m && row < p.N) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
+                    if (live && tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
                 }
             }
         }
@@ -217,31 +219,13 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
     };
 
     // This wave's pieces: a run of consecutive ones (a wave's scale loads and its 128-byte weight lines then
-    // follow each other in memory); kDepth in flight (requests past the run re-read its last piece).
+    // follow each other in memory), split evenly: the first `rem` waves take one piece more.
     {
-        const int per_wave = (piece_end - piece0 + kWaves - 1) / kWaves;
-        int pc = piece0 + wave * per_wave;
-        const int my_end = min(pc + per_wave, piece_end);
-        auto req = [&](int piece, int slot) { return request(min(piece, my_end - 1), slot); };
-        if (pc < my_end) {   // wave-uniform
-            PieceRegs ra = req(pc, 0), rb = req(pc + 1, 1), rc = req(pc + 2, 2), rd = req(pc + 3, 3);
-            while (true) {
-                consume(ra, pc, 0);
-                if (++pc >= my_end) break;
-                ra = req(pc + 3, 0);
-                consume(rb, pc, 1);
-                if (++pc >= my_end) break;
-                rb = req(pc + 3, 1);
-                consume(rc, pc, 2);
-                if (++pc >= my_end) break;
-                rc = req(pc + 3, 2);
-                consume(rd, pc, 3);
-                if (++pc >= my_end) break;
-                rd = req(pc + 3, 3);
-            }
-        }
+        const int np = piece_end - piece0, base = np / kWaves, rem = np - base * kWaves;
+        const int pc0 = piece0 + wave * base + min(wave, rem);
+        const int my_end = pc0 + base + (wave < rem ? 1 : 0);
+        for (int pc = pc0; pc < my_end; pc++) consume(request(pc), pc);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // no LDS-direct load is left in flight when the area is reused
 
     // the waves' partial tiles, added in wave order
     __syncthreads();
@@ -255,7 +239,7 @@ __global__ __launch_bounds__(64 * kWaves) void skinny_kernel(const SkinnyArgs p)
 #pragma unroll
         for (int w = 0; w < kWaves; w++) s += red[(w * 16 + i) * 64 + lane];
         const int tok = (i >> 2) * 8 + half * 4 + (i & 3), row = r0 + col;
-        if (tok < p.m && row < p.N) {
+        if (tok < p.m && row <= r_last) {
             float* o = p.y + (size_t)tok * p.N + row;
             if (p.ksplit == 1) *o = s;
             else atomicAdd(o, s);   // two addends onto a zeroed output: the sum does not depend on their order
@@ -339,12 +323,21 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
     p.N = (int)w.N;
     p.nb = (int)(w.K / 32);
     p.tslots = m <= 8 ? 8 : (m <= 16 ? 16 : 32);
-    const int nrg = (int)((w.N + 31) / 32);
     const int npieces = (p.nb + 3) / 4;
-    // two K slices per row group when one would leave CUs without a workgroup (and every wave still gets a
-    // piece): the second workgroup costs no further launch
-    int ksplit = c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, 2) : ((nrg <= c->num_cu && npieces >= 2 * kWaves) ? 2 : 1);
+    // Rows per workgroup and K slices: one workgroup per CU, so the launch takes ceil(workgroups / CUs) rounds.  Two K
+    // slices when a single round of 32-row groups would leave CUs without work (and every wave still gets a piece);
+    // then as few rows per group as keep the number of rounds (a last round of a few 32-row workgroups costs
+    // as much as a full one, and 19-row groups in two full rounds are 40 % less work per CU than 32-row groups in 1.2).
+    int nrg = (int)((w.N + 31) / 32);
+    int ksplit = c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, 2) : ((nrg <= c->num_cu && npieces >= 16) ? 2 : 1);
     if (dump || ((uintptr_t)y & 15) != 0 || (m * w.N) % 4 != 0) ksplit = 1;
+    {
+        const int rounds = (nrg * ksplit + c->num_cu - 1) / c->num_cu;
+        const int groups = rounds * c->num_cu / ksplit;            // row groups that fit these rounds
+        const int R = std::max(8, std::min(32, (int)((w.N + groups - 1) / groups)));   // (below 8 rows a group is all padding)
+        p.rows_per_group = R;
+        nrg = (int)((w.N + p.rows_per_group - 1) / p.rows_per_group);
+    }
     p.ksplit = ksplit;
     p.pieces_per_slice = (npieces + ksplit - 1) / ksplit;
     {
@@ -355,18 +348,25 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
                            (uint4*)sc.xq, sc.xd, (float4*)y, zero_n4);
         SMX_HIP(c, hipGetLastError());
     }
-    const size_t lds = (size_t)kWaves * kWaveLds;   // 128 KB; the reduction reuses the first 32 KB
-    const dim3 grid((unsigned)(nrg * ksplit));
-    ProfScope ps(c, w.type == kQ4_0 ? "skinny_q4_0" : "skinny_q8_0");
+    const bool q4 = w.type == kQ4_0;
+    const int nwg = nrg * ksplit;
+    const int nw = nwg <= c->num_cu ? 16 : 8;   // waves per workgroup (see the kernel)
+    const size_t lds = (size_t)nw * wave_lds(q4);   // the reduction reuses the first nw * 4 KB
+    const dim3 grid((unsigned)nwg);
+    ProfScope ps(c, q4 ? "skinny_q4_0" : "skinny_q8_0");
     auto go = [&](auto kern) -> int {
         int rc = set_dyn_lds(c, kern, lds);
         if (rc != SMX_OK) return rc;
-        hipLaunchKernelGGL(kern, grid, dim3(64 * kWaves), lds, c->stream, p);
+        hipLaunchKernelGGL(kern, grid, dim3(64 * nw), lds, c->stream, p);
         SMX_HIP(c, hipGetLastError());
         return SMX_OK;
     };
-    if (w.type == kQ4_0) return dump ? go(skinny_kernel<true, true>) : go(skinny_kernel<true, false>);
-    return dump ? go(skinny_kernel<false, true>) : go(skinny_kernel<false, false>);
+    if (nw == 16) {
+        if (q4) return dump ? go(skinny_kernel<true, true, 16>) : go(skinny_kernel<true, false, 16>);
+        return dump ? go(skinny_kernel<false, true, 16>) : go(skinny_kernel<false, false, 16>);
+    }
+    if (q4) return dump ? go(skinny_kernel<true, true, 8>) : go(skinny_kernel<true, false, 8>);
+    return dump ? go(skinny_kernel<false, true, 8>) : go(skinny_kernel<false, false, 8>);
 }
 
 }  // namespace smx
