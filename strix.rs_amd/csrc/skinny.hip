@@ -40,7 +40,8 @@ constexpr float kMagicF = 12582912.f;
 constexpr int kPiece = 32 * 128;          // LDS bytes of one piece: 32 rows x 4 blocks of int8
 // LDS bytes per wave: the landing area of its piece (Q8_0: 4 KB, already in operand order; Q4_0: 2 KB of raw
 // nibbles and the 4 KB area the widened piece is built in)
-constexpr int wave_lds(bool q4) { return q4 ? 2048 + kPiece : kPiece; }
+// and, when the activation fragments travel through LDS too (ALDS, up to 16 token slots), 2 KB for those of a piece
+constexpr int wave_lds(bool q4, bool alds) { return (q4 ? 2048 + kPiece : kPiece) + (alds ? 2048 : 0); }
 
 struct SkinnyArgs {
     const uint16_t* wscales;  // f16 [N][nb]
@@ -87,10 +88,13 @@ struct PieceRegs {
 
 // NW waves per workgroup: 16 when the launch has at most one workgroup per CU (otherwise a CU would hold 8 waves
 // with one piece in flight each), 8 when two workgroups share a CU.
-template <bool Q4, bool DUMP, int NW>
+// ALDS (8 or 16 token slots): the activation fragments of a piece, tslots * 128 contiguous bytes, go global -> LDS
+// directly in one or two instructions and every lane reads its own from there, instead of four register loads in
+// which most lanes fetch a copy (the kernel is bound by the number of vector-memory instructions).
+template <bool Q4, bool DUMP, int NW, bool ALDS>
 __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     constexpr int kWaves = NW;
-    constexpr int kWaveLds = wave_lds(Q4);
+    constexpr int kWaveLds = wave_lds(Q4, ALDS);
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 31, half = lane >> 5;
@@ -104,6 +108,7 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     const int piece_end = min(piece0 + p.pieces_per_slice, npieces_total);
     char* mine = smem + wave * kWaveLds;
     const unsigned mine_lds = __builtin_amdgcn_readfirstlane(lds_addr(mine));
+    const char* mine_a = mine + wave_lds(Q4, false);   // ALDS: the piece's activation fragments
 
     // loop-invariant lane roles
     const int wrow = min(r0 + col, r_last);                         // this lane's weight row (MFMA operand and scales)
@@ -119,7 +124,13 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     auto request = [&](int piece) -> PieceRegs {
         PieceRegs r;
         const int blk0 = piece * 4;
-        {   // with 32 token slots a wave's fragment load is one contiguous kilobyte
+        if (ALDS) {   // chunk (b * 2 + half) * tslots + token of the whole row set; chunks past the last block re-read it
+            const unsigned last = (unsigned)p.nb * 2 * p.tslots - 1;
+            for (int j = 0; j * 8 < p.tslots; j++)   // wave-uniform
+                load_to_lds16(p.xq + (size_t)min((unsigned)(piece * 8 * p.tslots + j * 64 + lane), last) * 16,
+                              mine_lds + wave_lds(Q4, false) + j * 1024);
+            r.a0 = r.a1 = r.a2 = r.a3 = v4i{0, 0, 0, 0};
+        } else {   // with 32 token slots a wave's fragment load is one contiguous kilobyte
             auto la = [&](int bi) {
                 return *(const v4i*)(p.xq + ((size_t)(min(blk0 + bi, p.nb - 1) * 2 + half) * p.tslots + atok) * 16);
             };
@@ -191,7 +202,8 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
 #pragma unroll
         for (int bi = 0; bi < 4; bi++) {
             const v4i bfrag = *(const v4i*)(buf + col * 128 + ((2 * bi + half + col) & 7) * 16);
-            const v4i afrag = bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3));
+            const v4i afrag = ALDS ? *(const v4i*)(mine_a + ((bi * 2 + half) * p.tslots + min(col, p.tslots - 1)) * 16)
+                                   : (bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3)));
             const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, bfrag, cmagic, 0, 0, 0);
             const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero scale
             const float dw = live ? h2f_s((uint16_t)dwh[bi]) : 0.f;
@@ -300,7 +312,7 @@ __global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restri
 // one 32-row group per workgroup, weights of more than about 12000 rows no longer fit one round of workgroups
 // and the tiled GEMM wins.
 bool skinny_serves(const Weight& w, size_t m) {
-    return (w.type == kQ8_0 || w.type == kQ4_0) && m > SMX_GEMV_MAX_M && m <= SMX_SKINNY_MAX_M && w.K >= 128 && w.N <= 12288;
+    return (w.type == kQ8_0 || w.type == kQ4_0) && m >= SMX_SKINNY_MIN_M && m <= SMX_SKINNY_MAX_M && w.K >= 128 && w.N <= 12288;
 }
 
 size_t skinny_xq_bytes(size_t m, size_t K) { return (K / 32) * 2 * (m <= 8 ? 8 : (m <= 16 ? 16 : 32)) * 16; }
@@ -351,7 +363,8 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
     const bool q4 = w.type == kQ4_0;
     const int nwg = nrg * ksplit;
     const int nw = nwg <= c->num_cu ? 16 : 8;   // waves per workgroup (see the kernel)
-    const size_t lds = (size_t)nw * wave_lds(q4);   // the reduction reuses the first nw * 4 KB
+    const bool alds = p.tslots <= 16;
+    const size_t lds = (size_t)nw * wave_lds(q4, alds);   // the reduction reuses the first nw * 4 KB
     const dim3 grid((unsigned)nwg);
     ProfScope ps(c, q4 ? "skinny_q4_0" : "skinny_q8_0");
     auto go = [&](auto kern) -> int {
@@ -361,12 +374,14 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
         SMX_HIP(c, hipGetLastError());
         return SMX_OK;
     };
+#define SMX_SK_GO(Q4_, NW_, AL_) (dump ? go(skinny_kernel<Q4_, true, NW_, AL_>) : go(skinny_kernel<Q4_, false, NW_, AL_>))
     if (nw == 16) {
-        if (q4) return dump ? go(skinny_kernel<true, true, 16>) : go(skinny_kernel<true, false, 16>);
-        return dump ? go(skinny_kernel<false, true, 16>) : go(skinny_kernel<false, false, 16>);
+        if (q4) return alds ? SMX_SK_GO(true, 16, true) : SMX_SK_GO(true, 16, false);
+        return alds ? SMX_SK_GO(false, 16, true) : SMX_SK_GO(false, 16, false);
     }
-    if (q4) return dump ? go(skinny_kernel<true, true, 8>) : go(skinny_kernel<true, false, 8>);
-    return dump ? go(skinny_kernel<false, true, 8>) : go(skinny_kernel<false, false, 8>);
+    if (q4) return alds ? SMX_SK_GO(true, 8, true) : SMX_SK_GO(true, 8, false);
+    return alds ? SMX_SK_GO(false, 8, true) : SMX_SK_GO(false, 8, false);
+#undef SMX_SK_GO
 }
 
 }  // namespace smx

@@ -251,6 +251,7 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
 // Small-batch matmul on the matrix cores (skinny.hip): m <= SMX_SKINNY_MAX_M fp32 rows against a Q8_0 / Q4_0
 // weight read once (its own quantiser launch + the matmul launch).  dump (optional): out[m][N][K/32] i32.
 #define SMX_SKINNY_MAX_M 32
+#define SMX_SKINNY_MIN_M 5
 bool skinny_serves(const Weight& w, size_t m);
 // bytes of sc.xq the call needs (quants in MFMA fragment order, 8, 16 or 32 token slots)
 size_t skinny_xq_bytes(size_t m, size_t K);
