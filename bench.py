@@ -32,7 +32,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 # HBM bytes per launch of the headline kernel from rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by
 # the same counter's reading for a 256 MiB copy (profiles/gemv_q4_0_9728x2560_hbm_traffic.md)
-HEADLINE_TRAFFIC_BYTES = 14264410
+HEADLINE_TRAFFIC_BYTES = 14232474
 # the same for the Q8_0 ffn_up GEMM launch (profiles/gemm_i8_q8_0_ffn_up_counters.md): L2 fills + writes
 GEMM_TRAFFIC_BYTES = {"gemm_q8_0_ffn_up": 667380565}
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
@@ -170,8 +170,8 @@ class Bench:
 
     # ------------------------------------------------------------------ GEMV
     def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False):
-        """m rows against rotating weight copies.  m <= 8: the dot4 GEMV (quantiser fused for m = 1); 9..32 rows: the
-        small-batch kernel on the matrix cores; f32: the fp32-activation GEMV (no quantiser)."""
+        """m rows against rotating weight copies.  m <= 4: the dot4 GEMV (quantiser fused for m = 1); 5..32 rows of a
+        Q8_0 / Q4_0 weight: the small-batch kernel on the matrix cores; f32: the fp32-activation GEMV (no quantiser)."""
         acc, sy = self.acc, self.synth
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
         algo, wbytes = gemv_bytes(ty, N, K, m)
@@ -196,7 +196,7 @@ class Bench:
             else:
                 acc.gemv_dev(keys[i % ncopies], xd, m, yd)
 
-        kname = ("gemv_f32_" + KERNEL[ty][5:]) if f32 else (KERNEL[ty] if m <= 8 or ty == Q6_K else "skinny_" + KERNEL[ty][5:])
+        kname = ("gemv_f32_" + KERNEL[ty][5:]) if f32 else (KERNEL[ty] if m <= 4 or ty == Q6_K else "skinny_" + KERNEL[ty][5:])
         ms, wall_ms = self._timed(step, steps, warmup)
         kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
         for k in keys:
@@ -594,6 +594,7 @@ def main():
         ("q4_0_gemv_9728x2560_batch8", lambda: b.gemv_group("q4_0_gemv_9728x2560_batch8", Q4_0, 9728, 2560, 8, int(1.1 * GB))),
         ("q4_0_ffn_decode_block_2560x9728", lambda: b.ffn_block("q4_0_ffn_decode_block_2560x9728", Q4_0, 2560, 9728, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m1", lambda: b.gemv("q8_0_gemv_2560x9728_m1", Q8_0, 2560, 9728, 1, int(1.1 * GB))),
+        ("q8_0_gemv_2560x9728_m4", lambda: b.gemv("q8_0_gemv_2560x9728_m4", Q8_0, 2560, 9728, 4, int(1.1 * GB))),
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
         ("q8_0_small_batch_2560x9728_m16", lambda: b.gemv("q8_0_small_batch_2560x9728_m16", Q8_0, 2560, 9728, 16, int(1.1 * GB))),
         ("q8_0_small_batch_2560x9728_m32", lambda: b.gemv("q8_0_small_batch_2560x9728_m32", Q8_0, 2560, 9728, 32, int(1.1 * GB))),

@@ -60,8 +60,8 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restric
 }
 
 // quantise m device rows and run the right matmul kernel into y_dev
-// Which kernel serves m rows: the dot4 GEMV up to SMX_GEMV_MAX_M rows, the small-batch MFMA kernel from there
-// to SMX_SKINNY_MAX_M rows of a Q8_0 / Q4_0 weight of moderate height (skinny_serves), the tiled GEMM otherwise.
+// Which kernel serves m rows: the small-batch MFMA kernel for SMX_SKINNY_MIN_M .. SMX_SKINNY_MAX_M rows of a Q8_0 / Q4_0
+// weight of moderate height (skinny_serves); otherwise the dot4 GEMV up to SMX_GEMV_MAX_M rows, the tiled GEMM beyond.
 }  // namespace
 
 namespace smx {

@@ -286,7 +286,7 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
                                                             const uint4* __restrict__ quants, const MoeRoute route,
                                                             int k, int eff, int hidden, float* __restrict__ y,
                                                             int* __restrict__ aq_out, float* __restrict__ ad_out,
-                                                            unsigned magic_units, unsigned magic_upe) {
+                                                            unsigned magic_units, unsigned magic_upe, int n_wgs) {
     extern __shared__ __align__(16) char smem[];
     constexpr int PRE = 3, XI = 4;
     const int nbe = eff / 32, upe = eff / 16, units = k * upe;
@@ -296,17 +296,8 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
     float* sw = (float*)(sid + k);                  // [k] routing weights
     float* part = sw + k;                           // [rows * units / GL]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid < k) {
-        sid[tid] = route_id(route, tid);
-        sw[tid] = route_w(route, tid);
-    }
-    __syncthreads();
-    const unsigned rbase = (unsigned)hidden / gridDim.x, rrem = (unsigned)hidden - rbase * gridDim.x;
-    const int r0 = blockIdx.x * (int)rbase + min((int)blockIdx.x, (int)rrem);
-    const int rows = (int)rbase + ((int)blockIdx.x < (int)rrem ? 1 : 0);
-    const int nv = rows * units;                    // < 2^16 (launcher)
-    const int nloads = (nv + 63) >> 6;
-
+    // g and u first: they do not depend on the routing, and the routing (read from the router's output when it ran
+    // on the device) is a memory round trip of its own that the weight addresses have to wait for
     const int items = k * eff / 4;                  // float4 items, 8 per block; <= XI * 1024 (launcher)
     float4 gv[XI], uv[XI];
 #pragma unroll
@@ -318,6 +309,17 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
             uv[j] = ((const float4*)u)[it];
         }
     }
+    if (tid < k) {
+        sid[tid] = route_id(route, tid);
+        sw[tid] = route_w(route, tid);
+    }
+    __syncthreads();
+    // (n_wgs = gridDim.x as an argument: the built-in is a load from the hidden arguments)
+    const unsigned rbase = (unsigned)hidden / (unsigned)n_wgs, rrem = (unsigned)hidden - rbase * (unsigned)n_wgs;
+    const int r0 = blockIdx.x * (int)rbase + min((int)blockIdx.x, (int)rrem);
+    const int rows = (int)rbase + ((int)blockIdx.x < (int)rrem ? 1 : 0);
+    const int nv = rows * units;                    // < 2^16 (launcher)
+    const int nloads = (nv + 63) >> 6;
 
     uint4 q[PRE];
     uint16_t sc[PRE];
@@ -388,11 +390,15 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
         consume();
     }
     __syncthreads();
+    // a row's G group sums: 8 lanes take groups l, l + 8, ... (ascending), then a fixed DPP tree -- one thread per
+    // row would pay the LDS latency G times in a row
     const int G = units / GL;
-    for (int r = tid; r < rows; r += 1024) {
+    for (int i8 = tid; i8 < rows * 8; i8 += 1024) {
+        const int r = i8 >> 3, l = i8 & 7;
         float s = 0.f;
-        for (int j = 0; j < G; j++) s += part[r * G + j];
-        y[r0 + r] = s;
+        for (int j = l; j < G; j += 8) s += part[r * G + j];
+        s = small_group_sum<8>(s);
+        if (l == 0) y[r0 + r] = s;
     }
 }
 
@@ -597,7 +603,7 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
                 if (rc2 != SMX_OK) return rc2;
                 hipLaunchKernelGGL(kern, dim3((unsigned)fgrid), dim3(1024), flds, c->stream, s.g, s.u, L.down.scales,
                                    (const uint4*)L.down.quants, route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad,
-                                   m_units, m_upe);
+                                   m_units, m_upe, (int)fgrid);
                 SMX_HIP(c, hipGetLastError());
                 return SMX_OK;
             };

@@ -306,11 +306,11 @@ __global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restri
 
 }  // namespace
 
-// Measured on MI355X (Q8_0 2560 x 9728 / Q4_0 9728 x 2560 / Q8_0 15360 x 3840, quantiser included): 16.1 / 16.8 /
-// 26.3 us at 9 rows and 18.3 / 21 / 32 us at 32 rows, against 23.5 / 22.2 / 25.3 and 24.5 / 24.2 / 27.4 us for the
-// tiled GEMM with split-K; up to 8 rows the dot4 GEMV is faster (13.8 us at 8 rows on the first shape).  With
-// one 32-row group per workgroup, weights of more than about 12000 rows no longer fit one round of workgroups
-// and the tiled GEMM wins.
+// Measured on MI355X (Q8_0 2560 x 9728 / Q4_0 9728 x 2560 / Q8_0 9728 x 2560, quantiser launch included): 11.0 / 10.9 /
+// 10.7 us at 5 rows, 12.3 / 12.0 / 11.9 us at 16 rows and 14.3 / 12.5 / 13.7 us at 32 rows; the dot4 GEMV takes 13.3 /
+// 11.8 / 13.0 us at 5 rows and 13.9 / 12.3 / 13.0 us at 8, 10.9 / 9.0 / 10.7 us at 4 (where it stays), and the tiled
+// GEMM with split-K 22 - 27 us.  Weights of more than about 12000 rows no longer fit two rounds of workgroups and the
+// tiled GEMM wins.
 bool skinny_serves(const Weight& w, size_t m) {
     return (w.type == kQ8_0 || w.type == kQ4_0) && m >= SMX_SKINNY_MIN_M && m <= SMX_SKINNY_MAX_M && w.K >= 128 && w.N <= 12288;
 }
