@@ -63,7 +63,7 @@ class Floors:
         L.sbk_empty_launch.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, dp]
         L.sbk_read_floor.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int, dp]
         L.sbk_copy.argtypes = [ctypes.c_size_t, ctypes.c_int, dp]
-        L.sbk_mfma_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, dp, dp, dp]
+        L.sbk_mfma_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, dp, dp, dp]
         self.L = L
 
     def empty_launch(self, grid, block, launches=2000):
@@ -85,9 +85,10 @@ class Floors:
         assert self.L.sbk_copy(nbytes, launches, ctypes.byref(d)) == 1
         return d.value
 
-    def mfma_valu(self, mode, row_tiles, waves_per_simd, nblocks=4000):
+    def mfma_valu(self, mode, row_tiles, waves_per_simd, nblocks=4000, warm_launches=15):
+        """15 untimed launches (30 ms) first: the rate the chip sustains, as for the GEMM workloads."""
         us, tops, cyc = ctypes.c_double(), ctypes.c_double(), ctypes.c_double()
-        assert self.L.sbk_mfma_valu(mode, row_tiles, waves_per_simd, nblocks, ctypes.byref(us), ctypes.byref(tops), ctypes.byref(cyc)) == 1
+        assert self.L.sbk_mfma_valu(mode, row_tiles, waves_per_simd, nblocks, warm_launches, ctypes.byref(us), ctypes.byref(tops), ctypes.byref(cyc)) == 1
         return {"us": us.value, "TOPS": tops.value, "cycles_per_mfma_per_wave": cyc.value,
                 "simd_cycles_per_mfma": cyc.value / waves_per_simd}
 
@@ -135,6 +136,15 @@ class Bench:
 
     def log(self, *a):
         print(*a, file=sys.stderr, flush=True)
+
+    def _first_touch(self, fn, n):
+        """Part of a workload's set-up: one untimed step per rotating weight copy (n of them), so that no timed launch is
+        the first access to freshly uploaded memory.  A decode loop reads every weight once per token; the first read
+        after the upload costs 0.4-0.5 us more per 14 MB launch (address translation), which a run of 5 + 20 steps
+        would otherwise measure instead of the kernel.  The rotation still exceeds the Infinity Cache: the data stay cold."""
+        for i in range(n):
+            fn(i)
+        self.acc.sync()
 
     def _timed(self, fn, steps, warmup):
         """W untimed + exactly K timed steps, bracketed by stream syncs; HIP events on the stream."""
@@ -196,6 +206,7 @@ class Bench:
             else:
                 acc.gemv_dev(keys[i % ncopies], xd, m, yd)
 
+        self._first_touch(step, ncopies)
         kname = ("gemv_f32_" + KERNEL[ty][5:]) if f32 else (KERNEL[ty] if m <= 4 or ty == Q6_K else "skinny_" + KERNEL[ty][5:])
         ms, wall_ms = self._timed(step, steps, warmup)
         kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
@@ -255,6 +266,7 @@ class Bench:
             else:
                 acc.gemv_batch_dev(keys[g0:g0 + G], [xd] * G, yds)
 
+        self._first_touch(step, ngroups)
         ms, wall_ms = self._timed(step, steps, warmup)
         for k in keys:
             acc.evict(k)
@@ -295,6 +307,7 @@ class Bench:
             acc.gemv_fused_dev([f"{name}.g{j}", f"{name}.u{j}"], 1, xd, wd, [gd, ud], 1e-6)
             acc.gemv_fused_dev([f"{name}.d{j}"], 2, gd, ud, [yd])
 
+        self._first_touch(step, nsets)
         ms, wall_ms = self._timed(step, steps, warmup)
         for i in range(nsets):
             for t in "gud":
@@ -312,7 +325,7 @@ class Bench:
         """M tokens through a dense FFN: rmsnorm + quantiser + gate GEMM, the same for up, then
         SwiGLU + quantiser + down GEMM (each producer runs inside its quantiser launch)."""
         acc, sy = self.acc, self.synth
-        steps, warmup = steps or max(5, self.steps // 20), warmup if warmup is not None else 2
+        steps, warmup = steps or max(20, self.steps // 20), warmup if warmup is not None else 20   # sustained clocks: see gemm()
         up_fn = getattr(acc, UPLOAD[ty])
         assert up_fn(name + ".g", sy.make_weight(ty, F, H, seed=1700), H, F)
         assert up_fn(name + ".u", sy.make_weight(ty, F, H, seed=1701), H, F)
@@ -356,7 +369,10 @@ class Bench:
     # ------------------------------------------------------------------ GEMM
     def gemm(self, name, ty, M, N, K, steps=None, warmup=None):
         acc, sy = self.acc, self.synth
-        steps, warmup = steps or max(5, self.steps // 20), warmup if warmup is not None else 2
+        # Under matrix load the chip takes some 20 ms to settle at the clock it sustains (the first launches after idle
+        # run 15 % slower, the next ones briefly faster): 50 untimed launches first, whatever --steps says; a prefill is
+        # hundreds of such launches back to back.
+        steps, warmup = steps or max(50, self.steps // 8), warmup if warmup is not None else 50
         raw = sy.make_weight(ty, N, K, seed=2000 + ty)
         assert getattr(acc, UPLOAD[ty])(name, raw, K, N)
         del raw
@@ -460,6 +476,7 @@ class Bench:
             def step(i):
                 acc.moe_ffn_dev(i % layers, ids[i % len(ids)], w[i % len(ids)], xd, yd)
 
+            self._first_touch(step, len(ids))   # (nearly) every expert of every layer once
             ms, wall_ms = self._timed(step, steps, warmup)
             kus, nk = self._kernel_avg_us(step, steps, warmup, "moe_gemv")
             acc.dev_free(xd)
@@ -471,32 +488,38 @@ class Bench:
                         "kernel": "moe_gemv_gate_up + moe_gemv_down", "kernel_avg_us_sum": kus * 2,
                         "kernel_GBps": wbytes / (kus * 2 * 1e-6) / 1e9})
         else:
-            steps = max(5, steps // 20)
+            # Host-buffer calls (every call uploads its rows and tables and waits for the result), then the resident form
+            # back to back: 100 untimed calls first so that the chip has settled at the clock it sustains (see gemm()),
+            # then `steps` calls between two events, then as many with an event pair around every kernel.
+            hsteps = max(5, steps // 20)
+            steps = max(50, steps // 8)
             ids, w = sy.zipf_routing(m, ne, k, seed=5)
             plan, slot_tok, wslot = sy.group_by_expert(ids, w, ne)
             xs = sy.make_acts(m, hidden, seed=9)
-            t0 = time.perf_counter()
             for _ in range(2):
                 acc.moe_layer_q8_dev(0, xs, m, plan, slot_tok, wslot)
-            acc.prof_reset()
-            acc.prof_enable(True)
             t0 = time.perf_counter()
-            for _ in range(steps):
+            for _ in range(hsteps):
                 acc.moe_layer_q8_dev(0, xs, m, plan, slot_tok, wslot)
-            wall_ms = (time.perf_counter() - t0) * 1e3
-            acc.prof_enable(False)
-            g_ms, _ = acc.prof_read("moe_gemm")
-            all_ms = sum(acc.prof_read(p)[0] for p in ("actquant", "moe_gemm", "silu_mul_quant", "moe_combine"))
-            acc.prof_reset()
+            wall_ms = (time.perf_counter() - t0) * 1e3 * steps / hsteps
             xd, yd = acc.dev_alloc(xs.nbytes), acc.dev_alloc(xs.nbytes)
             acc.h2d(xd, xs)
-            for _ in range(2):
+            for _ in range(100):
                 acc.moe_layer_resident(0, xd, m, plan, slot_tok, wslot, yd)
             acc.sync()
             acc.timer_begin()
             for _ in range(steps):
                 acc.moe_layer_resident(0, xd, m, plan, slot_tok, wslot, yd)
             res_ms = acc.timer_end()
+            acc.prof_reset()
+            acc.prof_enable(True)
+            for _ in range(steps):
+                acc.moe_layer_resident(0, xd, m, plan, slot_tok, wslot, yd)
+            acc.sync()
+            acc.prof_enable(False)
+            g_ms, _ = acc.prof_read("moe_gemm")
+            all_ms = sum(acc.prof_read(p)[0] for p in ("actquant", "moe_gemm", "silu_mul_quant", "moe_combine"))
+            acc.prof_reset()
             acc.dev_free(xd)
             acc.dev_free(yd)
             ops = 2 * slot_tok.size * 3 * eff * hidden
@@ -633,7 +656,9 @@ def main():
         "config": {"workload": "Q4_0 decode GEMV, weight 9728x2560, 1 token, Q8 activations, cache-cold: "
                                f"{head['weight_copies']} rotating resident weight copies "
                                f"({head['weight_copies'] * head['weight_bytes'] / 1e9:.2f} GB); "
-                               "step = activation quantiser + GEMV", "frac_hbm_peak": head["frac_hbm_peak"]},
+                               "step = activation quantiser + GEMV", "frac_hbm_peak": head["frac_hbm_peak"],
+                   "set_up": "weights uploaded, then read once each (one untimed GEMV per copy) before the warm-up: "
+                             "no timed launch is the first access to freshly uploaded memory"},
         "roofline": {"bound": "hbm", "achieved": head["kernel_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": head["kernel_frac_hbm_peak"], "traffic": HEADLINE_TRAFFIC_BYTES,
                      "traffic_source": "constant from profiles/gemv_q4_0_9728x2560_hbm_traffic.md (rocprofv3 FETCH_SIZE + WRITE_SIZE "

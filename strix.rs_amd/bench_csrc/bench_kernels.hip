@@ -310,8 +310,10 @@ int sbk_copy(size_t bytes, int launches, double* us_per_launch) {
 // spent per MFMA unit.
 // `row_tiles` (4 or 2): 32-row tiles per wave, i.e. a 32 x 128 or 32 x 64 wave tile; wgs_per_cu 1..4 (4-wave workgroups,
 // so also waves per SIMD; 32 x 128 tiles fit at most 3 per SIMD in registers).
-int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, double* us, double* tops, double* cycles_per_unit) {
-    if (!us || !tops || !cycles_per_unit || mode < 0 || mode > 5 || wgs_per_cu < 1 || wgs_per_cu > 4 || nblocks <= 0) return SBK_ERR;
+// `warm_launches` untimed launches come first: under matrix load the chip takes some 20 ms to settle at the clock it
+// then sustains (the first launches after idle run 15 % slower), and a prefill is hundreds of such launches.
+int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, int warm_launches, double* us, double* tops, double* cycles_per_unit) {
+    if (!us || !tops || !cycles_per_unit || mode < 0 || mode > 5 || wgs_per_cu < 1 || wgs_per_cu > 4 || nblocks <= 0 || warm_launches < 1) return SBK_ERR;
     if ((row_tiles != 4 && row_tiles != 2) || (row_tiles == 4 && wgs_per_cu > 3)) return SBK_ERR;
     Timer t;
     if (!t.ok) return SBK_ERR;
@@ -342,7 +344,7 @@ int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, double* 
         auto launch = [&]() { hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, t.s, (const float*)scales, nblocks, out, cyc, (const v4i*)aglob); };
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) rc = SBK_ERR;
         if (rc == SBK_OK) {
-            launch();
+            for (int i = 0; i < warm_launches; i++) launch();
             (void)hipStreamSynchronize(t.s);
             const int reps = 5;
             t.begin();
