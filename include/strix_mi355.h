@@ -100,10 +100,9 @@ int smx_gemv_f32(smx_ctx* ctx, const char* key, const float* x, size_t in_len, f
 int smx_gemv_f32_dev(smx_ctx* ctx, const char* key, const float* x_dev, float* y_dev);
 /* Small batches, m <= SMX_GEMV_ROWS_MAX rows against one weight read once (kernels.rs:1605-1632 q8_gemm_rows,
  * :830-857 q8_gemm_rows32, :1016-1045 q8i_gemm_rows32; the n-gram verify step and short prefill chunks):
- * xs[m][in_dim] -> y[m][out_dim].  Up to 4 rows run in the dot4 GEMV, 5..32 rows of a Q8_0 / Q4_0 weight of up to
- * 12288 rows in the small-batch kernel on the matrix cores, every other case (Q6_K weights, taller weights) in the
- * dot4 GEMV up to SMX_GEMV_MAX_M rows or the tiled GEMM; the integer block dots do not depend on which, the fp32
- * sums agree within 1e-5. */
+ * xs[m][in_dim] -> y[m][out_dim].  Up to 4 rows run in the dot4 GEMV; 5..32 rows of a Q8_0 / Q4_0 weight (17..32 rows:
+ * weights of up to 32768 rows) and 5..16 rows of a Q6_K weight in the small-batch kernel on the matrix cores; every other
+ * case in the tiled GEMM.  The integer block dots do not depend on which, the fp32 sums agree within 1e-5. */
 #define SMX_GEMV_MAX_M 8
 #define SMX_GEMV_ROWS_MAX 32
 int smx_gemv_rows(smx_ctx* ctx, const char* key, const float* xs, size_t m, size_t in_dim,
@@ -161,10 +160,7 @@ int smx_dev_copy(smx_ctx* ctx, void* dst_dev, const void* src_dev, size_t nbytes
 int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
 /* smx_gemv_dev for callers that cannot allocate (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same kernels and results
- * as smx_gemv_dev (except 5..8 rows of a Q6_K weight or of a weight of more than 12288 rows, where smx_gemv_dev
- * takes the tiled GEMM, whose scratch grows with the call, and this entry point keeps the dot4 GEMV: same integers,
- * fp32 sums within 1e-5); the rows quantised
- * for m >= 2 live in a static device array of the library (160 KB per
+ * as smx_gemv_dev; the rows quantised for m >= 2 live in a static device array of the library (160 KB per
  * GPU, held until the process ends) instead of the context's growable scratch, so the call never
  * allocates or frees device or host memory.  Limits: m <= SMX_NOALLOC_MAX_ROWS, in_dim <= SMX_NOALLOC_MAX_IN_DIM
  * (SMX_ERR_LIMIT beyond).  All contexts of one GPU share the array: calls that overlap on one GPU race. */

@@ -41,15 +41,20 @@ constexpr int kPiece = 32 * 128;          // LDS bytes of one piece: 32 rows x 4
 // LDS bytes per wave: the landing area of its piece (Q8_0: 4 KB, already in operand order; Q4_0: 2 KB of raw
 // nibbles and the 4 KB area the widened piece is built in)
 // and, when the activation fragments travel through LDS too (ALDS, up to 16 token slots), 2 KB for those of a piece
-constexpr int wave_lds(bool q4, bool alds) { return (q4 ? 2048 + kPiece : kPiece) + (alds ? 2048 : 0); }
+// Q6_K: 2 KB of ql + 1 KB of qh as they are, and the 4 KB widened area.
+constexpr int FMT_Q8 = 0, FMT_Q4 = 1, FMT_Q6 = 2;
+constexpr int weight_lds(int fmt) { return fmt == FMT_Q4 ? 2048 + kPiece : (fmt == FMT_Q6 ? 3072 + kPiece : kPiece); }
+constexpr int wave_lds(int fmt, bool alds) { return weight_lds(fmt) + (alds ? 2048 : 0); }
 
 struct SkinnyArgs {
-    const uint16_t* wscales;  // f16 [N][nb]
-    const void* wquants;      // Q8_0: i8 [N][K]; Q4_0: 16 B [N][nb]
+    const uint16_t* wscales;  // f16 [N][nb]; Q6_K: d [N][K / 256]
+    const void* wquants;      // Q8_0: i8 [N][K]; Q4_0: 16 B [N][nb]; Q6_K: ql, 128 B per superblock
+    const void* wqh;          // Q6_K: 64 B per superblock
+    const int8_t* wsc;        // Q6_K: 16 sub-block scales per superblock
     const int8_t* xq;         // fragment order: [nb][2 k-halves][tslots tokens][16 B] (see skinny_quant_kernel)
     const float* xd;          // [pieces][tslots][4]: the four block scales of a piece side by side per token slot
     float* y;                 // [m][N]
-    int* dump;                // optional [m][N][nb] i32 block dots
+    int* dump;                // optional [m][N][nb] i32 block dots (Q6_K: [m][N][2 nb] sub-block dots)
     int m, N, nb;
     int tslots;               // token slots of the fragment-ordered activations: 8, 16 or 32
     int ksplit;               // K slices per row group (1 or 2)
@@ -71,6 +76,11 @@ __device__ __forceinline__ void load_to_lds16(const void* g, unsigned lds_base) 
                  : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(g)
                  : "memory", "m0");
 }
+// four 6-bit quants (low nibbles in lo4, the two high bits in hi2) -> four signed bytes q - 32
+__device__ __forceinline__ unsigned q6_bytes_s(unsigned lo4, unsigned hi2) {
+    return (((lo4 & 0x0f0f0f0fu) | ((hi2 & 0x03030303u) << 4) | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+}
+
 __device__ __forceinline__ unsigned lds_addr(const void* p) {
     return (unsigned)(uintptr_t)(const __attribute__((address_space(3))) char*)p;
 }
@@ -80,7 +90,8 @@ __device__ __forceinline__ unsigned lds_addr(const void* p) {
 // go global -> LDS directly and are counted by vmcnt only.
 struct PieceRegs {
     v4i a0, a1, a2, a3;    // activation fragment of each block: lane = (token lane % 32, k-half lane / 32)
-    uint2 dw;              // four f16 scales of this lane's weight row
+    uint2 dw;              // four f16 scales of this lane's weight row; Q6_K: the eight int8 sub-block scales of the piece
+    uint16_t d6;           // Q6_K: d of the row's superblock
     uint4 dx;              // four f32 scales (one per block) of the token whose accumulators this lane feeds by row broadcast
 };
 // vector-memory loads per piece: 6 that return into registers, then up to 4 (Q8_0: 8 rows x 128 B each)
@@ -91,10 +102,17 @@ struct PieceRegs {
 // ALDS (8 or 16 token slots): the activation fragments of a piece, tslots * 128 contiguous bytes, go global -> LDS
 // directly in one or two instructions and every lane reads its own from there, instead of four register loads in
 // which most lanes fetch a copy (the kernel is bound by the number of vector-memory instructions).
-template <bool Q4, bool DUMP, int NW, bool ALDS>
+// Q6_K (always with ALDS, so up to 16 rows): a piece is half a superblock; its ql and qh bytes land as they are (3 LDS-direct
+// instructions), the wave widens them to signed int8 in operand order (thread = [row:5][p:1] makes the 16-byte chunks 2j + p,
+// ggml_quant.rs:417-426), and a 32-block is two v_mfma_i32_32x32x16_i8, one per 16-element sub-block with its own d * sc.
+// NACC: accumulators per lane that hold live tokens (accumulator i of lane half h is token (i / 4) * 8 + 4 h + i % 4: 4 for up
+// to 8 token slots, 8 for 16); only those are rescaled -- with all 16 the Q6_K variant would be bound by its vector ALU work.
+template <int FMT, bool DUMP, int NW, bool ALDS, int NACC = 16>
 __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
+    constexpr bool Q4 = FMT == FMT_Q4, Q6 = FMT == FMT_Q6;
+    static_assert(!Q6 || ALDS, "the Q6_K variant reads its activation fragments from LDS");
     constexpr int kWaves = NW;
-    constexpr int kWaveLds = wave_lds(Q4, ALDS);
+    constexpr int kWaveLds = wave_lds(FMT, ALDS);
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 31, half = lane >> 5;
@@ -108,7 +126,7 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     const int piece_end = min(piece0 + p.pieces_per_slice, npieces_total);
     char* mine = smem + wave * kWaveLds;
     const unsigned mine_lds = __builtin_amdgcn_readfirstlane(lds_addr(mine));
-    const char* mine_a = mine + wave_lds(Q4, false);   // ALDS: the piece's activation fragments
+    const char* mine_a = mine + weight_lds(FMT);   // ALDS: the piece's activation fragments
 
     // loop-invariant lane roles
     const int wrow = min(r0 + col, r_last);                         // this lane's weight row (MFMA operand and scales)
@@ -128,7 +146,7 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
             const unsigned last = (unsigned)p.nb * 2 * p.tslots - 1;
             for (int j = 0; j * 8 < p.tslots; j++)   // wave-uniform
                 load_to_lds16(p.xq + (size_t)min((unsigned)(piece * 8 * p.tslots + j * 64 + lane), last) * 16,
-                              mine_lds + wave_lds(Q4, false) + j * 1024);
+                              mine_lds + weight_lds(FMT) + j * 1024);
             r.a0 = r.a1 = r.a2 = r.a3 = v4i{0, 0, 0, 0};
         } else {   // with 32 token slots a wave's fragment load is one contiguous kilobyte
             auto la = [&](int bi) {
@@ -138,14 +156,28 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         }
         const uint16_t* ws = p.wscales + (size_t)wrow * p.nb;
         r.dx = *(const uint4*)(p.xd + ((size_t)piece * p.tslots + dx_tok) * 4);   // 16 contiguous bytes per token slot
-        if (vec_sc) {
+        r.d6 = 0;
+        if (Q6) {
+            const size_t sb = (size_t)wrow * (p.nb >> 3) + (piece >> 1);
+            r.d6 = p.wscales[sb];
+            r.dw = *(const uint2*)(p.wsc + sb * 16 + (piece & 1) * 8);
+        } else if (vec_sc) {
             r.dw = *(const uint2*)(ws + blk0);
         } else {   // (the scalar form costs more loads; the waits below are then over-conservative, never too lax)
             const int last = p.nb - 1;
             r.dw.x = (unsigned)ws[min(blk0, last)] | ((unsigned)ws[min(blk0 + 1, last)] << 16);
             r.dw.y = (unsigned)ws[min(blk0 + 2, last)] | ((unsigned)ws[min(blk0 + 3, last)] << 16);
         }
-        if (Q4) {   // lane = [row:4][block:2]: 64 contiguous bytes of nibbles per row, landing as they are
+        if (Q6) {   // ql: lane = [row:4][chunk:2], 64 bytes per row and half superblock; qh: lane = [row:5][chunk:1], 32 bytes
+            const int nsb = p.nb >> 3, sbi = piece >> 1, hs = piece & 1;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                if (j * 16 < nrows)   // wave-uniform
+                    load_to_lds16((const char*)p.wquants + ((size_t)min(r0 + j * 16 + (lane >> 2), r_last) * nsb + sbi) * 128 + hs * 64 + (lane & 3) * 16,
+                                  mine_lds + j * 1024);
+            load_to_lds16((const char*)p.wqh + ((size_t)min(r0 + (lane >> 1), r_last) * nsb + sbi) * 64 + hs * 32 + (lane & 1) * 16,
+                          mine_lds + 2048);
+        } else if (Q4) {   // lane = [row:4][block:2]: 64 contiguous bytes of nibbles per row, landing as they are
             const int b = min(blk0 + (lane & 3), p.nb - 1);
 #pragma unroll
             for (int j = 0; j < 2; j++)
@@ -173,7 +205,27 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     auto consume = [&](const PieceRegs r, int piece) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the piece's LDS-direct loads (the compiler does not see them)
         const char* buf;
-        if (Q4) {   // widen the raw nibbles (lane = [row:4][block:2]) into the operand-order area
+        if (Q6) {   // thread (row, p): ql[16p ..], ql[32 + 16p ..], qh[16p ..] of the row's half superblock -> chunks 2j + p
+            char* wide = mine + 3072;
+            const int r = lane >> 1, pp = lane & 1;
+            const uint4 qa = *(const uint4*)(mine + r * 64 + pp * 16), qb = *(const uint4*)(mine + r * 64 + 32 + pp * 16);
+            const uint4 h = *(const uint4*)(mine + 2048 + r * 32 + pp * 16);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint4 q = (j & 1) ? qb : qa;
+                const int ls = (j >> 1) * 4, hs = 2 * j;
+                uint4 o;
+                o.x = q6_bytes_s(q.x >> ls, h.x >> hs);
+                o.y = q6_bytes_s(q.y >> ls, h.y >> hs);
+                o.z = q6_bytes_s(q.z >> ls, h.z >> hs);
+                o.w = q6_bytes_s(q.w >> ls, h.w >> hs);
+                *(uint4*)(wide + r * 128 + ((2 * j + pp + r) & 7) * 16) = o;   // elements 32 j + 16 p .. + 15 of the piece
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            buf = wide;
+        } else if (Q4) {   // widen the raw nibbles (lane = [row:4][block:2]) into the operand-order area
             char* wide = mine + 2048;
             const char* raw = mine;
 #pragma unroll
@@ -199,28 +251,55 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         const int blk0 = piece * 4;
         const unsigned dwh[4] = {r.dw.x & 0xffffu, r.dw.x >> 16, r.dw.y & 0xffffu, r.dw.y >> 16};
         const unsigned dxs[4] = {r.dx.x, r.dx.y, r.dx.z, r.dx.w};
-#pragma unroll
-        for (int bi = 0; bi < 4; bi++) {
-            const v4i bfrag = *(const v4i*)(buf + col * 128 + ((2 * bi + half + col) & 7) * 16);
-            const v4i afrag = ALDS ? *(const v4i*)(mine_a + ((bi * 2 + half) * p.tslots + min(col, p.tslots - 1)) * 16)
-                                   : (bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3)));
-            const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, bfrag, cmagic, 0, 0, 0);
-            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero scale
-            const float dw = live ? h2f_s((uint16_t)dwh[bi]) : 0.f;
-            const float ndw = -dw * kMagicF;                          // exact: dw has 11 significant bits
-            const float dxv = __uint_as_float(dxs[bi]);
+        // acc[i] += dx(token of accumulator i) * fl(dw * I) for the live accumulators, I the exact i32 of MFMA result d
+        auto rescale = [&](const v16i& d, float dw, float dxv) {
+            const float ndw = -dw * kMagicF;   // exact: dw has at most 18 significant bits (f16, or f16 x int8)
             float t[16];
 #pragma unroll
-            for (int i = 0; i < 16; i++) t[i] = fmaf(dw, __int_as_float(d[i]), ndw);
-            SMX_SK_FMAC(0); SMX_SK_FMAC(1); SMX_SK_FMAC(2); SMX_SK_FMAC(3); SMX_SK_FMAC(4); SMX_SK_FMAC(5); SMX_SK_FMAC(6);
-            SMX_SK_FMAC(7); SMX_SK_FMAC(8); SMX_SK_FMAC(9); SMX_SK_FMAC(10); SMX_SK_FMAC(11); SMX_SK_FMAC(12);
-            SMX_SK_FMAC(13); SMX_SK_FMAC(14); SMX_SK_FMAC(15);
-            if (DUMP) {
-                const int row = r0 + col;
+            for (int i = 0; i < NACC; i++) t[i] = fmaf(dw, __int_as_float(d[i]), ndw);
+            SMX_SK_FMAC(0); SMX_SK_FMAC(1); SMX_SK_FMAC(2); SMX_SK_FMAC(3);
+            if constexpr (NACC > 4) { SMX_SK_FMAC(4); SMX_SK_FMAC(5); SMX_SK_FMAC(6); SMX_SK_FMAC(7); }
+            if constexpr (NACC > 8) {
+                SMX_SK_FMAC(8); SMX_SK_FMAC(9); SMX_SK_FMAC(10); SMX_SK_FMAC(11); SMX_SK_FMAC(12); SMX_SK_FMAC(13); SMX_SK_FMAC(14); SMX_SK_FMAC(15);
+            }
+        };
 #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
-                    if (live && tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
+        for (int bi = 0; bi < 4; bi++) {
+            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero scale
+            const float dxv = __uint_as_float(dxs[bi]);
+            if constexpr (Q6) {
+                const float d6 = h2f_s(r.d6);
+#pragma unroll
+                for (int jj = 0; jj < 2; jj++) {   // sub-block jj: chunk 2 bi + jj; a lane holds bytes 8 half .. + 7 of it on both sides
+                    const long bw = *(const long*)(buf + col * 128 + ((2 * bi + jj + col) & 7) * 16 + half * 8);
+                    const long aw = *(const long*)(mine_a + ((bi * 2 + jj) * p.tslots + min(col, p.tslots - 1)) * 16 + half * 8);
+                    const v16i d = __builtin_amdgcn_mfma_i32_32x32x16_i8(aw, bw, cmagic, 0, 0, 0);
+                    const unsigned sc8 = (2 * bi + jj) < 4 ? r.dw.x >> (8 * (2 * bi + jj)) : r.dw.y >> (8 * (2 * bi + jj - 4));
+                    const float dw = d6 * (float)(int)(signed char)(sc8 & 0xff);   // exact in fp32 (11 x 8 significant bits)
+                    rescale(d, dw, dxv);
+                    if (DUMP) {
+                        const int row = r0 + col;
+#pragma unroll
+                        for (int i = 0; i < NACC; i++) {
+                            const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
+                            if (tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * (2 * p.nb) + 2 * (blk0 + bi) + jj] = d[i] - kMagicI;
+                        }
+                    }
+                }
+            } else {
+                const v4i bfrag = *(const v4i*)(buf + col * 128 + ((2 * bi + half + col) & 7) * 16);
+                const v4i afrag = ALDS ? *(const v4i*)(mine_a + ((bi * 2 + half) * p.tslots + min(col, p.tslots - 1)) * 16)
+                                       : (bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3)));
+                const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, bfrag, cmagic, 0, 0, 0);
+                const float dw = live ? h2f_s((uint16_t)dwh[bi]) : 0.f;
+                rescale(d, dw, dxv);
+                if (DUMP) {
+                    const int row = r0 + col;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
+                        if (live && tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
+                    }
                 }
             }
         }
@@ -243,10 +322,10 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     __syncthreads();
     float* red = (float*)smem;   // [wave][16][64]
 #pragma unroll
-    for (int i = 0; i < 16; i++) red[(wave * 16 + i) * 64 + lane] = acc[i];
+    for (int i = 0; i < NACC; i++) red[(wave * 16 + i) * 64 + lane] = acc[i];
     __syncthreads();
 #pragma unroll
-    for (int i = wave; i < 16; i += kWaves) {   // accumulator index; lane as above
+    for (int i = wave; i < NACC; i += kWaves) {   // accumulator index; lane as above
         float s = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; w++) s += red[(w * 16 + i) * 64 + lane];
@@ -309,10 +388,13 @@ __global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restri
 // Measured on MI355X (Q8_0 2560 x 9728 / Q4_0 9728 x 2560 / Q8_0 9728 x 2560, quantiser launch included): 11.0 / 10.9 /
 // 10.7 us at 5 rows, 12.3 / 12.0 / 11.9 us at 16 rows and 14.3 / 12.5 / 13.7 us at 32 rows; the dot4 GEMV takes 13.3 /
 // 11.8 / 13.0 us at 5 rows and 13.9 / 12.3 / 13.0 us at 8, 10.9 / 9.0 / 10.7 us at 4 (where it stays), and the tiled
-// GEMM with split-K 22 - 27 us.  Weights of more than about 12000 rows no longer fit two rounds of workgroups and the
-// tiled GEMM wins.
+// GEMM with split-K 22 - 27 us.
 bool skinny_serves(const Weight& w, size_t m) {
-    return (w.type == kQ8_0 || w.type == kQ4_0) && m >= SMX_SKINNY_MIN_M && m <= SMX_SKINNY_MAX_M && w.K >= 128 && w.N <= 12288;
+    // 17..32 rows of a very tall weight: the tiled GEMM is ahead (Q8_0 65536 x 3840 at 32 rows 61.6 against 70.7 us; at 16 rows
+    // 58.3 / 61.8, at 8 rows the dot4 GEMV 68.2 / 57.6 us; 262144 x 2560: 174.5 / 169.6, 159.2 / 155.5, 171.6 / 139.0 us)
+    if (m < SMX_SKINNY_MIN_M || m > SMX_SKINNY_MAX_M || w.K < 128) return false;
+    if (w.type == kQ6_K) return m <= 16;   // its activation fragments travel through LDS: up to 16 token slots
+    return (w.type == kQ8_0 || w.type == kQ4_0) && (m <= 16 || w.N <= 32768);
 }
 
 size_t skinny_xq_bytes(size_t m, size_t K) { return (K / 32) * 2 * (m <= 8 ? 8 : (m <= 16 ? 16 : 32)) * 16; }
@@ -327,13 +409,15 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
     SkinnyArgs p = {};
     p.wscales = w.scales;
     p.wquants = w.quants;
+    p.wqh = w.qh;
+    p.wsc = w.sc;
     p.xq = sc.xq;
     p.xd = sc.xd;
     p.y = y;
     p.dump = dump;
     p.m = (int)m;
     p.N = (int)w.N;
-    p.nb = (int)(w.K / 32);
+    p.nb = (int)(w.K / 32);   // 32-blocks per row in every format
     p.tslots = m <= 8 ? 8 : (m <= 16 ? 16 : 32);
     const int npieces = (p.nb + 3) / 4;
     // Rows per workgroup and K slices: one workgroup per CU, so the launch takes ceil(workgroups / CUs) rounds.  Two K
@@ -360,13 +444,13 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
                            (uint4*)sc.xq, sc.xd, (float4*)y, zero_n4);
         SMX_HIP(c, hipGetLastError());
     }
-    const bool q4 = w.type == kQ4_0;
+    const int fmt = w.type == kQ4_0 ? FMT_Q4 : (w.type == kQ6_K ? FMT_Q6 : FMT_Q8);
     const int nwg = nrg * ksplit;
     const int nw = nwg <= c->num_cu ? 16 : 8;   // waves per workgroup (see the kernel)
     const bool alds = p.tslots <= 16;
-    const size_t lds = (size_t)nw * wave_lds(q4, alds);   // the reduction reuses the first nw * 4 KB
+    const size_t lds = (size_t)nw * wave_lds(fmt, alds);   // the reduction reuses the first nw * 4 KB
     const dim3 grid((unsigned)nwg);
-    ProfScope ps(c, q4 ? "skinny_q4_0" : "skinny_q8_0");
+    ProfScope ps(c, fmt == FMT_Q4 ? "skinny_q4_0" : (fmt == FMT_Q6 ? "skinny_q6_k" : "skinny_q8_0"));
     auto go = [&](auto kern) -> int {
         int rc = set_dyn_lds(c, kern, lds);
         if (rc != SMX_OK) return rc;
@@ -374,13 +458,17 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
         SMX_HIP(c, hipGetLastError());
         return SMX_OK;
     };
-#define SMX_SK_GO(Q4_, NW_, AL_) (dump ? go(skinny_kernel<Q4_, true, NW_, AL_>) : go(skinny_kernel<Q4_, false, NW_, AL_>))
-    if (nw == 16) {
-        if (q4) return alds ? SMX_SK_GO(true, 16, true) : SMX_SK_GO(true, 16, false);
-        return alds ? SMX_SK_GO(false, 16, true) : SMX_SK_GO(false, 16, false);
+#define SMX_SK_GO(F_, NW_, AL_, NA_) (dump ? go(skinny_kernel<F_, true, NW_, AL_, NA_>) : go(skinny_kernel<F_, false, NW_, AL_, NA_>))
+    if (fmt == FMT_Q6) {
+        if (nw == 16) return p.tslots == 8 ? SMX_SK_GO(FMT_Q6, 16, true, 4) : SMX_SK_GO(FMT_Q6, 16, true, 8);
+        return p.tslots == 8 ? SMX_SK_GO(FMT_Q6, 8, true, 4) : SMX_SK_GO(FMT_Q6, 8, true, 8);
     }
-    if (q4) return alds ? SMX_SK_GO(true, 8, true) : SMX_SK_GO(true, 8, false);
-    return alds ? SMX_SK_GO(false, 8, true) : SMX_SK_GO(false, 8, false);
+    if (nw == 16) {
+        if (fmt == FMT_Q4) return alds ? SMX_SK_GO(FMT_Q4, 16, true, 16) : SMX_SK_GO(FMT_Q4, 16, false, 16);
+        return alds ? SMX_SK_GO(FMT_Q8, 16, true, 16) : SMX_SK_GO(FMT_Q8, 16, false, 16);
+    }
+    if (fmt == FMT_Q4) return alds ? SMX_SK_GO(FMT_Q4, 8, true, 16) : SMX_SK_GO(FMT_Q4, 8, false, 16);
+    return alds ? SMX_SK_GO(FMT_Q8, 8, true, 16) : SMX_SK_GO(FMT_Q8, 8, false, 16);
 #undef SMX_SK_GO
 }
 

@@ -63,19 +63,21 @@ def test_gemm_declines_and_errors(accel, synth, pkg):
         accel.prefill_q8_gemm("t.e", np.zeros((16, 128), np.float32), 16, 8)
 
 
-# The small-batch kernel on the matrix cores serves 9..32 rows of a Q8_0 / Q4_0 weight of up to 12288 rows
-# (kernels.rs:830-857, 1016-1045, 1605-1632).  (type, N, K): one and two K slices per row group (two when the row
-# groups alone would leave CUs idle and K has at least 64 blocks), K not a multiple of the 4-block piece, ragged row
-# counts, fewer pieces than waves, the two decode shapes of the benchmark.
+# The small-batch kernel on the matrix cores serves 5..32 rows of a Q8_0 / Q4_0 weight (17..32 rows up to 32768 weight
+# rows) and 5..16 rows of a Q6_K weight (kernels.rs:830-857, 1016-1045, 1605-1632).  (type, N, K): one and two K slices
+# per row group (two when the row groups alone would leave CUs idle and K has at least 64 blocks), K not a multiple of
+# the 4-block piece, ragged row counts, fewer pieces than waves, row groups of fewer than 32 rows (whole rounds of
+# CUs), the two decode shapes of the benchmark, a weight taller than 32768 rows, Q6_K from one superblock to a long row.
 SMALL_BATCH = [(8, 96, 256), (8, 130, 2560), (8, 37, 9728), (2, 130, 2560), (2, 33, 4128), (8, 64, 2592), (2, 1000, 160),
-               (8, 300, 128), (2, 7, 15360), (8, 2560, 9728), (2, 9728, 2560), (8, 12288, 512)]
+               (8, 300, 128), (2, 7, 15360), (8, 2560, 9728), (2, 9728, 2560), (8, 12288, 512), (8, 40000, 256), (2, 9000, 320),
+               (14, 96, 256), (14, 130, 2560), (14, 37, 9728), (14, 1000, 512), (14, 300, 768), (14, 9000, 1024)]
 
 
 @pytest.mark.parametrize("ty,N,K", SMALL_BATCH)
 def test_small_batch_matches_oracle(accel, orc, synth, relerr, ty, N, K):
     raw = synth.make_weight(ty, N, K, seed=N + K)
     assert getattr(accel, UPLOAD[ty])("t.sb", raw, K, N)
-    for m in (9, 16, 17, 32):
+    for m in (5, 8, 9, 16, 17, 32):
         xs = synth.make_acts(m, K, seed=m + N)
         ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
         y = accel.prefill_q8_gemm("t.sb", xs, m, N)               # WeightAccel::prefill_q8_gemm with a short chunk
@@ -84,7 +86,7 @@ def test_small_batch_matches_oracle(accel, orc, synth, relerr, ty, N, K):
         assert np.array_equal(accel.prefill_q8_gemm("t.sb", xs, m, N), y)   # two K slices add in either order: same bits
         if N * K <= 400000:   # the integers behind it, dumped by the same kernel
             xq, _, _ = orc.actquant(xs, K)
-            dots = accel.gemm_block_dots("t.sb", xs, m, N, K // 32)
+            dots = accel.gemm_block_dots("t.sb", xs, m, N, K // (16 if ty == 14 else 32))
             for t in range(m):
                 assert np.array_equal(dots[t], orc.block_dots(ty, raw, K, N, xq[t])), (m, t)
     accel.evict("t.sb")
@@ -98,8 +100,8 @@ def test_small_batch_rows_equal_single_rows(accel, synth, relerr):
         xs = synth.make_acts(20, K, seed=5)
         assert getattr(accel, UPLOAD[ty])("t.sbr", raw, K, N)
         y = accel.gemv_rows("t.sbr", xs, N)
-        y8 = accel.gemv_rows("t.sbr", xs[:8], N)                    # 8 rows: the dot4 GEMV
-        assert relerr(y[:8], y8) <= TOL
+        y4 = accel.gemv_rows("t.sbr", xs[:4], N)                    # 4 rows: the dot4 GEMV
+        assert relerr(y[:4], y4) <= TOL
         for t in (0, 9, 19):
             assert relerr(y[t], accel.gemv("t.sbr", xs[t], N)) <= TOL
     with pytest.raises(Exception):
