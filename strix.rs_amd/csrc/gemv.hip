@@ -95,6 +95,7 @@ constexpr size_t kProducerSplitK = 4096;
 struct Geom {
     bool prod = false;  // an activation producer runs in the staging
     bool preq = false;  // the (single) activation row arrives quantised
+    bool rowsf = false; // 2..4 fp32 activation rows are quantised inside the flat kernel
     int flat = 0;       // flat form: lanes per group (16 or 8), 0 = not used
     int flat_pre = 0;   // its loads per round
     int rpw, pre, ks, lpr, nt;
@@ -171,6 +172,15 @@ int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nbl
         // several rows arrive quantised
         constexpr int PRE = 1;
         if (g.flat_pre == PRE) {
+            if constexpr (MT <= 4) {
+                if (g.rowsf) {   // fp32 rows, quantised by the kernel
+                    if (g.flat == 16) return launch_flat_fq<Ops, MT, PRE, 16, 1>(c, g, J, njobs, nblk, m);
+                    if (g.flat == 8) return launch_flat_fq<Ops, MT, PRE, 8, 1>(c, g, J, njobs, nblk, m);
+                    if constexpr (kQ6) {
+                        if (g.flat == 4) return launch_flat_fq<Ops, MT, PRE, 4, 1>(c, g, J, njobs, nblk, m);
+                    }
+                }
+            }
             if (g.flat == 16) return launch_flat_fq<Ops, MT, PRE, 16, 0>(c, g, J, njobs, nblk, m);
             if (g.flat == 8) return launch_flat_fq<Ops, MT, PRE, 8, 0>(c, g, J, njobs, nblk, m);
             if constexpr (kQ6) {
@@ -352,7 +362,7 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
         return launch_gemv(c, w, x + 4 * w.K, m - 4, y + 4 * w.N, nullptr, sc);   // same stream: the second pass may reuse sc
     }
     const int mt = m == 1 ? 1 : (m == 2 ? 2 : (m <= 4 ? 4 : 8));
-    const Geom g = pick_geom(c, w.type, w.N, w.nblk, mt, dump != nullptr, 1);
+    Geom g = pick_geom(c, w.type, w.N, w.nblk, mt, dump != nullptr, 1);
     if (g.lds > 160 * 1024)
         return fail(c, SMX_ERR_LIMIT, "gemv: %zu activation rows of %zu need %zu bytes of LDS (limit 163840)", m, w.K, g.lds);
     GemvJobs J = {};
@@ -360,7 +370,10 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
     J.job[0].x = x;
     J.job[0].y = y;
     J.job[0].N = (int)w.N;
-    if (mt > 1) {
+    // 2..4 rows of at most 16384 values in all: the flat kernel quantises them itself (a half block per thread), which
+    // saves the quantiser launch; longer rows are quantised once for all workgroups by their own launch
+    g.rowsf = mt > 1 && mt <= 4 && g.flat && !dump && (size_t)mt * w.K <= 16384;
+    if (mt > 1 && !g.rowsf) {
         // each of the persistent workgroups would repeat the quantiser for all m rows: do it once instead
         int rc;
         ActScratch a;

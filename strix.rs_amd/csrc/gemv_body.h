@@ -598,6 +598,39 @@ __device__ __forceinline__ float small_group_sum(float v) {
     return v;
 }
 
+// One half block (16 fp32 values in v[0..3]) of an activation row on its way into LDS, as item `hb` of the row at `tok`
+// (hb / 2 = block, hb % 2 = half): d = amax / 127 over the block (the other half sits in the neighbouring lane),
+// q = rint(x / d) (kernels.rs:75-96).  Whole lane pairs are live or not together; every lane of the wave calls this.
+template <class Ops>
+__device__ __forceinline__ void quantize_half_block(char* tok, int nblk, int hb, bool live, const float4 (&v)[4]) {
+    const float f[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
+                         v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
+    float a = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; k++) a = fmaxf(a, fabsf(f[k]));
+    a = fmaxf(a, dpp_f<0xB1>(a));   // the block's other half: the neighbouring lane
+    const float d = a / 127.f;
+    const float inv = d > 0.f ? 1.f / d : 0.f;
+    unsigned pkw[4];
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        unsigned pk = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) pk |= (unsigned)(max(-127, min(127, (int)rintf(f[4 * w + k] * inv))) & 0xff) << (8 * k);
+        pkw[w] = pk;
+    }
+    int s_half = 0;
+    if (Ops::kNeedsSums) {
+#pragma unroll
+        for (int w = 0; w < 4; w++) s_half = dot4((int)pkw[w], 0x01010101, s_half);
+    }
+    const int s_other = Ops::kNeedsSums ? dpp_i<0xB1>(s_half) : 0;
+    if (live) {
+        *(uint4*)Ops::xq_dword(tok, nblk, hb >> 1, (hb & 1) * 4) = make_uint4(pkw[0], pkw[1], pkw[2], pkw[3]);
+        if ((hb & 1) == 0) Ops::put_scale(tok, nblk, hb >> 1, d, s_half, s_other);
+    }
+}
+
 // The activation row of the flat form: every global load is requested up front (before the weight
 // stream, so that waiting for the row does not wait for the weights: a wave's loads complete in
 // order), the values are quantised and written to LDS later.  Thread t holds items t, t + 1024, ...
@@ -666,35 +699,10 @@ struct FlatX {
             }
             return;
         }
-        if (wide(nb32)) {
+        if constexpr (FQ == 1) {
             const int i = threadIdx.x;
             if ((i & ~63) >= nb32 * 2) return;   // whole waves
-            const float f[16] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
-                                 v[2].x, v[2].y, v[2].z, v[2].w, v[3].x, v[3].y, v[3].z, v[3].w};
-            float a = 0.f;
-#pragma unroll
-            for (int k = 0; k < 16; k++) a = fmaxf(a, fabsf(f[k]));
-            a = fmaxf(a, dpp_f<0xB1>(a));   // the block's other half: the neighbouring lane
-            const float d = a / 127.f;
-            const float inv = d > 0.f ? 1.f / d : 0.f;
-            unsigned pkw[4];
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                unsigned pk = 0;
-#pragma unroll
-                for (int k = 0; k < 4; k++) pk |= (unsigned)(max(-127, min(127, (int)rintf(f[4 * w + k] * inv))) & 0xff) << (8 * k);
-                pkw[w] = pk;
-            }
-            int s_half = 0;
-            if (Ops::kNeedsSums) {
-#pragma unroll
-                for (int w = 0; w < 4; w++) s_half = dot4((int)pkw[w], 0x01010101, s_half);
-            }
-            const int s_other = Ops::kNeedsSums ? dpp_i<0xB1>(s_half) : 0;
-            if (i < nb32 * 2) {
-                *(uint4*)Ops::xq_dword(tok, nblk, i >> 1, (i & 1) * 4) = make_uint4(pkw[0], pkw[1], pkw[2], pkw[3]);
-                if ((i & 1) == 0) Ops::put_scale(tok, nblk, i >> 1, d, s_half, s_other);
-            }
+            quantize_half_block<Ops>(tok, nblk, i, i < nb32 * 2, v);
             return;
         }
         const int items = nb32 * 8;
@@ -769,6 +777,33 @@ struct FlatXRows {
     }
 };
 
+// The same for up to MT fp32 rows that are quantised here (FQ = 1 with MT > 1): thread i takes half block i % hb of row
+// i / hb, hb = half blocks per row; MT * hb <= 1024 (the launcher's bound: 4 rows of up to 4096 elements).  Saves the
+// quantiser launch in front of a 2..4-row GEMV (2.5 of the 7.6 us Q4_0 9728 x 2560 takes at 2 rows).
+template <class Ops, int MT>
+struct FlatXRowsF {
+    static_assert(MT <= 4, "row = number of row boundaries at or below the thread index");
+    float4 v[4];
+    int t, h;
+
+    __device__ __forceinline__ void request(const GemvX& X, int nblk, int m) {
+        const int hb = Ops::nb32(nblk) * 2, i = threadIdx.x;
+        t = (i >= hb ? 1 : 0) + (i >= 2 * hb ? 1 : 0) + (i >= 3 * hb ? 1 : 0);
+        h = i - t * hb;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (t < m && i < MT * hb) v[j] = ((const float4*)(X.x + (size_t)t * hb * 16))[h * 4 + j];
+        }
+    }
+    // rows past m are staged as zeros (their results are not written)
+    __device__ __forceinline__ void store(char* smem, int tokb, int nblk) {
+        const int hb = Ops::nb32(nblk) * 2, i = threadIdx.x;
+        if ((i & ~63) >= MT * hb) return;   // whole waves
+        quantize_half_block<Ops>(smem + min(t, MT - 1) * tokb, nblk, h, i < MT * hb, v);
+    }
+};
+
 // Flat form for weight rows that are a whole number of GL-lane groups (GL = 16, 8 or 4 units).  Rows are contiguous in the planar layout, so the units of a workgroup's rows [r0, r1) are
 // one flat sequence: a wave load covers 64 consecutive units of it (1 KB of quants, whatever the row
 // length), wave w takes loads w, w + 16, ...  Every GL-lane group lies inside one row; its sum goes
@@ -786,7 +821,7 @@ template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP = false>
 __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, float* __restrict__ y, int ldy, int nblk,
                                                int N, int m, int wg, int n_wgs, unsigned magic_u,
                                                int* __restrict__ dump = nullptr, int dump_per_row = 0) {
-    static_assert(MT == 1 || FQ == 0, "several activation rows are staged from quantised rows");
+    static_assert(MT == 1 || FQ == 0 || FQ == 1, "several activation rows: staged from quantised rows or quantised here");
     static_assert(!DUMP || MT == 1, "the block-dot dump covers one activation row");
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -802,9 +837,12 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     // loads go to the weight's first unit
     const size_t f_base = nunits > 0 ? (size_t)r0 * U : 0;
 
-    FlatX<Ops, FQ> xs;
+    FlatX<Ops, MT == 1 ? FQ : 0> xs;
     FlatXRows<Ops, MT> xr;
+    FlatXRowsF<Ops, MT <= 4 ? MT : 4> xf;
+    constexpr bool kRowsF = MT > 1 && MT <= 4 && FQ == 1;
     if (MT == 1) xs.request(X, nblk);
+    else if (kRowsF) xf.request(X, nblk, m);
     else xr.request(X, nblk, m);
 
     typename Ops::Regs ring[PRE];
@@ -842,6 +880,7 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     };
     request();
     if (MT == 1) xs.store(smem, nblk, X);
+    else if (kRowsF) xf.store(smem, tokb, nblk);
     else xr.store(smem, tokb, nblk);
     __syncthreads();
     consume();

@@ -150,6 +150,24 @@ def test_gemv_rows_q6k(accel, orc, synth, relerr, m):
     accel.evict("t.q6rows")
 
 
+@pytest.mark.parametrize("ty,N,K", [(2, 130, 256), (8, 96, 4096), (14, 200, 4096), (2, 64, 4128), (8, 300, 8192), (14, 40, 8192), (2, 9728, 2560)])
+def test_gemv_rows_quantised_in_kernel(accel, orc, synth, relerr, ty, N, K):
+    # 2..4 fp32 rows of at most 16384 values in all (counting 4 rows for 3) are quantised by the GEMV kernel itself, a half
+    # block per thread; longer ones by a quantiser launch of their own: both sides of the bound, a row of eight blocks,
+    # three rows in the four-row variant (its fourth row is staged as zeros)
+    raw = synth.make_weight(ty, N, K, seed=N + K)
+    _up(accel, ty, "t.rq", raw, K, N)
+    for m in (2, 3, 4):
+        xs = synth.make_acts(m, K, seed=m + K)
+        xs[m - 1, 32:64] = 0.0                # an all-zero block: d = 0
+        y = accel.gemv_rows("t.rq", xs, N)
+        ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
+        assert y.shape == ref.shape and relerr(y, ref) <= TOL, m
+        for t in range(m):                    # the single-row kernel quantises with the same arithmetic
+            assert relerr(y[t], accel.gemv("t.rq", xs[t], N)) <= TOL, (m, t)
+    accel.evict("t.rq")
+
+
 def test_gemv_rows_long_k_batched(accel, orc, synth, relerr):
     # the batched verify shape: Q8_0 2560 x 9728, M = 8 (large LDS staging, 16-wave groups)
     N, K, m = 2560, 9728, 8
