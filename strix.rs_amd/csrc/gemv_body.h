@@ -74,6 +74,25 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// The same moves for a double (both halves), and the sum over the 64 lanes of a wave in a fixed order: lane 63 ends up
+// holding the total.  (__shfl_xor on a double is two LDS permutes per step, six steps one after the other.)
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ double dpp_d(double v) {
+    const long long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)b, CTRL, ROW_MASK, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, ROW_MASK, 0xf, false);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+    v += dpp_d<0xB1>(v);
+    v += dpp_d<0x4E>(v);
+    v += dpp_d<0x141>(v);
+    v += dpp_d<0x140>(v);
+    v += dpp_d<0x142, 0xa>(v);
+    v += dpp_d<0x143, 0xc>(v);
+    return v;
+}
+
 // Pointers of one resident weight (planar layout) and of the activation.
 struct GemvW {
     const uint16_t* scales;  // Q4_0/Q8_0: f16 per block; Q6_K: f16 d per superblock
@@ -647,17 +666,23 @@ struct FlatX {
     // divisions, the 16-element sums, the scale's LDS write) runs once per 2 lanes instead of once per 8: with
     // one float4 per thread the staging held every CU for 1 us before it could touch its weights on a
     // 9728-element row, and Q6_K 15360 x 3840 ran 0.6 us longer.  Same arithmetic per element, same results.
-    static __device__ __forceinline__ bool wide(int) { return FQ == 1; }
+    // rmsnorm in front of the quantiser (FQ == 2) uses the same mapping; the exp-based producers keep one float4 per thread
+    // (their per-element work is what counts, and it spreads over four times as many threads).
+    static __device__ __forceinline__ bool wide(const GemvX& X) { return FQ == 1 || (FQ == 2 && X.prod == SMX_ACT_RMSNORM); }
 
     __device__ __forceinline__ void request(const GemvX& X, int nblk) {
         const int nb32 = Ops::nb32(nblk);
         const int items = FQ == 0 ? nb32 * 2 : nb32 * 8;
-        if (wide(nb32)) {
+        if (wide(X)) {
             const int i = threadIdx.x;   // half block
 #pragma unroll
             for (int j = 0; j < XI; j++) {
                 v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (i < nb32 * 2) v[j] = ((const float4*)X.x)[i * 4 + j];
+                v2[j] = make_float4(1.f, 1.f, 1.f, 1.f);
+                if (i < nb32 * 2) {
+                    v[j] = ((const float4*)X.x)[i * 4 + j];
+                    if (FQ == 2 && X.x2) v2[j] = ((const float4*)X.x2)[i * 4 + j];
+                }
             }
             return;
         }
@@ -705,30 +730,39 @@ struct FlatX {
             quantize_half_block<Ops>(tok, nblk, i, i < nb32 * 2, v);
             return;
         }
-        const int items = nb32 * 8;
-        float rs = 1.f;
-        if (FQ == 2 && X.prod == SMX_ACT_RMSNORM) {
-            // the reduction of rms_scale over the values already in registers (same elements per thread, same order)
+        if constexpr (FQ == 2) {
+            if (X.prod == SMX_ACT_RMSNORM) {   // workgroup-uniform
 #pragma clang fp contract(off)
-            double ss = 0.0;
+                const int i = threadIdx.x;
+                // mean of squares in double over the values already in registers (threads past the row hold zeros), rounded to
+                // fp32 once: independent of the summation order
+                double ss = 0.0;
 #pragma unroll
-            for (int j = 0; j < XI; j++) {
-                if ((int)threadIdx.x + j * 1024 < items) {
+                for (int j = 0; j < XI; j++) {
                     ss += (double)v[j].x * (double)v[j].x;
                     ss += (double)v[j].y * (double)v[j].y;
                     ss += (double)v[j].z * (double)v[j].z;
                     ss += (double)v[j].w * (double)v[j].w;
                 }
+                ss = wave_sum_d(ss);
+                double* red = (double*)tok;
+                if ((i & 63) == 63) red[i >> 6] = ss;
+                __syncthreads();
+                double tot = 0.0;
+                for (int w = 0; w < 16; w++) tot += red[w];
+                __syncthreads();
+                const float rs = (float)(1.0 / sqrt(tot / (double)(nb32 * 32) + (double)X.eps));
+                if ((i & ~63) >= nb32 * 2) return;   // whole waves
+                float4 w4[4];
+#pragma unroll
+                for (int j = 0; j < XI; j++)
+                    w4[j] = make_float4((v[j].x * rs) * v2[j].x, (v[j].y * rs) * v2[j].y, (v[j].z * rs) * v2[j].z, (v[j].w * rs) * v2[j].w);
+                quantize_half_block<Ops>(tok, nblk, i, i < nb32 * 2, w4);
+                return;
             }
-            for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off);
-            double* red = (double*)tok;
-            if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
-            __syncthreads();
-            double tot = 0.0;
-            for (int w = 0; w < 16; w++) tot += red[w];
-            __syncthreads();
-            rs = (float)(1.0 / sqrt(tot / (double)(nb32 * 32) + (double)X.eps));
         }
+        const int items = nb32 * 8;
+        const float rs = 1.f;   // (rmsnorm is handled above)
 #pragma unroll
         for (int j = 0; j < XI; j++) {
             const int i = threadIdx.x + j * 1024;
