@@ -25,6 +25,7 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "smx_internal.h"
 
@@ -76,9 +77,15 @@ __device__ __forceinline__ void load_to_lds16(const void* g, unsigned lds_base) 
                  : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(g)
                  : "memory", "m0");
 }
-// four 6-bit quants (low nibbles in lo4, the two high bits in hi2) -> four signed bytes q - 32
-__device__ __forceinline__ unsigned q6_bytes_s(unsigned lo4, unsigned hi2) {
-    return (((lo4 & 0x0f0f0f0fu) | ((hi2 & 0x03030303u) << 4) | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+// Four 6-bit quants -> four signed bytes q - 32.  ql: the dword whose nibbles (low: LS = 0, high: LS = 4) are the low four
+// bits; qh: the dword whose bit pairs HS, HS + 1 of every byte are the high two.  q + 96 stays below 256 in every byte, and
+// flipping bit 7 then subtracts 128 where it is set and adds 128 (= -128 mod 256) where it is not: two operations after
+// the merge, five or six per dword in all.
+template <int LS, int HS>
+__device__ __forceinline__ unsigned q6_bytes_s(unsigned ql, unsigned qh) {
+    const unsigned hi = (HS <= 4 ? qh << (4 - HS) : qh >> (HS - 4)) & 0x30303030u;
+    const unsigned q = ((ql >> LS) & 0x0f0f0f0fu) | hi;
+    return (q + 0x60606060u) ^ 0x80808080u;
 }
 
 __device__ __forceinline__ unsigned lds_addr(const void* p) {
@@ -210,17 +217,18 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
             const int r = lane >> 1, pp = lane & 1;
             const uint4 qa = *(const uint4*)(mine + r * 64 + pp * 16), qb = *(const uint4*)(mine + r * 64 + 32 + pp * 16);
             const uint4 h = *(const uint4*)(mine + 2048 + r * 32 + pp * 16);
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
+            auto chunk = [&](auto jc) {   // chunk 2j + p: ql nibble j / 2 of ql half j % 2, bit pair 2j of qh
+                constexpr int j = decltype(jc)::value;
                 const uint4 q = (j & 1) ? qb : qa;
-                const int ls = (j >> 1) * 4, hs = 2 * j;
                 uint4 o;
-                o.x = q6_bytes_s(q.x >> ls, h.x >> hs);
-                o.y = q6_bytes_s(q.y >> ls, h.y >> hs);
-                o.z = q6_bytes_s(q.z >> ls, h.z >> hs);
-                o.w = q6_bytes_s(q.w >> ls, h.w >> hs);
+                o.x = q6_bytes_s<(j >> 1) * 4, 2 * j>(q.x, h.x);
+                o.y = q6_bytes_s<(j >> 1) * 4, 2 * j>(q.y, h.y);
+                o.z = q6_bytes_s<(j >> 1) * 4, 2 * j>(q.z, h.z);
+                o.w = q6_bytes_s<(j >> 1) * 4, 2 * j>(q.w, h.w);
                 *(uint4*)(wide + r * 128 + ((2 * j + pp + r) & 7) * 16) = o;   // elements 32 j + 16 p .. + 15 of the piece
-            }
+            };
+            chunk(std::integral_constant<int, 0>()); chunk(std::integral_constant<int, 1>());
+            chunk(std::integral_constant<int, 2>()); chunk(std::integral_constant<int, 3>());
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -268,14 +276,15 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
             const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero scale
             const float dxv = __uint_as_float(dxs[bi]);
             if constexpr (Q6) {
-                const float d6 = h2f_s(r.d6);
+                const float d6 = h2f_s(r.d6), d6m128 = -128.f * d6;
 #pragma unroll
                 for (int jj = 0; jj < 2; jj++) {   // sub-block jj: chunk 2 bi + jj; a lane holds bytes 8 half .. + 7 of it on both sides
                     const long bw = *(const long*)(buf + col * 128 + ((2 * bi + jj + col) & 7) * 16 + half * 8);
                     const long aw = *(const long*)(mine_a + ((bi * 2 + jj) * p.tslots + min(col, p.tslots - 1)) * 16 + half * 8);
                     const v16i d = __builtin_amdgcn_mfma_i32_32x32x16_i8(aw, bw, cmagic, 0, 0, 0);
-                    const unsigned sc8 = (2 * bi + jj) < 4 ? r.dw.x >> (8 * (2 * bi + jj)) : r.dw.y >> (8 * (2 * bi + jj - 4));
-                    const float dw = d6 * (float)(int)(signed char)(sc8 & 0xff);   // exact in fp32 (11 x 8 significant bits)
+                    // d * sc, exact in fp32 (11 x 8 significant bits): sc + 128 as an unsigned byte -> float, then one FMA
+                    const unsigned scw = ((2 * bi + jj) < 4 ? r.dw.x : r.dw.y) ^ 0x80808080u;
+                    const float dw = fmaf((float)((scw >> (8 * ((2 * bi + jj) & 3))) & 0xffu), d6, d6m128);
                     rescale(d, dw, dxv);
                     if (DUMP) {
                         const int row = r0 + col;
