@@ -622,6 +622,8 @@ def main():
         ("q8_0_small_batch_2560x9728_m16", lambda: b.gemv("q8_0_small_batch_2560x9728_m16", Q8_0, 2560, 9728, 16, int(1.1 * GB))),
         ("q8_0_small_batch_2560x9728_m32", lambda: b.gemv("q8_0_small_batch_2560x9728_m32", Q8_0, 2560, 9728, 32, int(1.1 * GB))),
         ("q4_0_gemv_f32_9728x2560", lambda: b.gemv("q4_0_gemv_f32_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB), f32=True)),
+        ("q8_0_gemv_f32_2560x9728", lambda: b.gemv("q8_0_gemv_f32_2560x9728", Q8_0, 2560, 9728, 1, int(1.1 * GB), f32=True)),
+        ("q6_k_gemv_f32_15360x3840", lambda: b.gemv("q6_k_gemv_f32_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB), f32=True)),
         ("q6_k_gemv_15360x3840", lambda: b.gemv("q6_k_gemv_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB))),
         ("q6_k_lm_head_262144x3840", lambda: b.gemv("q6_k_lm_head_262144x3840", Q6_K, 262144, 3840, 1, int(1.6 * GB),
                                                      steps=max(10, a.steps // 10), warmup=2)),

@@ -26,6 +26,8 @@ def test_decode_gemv_full_size(accel, orc, synth, relerr, ty, N, K):
         ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
         for m in (2, 3, 8):
             assert relerr(accel.gemv_rows("t.full", xs[:m], N), ref[:m]) <= TOL
+    # the fp32-activation form of the same weight against the f32 oracle
+    assert relerr(accel.gemv_f32("t.full", x, N), orc.matmul_f32(ty, raw, K, N, x, order=0)[0]) <= TOL
     accel.evict("t.full")
 
 
@@ -48,7 +50,30 @@ def test_lm_head_q6k_sampled(accel, orc, synth, relerr):
     refs = orc.matmul_q8_from_f32(14, sub, K, rows.size, xs)
     assert np.abs(ys[:, rows] - refs).max() / np.abs(ys).max() <= TOL
     assert [int(v) for v in accel.lm_head_argmax_rows("t.head", xs, 3)] == [int(np.argmax(r)) for r in ys]
+    # fp32 activations: a CU's share is 1024 rows x 60 units, just inside the flat form's 16-bit unit index
+    yf = accel.gemv_f32("t.head", x, N)
+    reff = orc.matmul_f32(14, sub, K, rows.size, x, order=0)[0]
+    assert np.abs(yf[rows] - reff).max() / np.abs(yf).max() <= TOL
     accel.evict("t.head")
+
+
+def test_gemv_f32_two_rounds_of_workgroups(accel, orc, synth):
+    # 33000 rows of 512 units: a CU's share (129 rows) no longer fits the flat form's 16-bit unit index, so the launch
+    # takes two rounds of workgroups; oracle on sampled rows
+    ty, N, K = 8, 33000, 8192
+    raw = synth.make_weight(ty, N, K, seed=77)
+    x = synth.make_acts(1, K, seed=78)
+    assert accel.upload_q8_0("t.rounds", raw, K, N)
+    y = accel.gemv_f32("t.rounds", x, N)
+    rows = np.unique(np.concatenate([np.arange(0, 140), np.arange(N - 140, N), np.random.default_rng(2).integers(0, N, 600)]))
+    sub = raw.reshape(N, -1)[rows].reshape(-1)
+    ref = orc.matmul_f32(ty, sub, K, rows.size, x, order=0)[0]
+    assert np.abs(y[rows] - ref).max() / np.abs(y).max() <= TOL
+    # and the int8-activation form of the same launch geometry
+    yq = accel.gemv("t.rounds", x, N)
+    refq = orc.matmul_q8_from_f32(ty, sub, K, rows.size, x)[0]
+    assert np.abs(yq[rows] - refq).max() / np.abs(yq).max() <= TOL
+    accel.evict("t.rounds")
 
 
 @pytest.mark.parametrize("ty,M,N,K", [(8, 2048, 15360, 3840), (2, 2048, 15360, 3840), (8, 2048, 3840, 15360), (2, 2048, 3840, 15360),

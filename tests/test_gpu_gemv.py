@@ -262,7 +262,13 @@ def test_reference_device_test_through_both_gemv_forms(accel, orc):
     accel.evict("t.ref")
 
 
-@pytest.mark.parametrize("ty,N,K", SHAPES + [(2, 9728, 2560), (8, 2560, 9728), (14, 1000, 3840), (2, 5, 32768)])
+# flat form: rows of up to 16384 elements in whole unit groups; the row-per-wave form: the others (96, 4128, 32 * 67,
+# 16384 + 512 and 32768 elements)
+F32_SHAPES = SHAPES + FORM_SHAPES + [(2, 9728, 2560), (8, 2560, 9728), (14, 1000, 3840), (2, 5, 32768), (2, 300, 16384),
+                                     (8, 200, 8192), (14, 257, 16384), (2, 100000, 256)]
+
+
+@pytest.mark.parametrize("ty,N,K", F32_SHAPES)
 def test_gemv_f32_matches_f32_oracle(accel, orc, synth, relerr, ty, N, K):
     raw = synth.make_weight(ty, N, K, seed=19 * N + K)
     x = synth.make_acts(1, K, seed=3 * N + K)
