@@ -22,41 +22,72 @@ int ensure_act(smx_ctx* c, size_t m, size_t K) {
     return ensure(c, c->xs, m * (K / 32) * 4);
 }
 
-// argmax per row of y[m][N], lowest index on ties (strict '>' scan order of decode.rs:3677-3683).
-__global__ __launch_bounds__(256) void argmax_rows_kernel(const float* __restrict__ y, size_t N,
-                                                          unsigned* __restrict__ out) {
-    const float* row = y + (size_t)blockIdx.x * N;
-    float best = -INFINITY;
-    size_t bi = 0;
-    bool have = false;
-    for (size_t i = threadIdx.x; i < N; i += 256) {  // ascending i: strict '>' keeps the lowest index
-        const float v = row[i];
-        if (!have || v > best) {
-            best = v;
-            bi = i;
-            have = true;
-        }
-    }
-    __shared__ float sb[256];
-    __shared__ size_t si[256];
-    __shared__ int sh[256];
-    sb[threadIdx.x] = best;
-    si[threadIdx.x] = bi;
-    sh[threadIdx.x] = have ? 1 : 0;
+// argmax per row of y[m][N], lowest index on ties (strict '>' scan order of decode.rs:3677-3683), in two launches:
+// workgroup (chunk, row) finds the best of kArgmaxChunk consecutive logits, one workgroup per row then takes the best of
+// the chunks.  (One workgroup scanning a 262144-entry row alone took 265 us, more than the lm_head GEMV in front of it.)
+constexpr int kArgmaxChunk = 2048;
+struct Best { float v; unsigned i; };
+// the better of two candidates: larger value, lower index on equal values; index 0xffffffff = none yet
+__device__ __forceinline__ Best better(Best a, Best b) {
+    const bool take = b.i != 0xffffffffu && (a.i == 0xffffffffu || b.v > a.v || (b.v == a.v && b.i < a.i));
+    return take ? b : a;
+}
+__device__ __forceinline__ Best workgroup_best(Best me) {   // 256 threads; valid in thread 0
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) me = better(me, Best{__shfl_xor(me.v, o), (unsigned)__shfl_xor((int)me.i, o)});
+    __shared__ float sv[4];
+    __shared__ unsigned si[4];
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = me.v; si[threadIdx.x >> 6] = me.i; }
     __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if ((int)threadIdx.x < s) {
-            const int o = threadIdx.x + s;
-            if (sh[o] && (!sh[threadIdx.x] || sb[o] > sb[threadIdx.x] ||
-                          (sb[o] == sb[threadIdx.x] && si[o] < si[threadIdx.x]))) {
-                sb[threadIdx.x] = sb[o];
-                si[threadIdx.x] = si[o];
-                sh[threadIdx.x] = 1;
-            }
-        }
-        __syncthreads();
+    Best r = Best{sv[0], si[0]};
+#pragma unroll
+    for (int w = 1; w < 4; w++) r = better(r, Best{sv[w], si[w]});
+    return r;
+}
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ y, size_t N, int nchunks,
+                                                            float* __restrict__ pv, unsigned* __restrict__ pi) {
+    const float* row = y + (size_t)blockIdx.y * N;
+    const size_t base = (size_t)blockIdx.x * kArgmaxChunk;
+    float v[kArgmaxChunk / 256];
+#pragma unroll
+    for (int j = 0; j < kArgmaxChunk / 256; j++) {   // all loads first
+        const size_t i = base + j * 256 + threadIdx.x;
+        v[j] = i < N ? row[i] : 0.f;
     }
-    if (threadIdx.x == 0) out[blockIdx.x] = (unsigned)si[0];
+    Best me = Best{0.f, 0xffffffffu};
+#pragma unroll
+    for (int j = 0; j < kArgmaxChunk / 256; j++) {
+        const size_t i = base + j * 256 + threadIdx.x;
+        if (i < N && !(v[j] != v[j])) me = better(me, Best{v[j], (unsigned)i});   // NaN never wins
+    }
+    const Best r = workgroup_best(me);
+    if (threadIdx.x == 0) {
+        pv[(size_t)blockIdx.y * nchunks + blockIdx.x] = r.v;
+        pi[(size_t)blockIdx.y * nchunks + blockIdx.x] = r.i;
+    }
+}
+__global__ __launch_bounds__(256) void argmax_final_kernel(const float* __restrict__ pv, const unsigned* __restrict__ pi,
+                                                           int nchunks, unsigned* __restrict__ out) {
+    Best me = Best{0.f, 0xffffffffu};
+    for (int c = threadIdx.x; c < nchunks; c += 256)
+        me = better(me, Best{pv[(size_t)blockIdx.x * nchunks + c], pi[(size_t)blockIdx.x * nchunks + c]});
+    const Best r = workgroup_best(me);
+    if (threadIdx.x == 0) out[blockIdx.x] = r.i == 0xffffffffu ? 0u : r.i;   // a row of NaNs: index 0
+}
+
+// ids[m] (device) = argmax of each row of y[m][N]; `part`: m * ceil(N / kArgmaxChunk) * 8 bytes of device scratch
+static size_t argmax_scratch_bytes(size_t m, size_t N) { return m * ((N + kArgmaxChunk - 1) / kArgmaxChunk) * 8; }
+static int launch_argmax_rows(smx_ctx* c, const float* y, size_t m, size_t N, void* part, unsigned* ids) {
+    if (N >= 0xffffffffull) return fail(c, SMX_ERR_LIMIT, "argmax: %zu entries per row exceed the 32-bit index", N);
+    const int nchunks = (int)((N + kArgmaxChunk - 1) / kArgmaxChunk);
+    float* pv = (float*)part;
+    unsigned* pi = (unsigned*)(pv + m * (size_t)nchunks);
+    ProfScope ps(c, "argmax_rows");
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3((unsigned)nchunks, (unsigned)m), dim3(256), 0, c->stream, y, N, nchunks, pv, pi);
+    SMX_HIP(c, hipGetLastError());
+    hipLaunchKernelGGL(argmax_final_kernel, dim3((unsigned)m), dim3(256), 0, c->stream, (const float*)pv, (const unsigned*)pi, nchunks, ids);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
 }
 
 // quantise m device rows and run the right matmul kernel into y_dev
@@ -243,16 +274,13 @@ int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t
     int rc;
     if ((rc = ensure(c, c->xf32, m * w->K * 4)) != SMX_OK) return rc;
     if ((rc = ensure(c, c->yf32, m * w->N * 4)) != SMX_OK) return rc;
-    if ((rc = ensure(c, c->tab, m * 4)) != SMX_OK) return rc;
+    const size_t ids_bytes = (m * 4 + 255) & ~size_t(255);   // ids, then the chunk candidates
+    if ((rc = ensure(c, c->tab, ids_bytes + argmax_scratch_bytes(m, w->N))) != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(c->xf32.p, xs, m * w->K * 4, hipMemcpyHostToDevice, c->stream));
     rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, false, nullptr, nullptr);
     if (rc != SMX_OK) return rc;
-    {
-        ProfScope ps(c, "argmax_rows");
-        hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)m), dim3(256), 0, c->stream, (const float*)c->yf32.p,
-                           w->N, (unsigned*)c->tab.p);
-        SMX_HIP(c, hipGetLastError());
-    }
+    rc = launch_argmax_rows(c, (const float*)c->yf32.p, m, w->N, (char*)c->tab.p + ids_bytes, (unsigned*)c->tab.p);
+    if (rc != SMX_OK) return rc;
     SMX_HIP(c, hipMemcpyAsync(out, c->tab.p, m * 4, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
     return SMX_OK;

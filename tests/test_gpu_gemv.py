@@ -225,6 +225,29 @@ def test_lm_head_argmax_rows(accel, orc, synth):
             assert ref[t, got[t]] >= ref[t].max() - 1e-5 * np.abs(ref[t]).max()
 
 
+def test_lm_head_argmax_ties_take_the_lowest_index(accel, synth):
+    """Identical weight rows give bit-identical logits: the strict '>' scan of the reference (decode.rs:3677-3683)
+    keeps the first of them.  The winning row is copied to places in other chunks of the two-stage argmax."""
+    N, K, m = 9000, 256, 3
+    raw = synth.make_weight(8, N, K, seed=5).reshape(N, -1).copy()
+    xs = synth.make_acts(m, K, seed=6)
+    assert accel.upload_q8_0("t.tie", raw.reshape(-1), K, N)
+    y = accel.gemv_rows("t.tie", xs, N)
+    top = [int(np.argmax(r)) for r in y]
+    dup = raw.copy()
+    for t in top:                       # every row's winner also sits later in its own chunk and in later chunks
+        for pos in (t + 1, 2048 + 7, 4096 + 300, N - 1):
+            if pos != t and pos < N and pos not in top:
+                dup[pos] = raw[t]
+    assert accel.upload_q8_0("t.tie", dup.reshape(-1), K, N)
+    y2 = accel.gemv_rows("t.tie", xs, N)
+    got = [int(v) for v in accel.lm_head_argmax_rows("t.tie", xs, m)]
+    assert got == [int(np.argmax(r)) for r in y2]     # numpy's argmax also returns the first maximum
+    for t, g in zip(range(m), got):
+        assert (y2[t] == y2[t, g]).sum() >= 2 or g == top[t]
+    accel.evict("t.tie")
+
+
 def _reference_device_test_data(orc, in_dim=15360, out_dim=3840):
     """The data of the reference's own device test (strix-backend-rocm/src/lib.rs:135-153): LCG
     0xA5A5_1234, per block one draw for the scale 0.03 + (r % 32) * 0.003 (made f16 by truncating the
