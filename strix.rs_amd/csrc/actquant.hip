@@ -62,9 +62,12 @@ __global__ __launch_bounds__(256) void actprod_quant_kernel(const ProdRows R, in
     }
 }
 
-// m rows through an activation producer and the quantiser, one workgroup per row: the prefill form of
-// the producers (kernels.rs:101-147 rmsnorm_xquant per row, :1174-1187 silu_quant_rows).  b: rmsnorm
-// weight [K] (or null) shared by the rows (b_stride 0), or the second operand [m][K] of silu / gelu.
+// m rows through an activation producer and the quantiser: the prefill form of the producers (kernels.rs:101-147
+// rmsnorm_xquant per row, :1174-1187 silu_quant_rows).  b: rmsnorm weight [K] (or null) shared by the rows
+// (b_stride 0), or the second operand [m][K] of silu / gelu.  Workgroup (row, part) takes the 256-item slices
+// part, part + gridDim.y, ... of its row: rmsnorm needs the whole row's sum of squares and runs one workgroup per
+// row; the exp-based producers have independent blocks and spread a row over one workgroup per slice (a single
+// workgroup per 9728-element row left 64 rows on 64 of the 256 CUs, ten exp-heavy rounds each).
 __global__ __launch_bounds__(256) void rows_prod_quant_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                               size_t b_stride, int kind, float eps, int* __restrict__ xq4,
                                                               float* __restrict__ xd, int* __restrict__ xs, int nb32) {
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(256) void rows_prod_quant_kernel(const float* __res
     float rs = 1.f;
     if (kind == SMX_ACT_RMSNORM) rs = rms_scale((char*)red, ar, nb32 * 32, eps);
     const int items = nb32 * 8;
-    for (int i0 = 0; i0 < items; i0 += 256) {  // whole 8-lane groups stay together: items % 8 == 0
+    for (int i0 = blockIdx.y * 256; i0 < items; i0 += gridDim.y * 256) {  // whole 8-lane groups stay together: items % 8 == 0
         const int i = i0 + threadIdx.x;
         const bool live = i < items;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f), g = make_float4(1.f, 1.f, 1.f, 1.f);
@@ -123,7 +126,8 @@ int launch_rows_prod_quant(smx_ctx* c, int kind, const float* a, const float* b,
     if (kind != SMX_ACT_RMSNORM && kind != SMX_ACT_SILU_MUL && kind != SMX_ACT_GEGLU)
         return fail(c, SMX_ERR_ARG, "producer quantiser: kind %d", kind);
     ProfScope ps(c, "rows_prod_quant");
-    hipLaunchKernelGGL(rows_prod_quant_kernel, dim3((unsigned)m), dim3(256), 0, c->stream, a, b,
+    const unsigned parts = kind == SMX_ACT_RMSNORM ? 1u : (unsigned)std::min<size_t>((K / 4 + 255) / 256, 65535);
+    hipLaunchKernelGGL(rows_prod_quant_kernel, dim3((unsigned)m, parts), dim3(256), 0, c->stream, a, b,
                        kind == SMX_ACT_RMSNORM ? (size_t)0 : K, kind, eps, (int*)xq, xd, (int*)xs, (int)(K / 32));
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
