@@ -113,7 +113,8 @@ struct PieceRegs {
 // instructions), the wave widens them to signed int8 in operand order (thread = [row:5][p:1] makes the 16-byte chunks 2j + p,
 // ggml_quant.rs:417-426), and a 32-block is two v_mfma_i32_32x32x16_i8, one per 16-element sub-block with its own d * sc.
 // NACC: accumulators per lane that hold live tokens (accumulator i of lane half h is token (i / 4) * 8 + 4 h + i % 4: 4 for up
-// to 8 token slots, 8 for 16); only those are rescaled -- with all 16 the Q6_K variant would be bound by its vector ALU work.
+// to 8 token slots, 8 for 16); only those are rescaled -- with all 16 the Q6_K variant would be bound by its vector ALU work,
+// and Q4_0 9728 x 2560 takes 1.3 us longer at 5..16 rows.
 template <int FMT, bool DUMP, int NW, bool ALDS, int NACC = 16>
 __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     constexpr bool Q4 = FMT == FMT_Q4, Q6 = FMT == FMT_Q6;
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
                 if (DUMP) {
                     const int row = r0 + col;
 #pragma unroll
-                    for (int i = 0; i < 16; i++) {
+                    for (int i = 0; i < NACC; i++) {
                         const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
                         if (live && tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
                     }
@@ -394,8 +395,8 @@ __global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restri
 
 }  // namespace
 
-// Measured on MI355X (Q8_0 2560 x 9728 / Q4_0 9728 x 2560 / Q8_0 9728 x 2560, quantiser launch included): 11.0 / 10.9 /
-// 10.7 us at 5 rows, 12.3 / 12.0 / 11.9 us at 16 rows and 14.3 / 12.5 / 13.7 us at 32 rows; the dot4 GEMV takes 13.3 /
+// Measured on MI355X (Q8_0 2560 x 9728 / Q4_0 9728 x 2560 / Q8_0 9728 x 2560, quantiser launch included): 10.4 / 9.6 /
+// 10.1 us at 5 rows, 12.0 / 10.7 / 11.6 us at 16 rows and 14.3 / 12.6 / 13.7 us at 32 rows; the dot4 GEMV takes 13.3 /
 // 11.8 / 13.0 us at 5 rows and 13.9 / 12.3 / 13.0 us at 8, 10.9 / 9.0 / 10.7 us at 4 (where it stays), and the tiled
 // GEMM with split-K 22 - 27 us.
 bool skinny_serves(const Weight& w, size_t m) {
@@ -472,12 +473,12 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
         if (nw == 16) return p.tslots == 8 ? SMX_SK_GO(FMT_Q6, 16, true, 4) : SMX_SK_GO(FMT_Q6, 16, true, 8);
         return p.tslots == 8 ? SMX_SK_GO(FMT_Q6, 8, true, 4) : SMX_SK_GO(FMT_Q6, 8, true, 8);
     }
-    if (nw == 16) {
-        if (fmt == FMT_Q4) return alds ? SMX_SK_GO(FMT_Q4, 16, true, 16) : SMX_SK_GO(FMT_Q4, 16, false, 16);
-        return alds ? SMX_SK_GO(FMT_Q8, 16, true, 16) : SMX_SK_GO(FMT_Q8, 16, false, 16);
-    }
-    if (fmt == FMT_Q4) return alds ? SMX_SK_GO(FMT_Q4, 8, true, 16) : SMX_SK_GO(FMT_Q4, 8, false, 16);
-    return alds ? SMX_SK_GO(FMT_Q8, 8, true, 16) : SMX_SK_GO(FMT_Q8, 8, false, 16);
+    // live accumulators per lane: 4 with up to 8 token slots, 8 with 16, all 16 with 32
+#define SMX_SK_ROWS(F_, NW_)                                                                      \
+    (p.tslots == 8 ? SMX_SK_GO(F_, NW_, true, 4) : (p.tslots == 16 ? SMX_SK_GO(F_, NW_, true, 8) : SMX_SK_GO(F_, NW_, false, 16)))
+    if (nw == 16) return fmt == FMT_Q4 ? SMX_SK_ROWS(FMT_Q4, 16) : SMX_SK_ROWS(FMT_Q8, 16);
+    return fmt == FMT_Q4 ? SMX_SK_ROWS(FMT_Q4, 8) : SMX_SK_ROWS(FMT_Q8, 8);
+#undef SMX_SK_ROWS
 #undef SMX_SK_GO
 }
 
