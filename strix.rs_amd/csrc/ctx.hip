@@ -1,6 +1,5 @@
 // Context, weight residency (upload + repack to planar HBM layout), scratch and profiling.
 #include <cstring>
-#include <memory>
 
 #include "smx_internal.h"
 
@@ -109,9 +108,51 @@ static void drop_weight(smx_ctx* c, Weight& w) {
     w.base = nullptr;
 }
 
-// Host-side repack of raw GGUF blocks into the planar layout (the reference
-// repacks on the host too: decode.rs:2500-2509, 2639-2664, 2693-2700), then one
-// copy to a fresh device allocation.
+// ---- repack of raw GGUF blocks into the planar layout, on the device.  (The reference repacks on the host,
+//      decode.rs:2500-2509, 2639-2664, 2693-2700; so did this library at first, at 4 GB/s of one host core: the raw
+//      bytes now cross PCIe as they are, 30 GB/s from pageable memory, and a kernel of a few microseconds per 100 MB splits them
+//      into planes.)  A workgroup copies a run of whole blocks into LDS with 16-byte loads -- 8 blocks of every format are a
+//      multiple of 16 bytes -- and writes every plane with 16-byte stores; block fields are only 2-byte aligned, so LDS
+//      is read in 16-bit pieces. ----
+constexpr int kRepackBlocks = 256;   // blocks per workgroup (Q6_K: 128)
+__device__ __forceinline__ uint4 lds_bytes16(const uint16_t* l16, int byte_off) {   // 16 bytes at an even offset
+    const uint16_t* p = l16 + (byte_off >> 1);
+    return make_uint4(p[0] | ((unsigned)p[1] << 16), p[2] | ((unsigned)p[3] << 16), p[4] | ((unsigned)p[5] << 16),
+                      p[6] | ((unsigned)p[7] << 16));
+}
+// BB = 18 (Q4_0) or 34 (Q8_0): f16 scale, then 16 or 32 bytes of quants
+template <int BB>
+__global__ __launch_bounds__(256) void repack_q4q8_kernel(const uint4* __restrict__ raw, size_t total, uint16_t* __restrict__ scales,
+                                                          uint4* __restrict__ quants) {
+    __shared__ __align__(16) uint16_t lds[kRepackBlocks * BB / 2];
+    const size_t b0 = (size_t)blockIdx.x * kRepackBlocks;
+    const int nblk = (int)min((size_t)kRepackBlocks, total - b0);
+    const int n16 = (nblk * BB + 15) / 16;   // the raw buffer is padded to a multiple of 16 bytes
+    for (int i = threadIdx.x; i < n16; i += 256) ((uint4*)lds)[i] = raw[b0 * BB / 16 + i];
+    __syncthreads();
+    constexpr int QV = (BB - 2) / 16;   // 16-byte pieces of quants per block
+    if ((int)threadIdx.x < nblk) scales[b0 + threadIdx.x] = lds[threadIdx.x * (BB / 2)];
+    for (int i = threadIdx.x; i < nblk * QV; i += 256)
+        quants[b0 * QV + i] = lds_bytes16(lds, (i / QV) * BB + 2 + (i % QV) * 16);
+}
+// Q6_K block: ql 128 | qh 64 | 16 sub-block scales | f16 d (210 bytes)
+__global__ __launch_bounds__(256) void repack_q6k_kernel(const uint4* __restrict__ raw, size_t total, uint4* __restrict__ ql,
+                                                         uint4* __restrict__ qh, uint4* __restrict__ sc, uint16_t* __restrict__ d) {
+    constexpr int NB = kRepackBlocks / 2;
+    __shared__ __align__(16) uint16_t lds[NB * 105];
+    const size_t b0 = (size_t)blockIdx.x * NB;
+    const int nblk = (int)min((size_t)NB, total - b0);
+    const int n16 = (nblk * 210 + 15) / 16;
+    for (int i = threadIdx.x; i < n16; i += 256) ((uint4*)lds)[i] = raw[b0 * 210 / 16 + i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < nblk * 8; i += 256) ql[b0 * 8 + i] = lds_bytes16(lds, (i >> 3) * 210 + (i & 7) * 16);
+    for (int i = threadIdx.x; i < nblk * 4; i += 256) qh[b0 * 4 + i] = lds_bytes16(lds, (i >> 2) * 210 + 128 + (i & 3) * 16);
+    for (int i = threadIdx.x; i < nblk; i += 256) {
+        sc[b0 + i] = lds_bytes16(lds, i * 210 + 192);
+        d[b0 + i] = lds[i * 105 + 104];
+    }
+}
+
 static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nbytes, size_t K, size_t N,
                         Weight* out) {
     const size_t be = type == kQ6_K ? 256 : 32;
@@ -122,6 +163,7 @@ static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nby
     const size_t nblk = K / be, total = nblk * N;
     if (nbytes != total * bb)
         return fail(c, SMX_ERR_ARG, "upload: got %zu bytes, [%zu x %zu] needs %zu", nbytes, N, K, total * bb);
+    if (c->capturing) return fail(c, SMX_ERR_ARG, "upload: not during graph capture");
     Weight w;
     w.type = type;
     w.K = K;
@@ -141,41 +183,44 @@ static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nby
         off_scales = off_sc + align256(total * 16);
         w.bytes = off_scales + total * 2;
     }
-    std::unique_ptr<uint8_t[]> host(new (std::nothrow) uint8_t[w.bytes]);
-    if (!host) return fail(c, SMX_ERR_NOMEM, "upload: host staging of %zu bytes failed", w.bytes);
-    uint8_t* h = host.get();
-    if (type == kQ4_0 || type == kQ8_0) {
-        const size_t qb = bb - 2;
-        for (size_t b = 0; b < total; b++) {
-            const uint8_t* blk = bytes + b * bb;
-            h[off_scales + b * 2] = blk[0];
-            h[off_scales + b * 2 + 1] = blk[1];
-            memcpy(h + off_quants + b * qb, blk + 2, qb);
-        }
-        if (off_quants > total * 2) memset(h + total * 2, 0, off_quants - total * 2);
-    } else {
-        memset(h, 0, w.bytes);
-        for (size_t b = 0; b < total; b++) {
-            const uint8_t* blk = bytes + b * 210;
-            memcpy(h + off_quants + b * 128, blk, 128);
-            memcpy(h + off_qh + b * 64, blk + 128, 64);
-            memcpy(h + off_sc + b * 16, blk + 192, 16);
-            h[off_scales + b * 2] = blk[208];
-            h[off_scales + b * 2 + 1] = blk[209];
-        }
-    }
-    hipError_t e = hipMalloc((void**)&w.base, w.bytes);
+    // the raw blocks, padded to whole 16-byte pieces, next to the planes they are split into
+    char* raw = nullptr;
+    const size_t raw_bytes = (nbytes + 15) & ~size_t(15);
+    hipError_t e = hipMalloc((void**)&raw, raw_bytes);
+    if (e == hipSuccess) e = hipMalloc((void**)&w.base, w.bytes);
     if (e != hipSuccess) {
         (void)hipGetLastError();
-        return fail(c, SMX_ERR_NOMEM, "upload: device allocation of %zu bytes failed: %s", w.bytes,
+        if (raw) (void)hipFree(raw);
+        return fail(c, SMX_ERR_NOMEM, "upload: device allocation of %zu + %zu bytes failed: %s", w.bytes, raw_bytes,
                     hipGetErrorString(e));
     }
-    e = hipMemcpy(w.base, h, w.bytes, hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
+    auto bail = [&](hipError_t err, const char* what) {
+        (void)hipStreamSynchronize(c->stream);
+        (void)hipFree(raw);
         (void)hipFree(w.base);
-        return hip_fail(c, e, "hipMemcpy(weight)");
+        return hip_fail(c, err, what);
+    };
+    if ((e = hipMemcpyAsync(raw, bytes, nbytes, hipMemcpyHostToDevice, c->stream)) != hipSuccess) return bail(e, "hipMemcpy(weight)");
+    // the alignment gaps between the planes read as zero
+    if ((e = hipMemsetAsync(w.base, 0, w.bytes, c->stream)) != hipSuccess) return bail(e, "hipMemset(weight)");
+    uint16_t* scales = (uint16_t*)(w.base + off_scales);
+    if (type == kQ6_K) {
+        const unsigned grid = (unsigned)((total + kRepackBlocks / 2 - 1) / (kRepackBlocks / 2));
+        hipLaunchKernelGGL(repack_q6k_kernel, dim3(grid), dim3(256), 0, c->stream, (const uint4*)raw, total, (uint4*)(w.base + off_quants),
+                           (uint4*)(w.base + off_qh), (uint4*)(w.base + off_sc), scales);
+    } else {
+        const unsigned grid = (unsigned)((total + kRepackBlocks - 1) / kRepackBlocks);
+        if (type == kQ4_0)
+            hipLaunchKernelGGL(repack_q4q8_kernel<18>, dim3(grid), dim3(256), 0, c->stream, (const uint4*)raw, total, scales,
+                               (uint4*)(w.base + off_quants));
+        else
+            hipLaunchKernelGGL(repack_q4q8_kernel<34>, dim3(grid), dim3(256), 0, c->stream, (const uint4*)raw, total, scales,
+                               (uint4*)(w.base + off_quants));
     }
-    w.scales = (const uint16_t*)(w.base + off_scales);
+    if ((e = hipGetLastError()) != hipSuccess) return bail(e, "repack launch");
+    if ((e = hipStreamSynchronize(c->stream)) != hipSuccess) return bail(e, "repack");
+    (void)hipFree(raw);
+    w.scales = scales;
     w.quants = w.base + off_quants;
     w.qh = type == kQ6_K ? w.base + off_qh : nullptr;
     w.sc = type == kQ6_K ? (const int8_t*)(w.base + off_sc) : nullptr;
