@@ -201,8 +201,15 @@ static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nby
         return hip_fail(c, err, what);
     };
     if ((e = hipMemcpyAsync(raw, bytes, nbytes, hipMemcpyHostToDevice, c->stream)) != hipSuccess) return bail(e, "hipMemcpy(weight)");
-    // the alignment gaps between the planes read as zero
-    if ((e = hipMemsetAsync(w.base, 0, w.bytes, c->stream)) != hipSuccess) return bail(e, "hipMemset(weight)");
+    // the alignment gaps behind the planes (up to 255 bytes each) read as zero
+    {
+        const size_t ends[3][2] = {{type == kQ6_K ? total * 128 : total * 2, type == kQ6_K ? off_qh : off_quants},
+                                   {off_qh + total * 64, off_sc}, {off_sc + total * 16, off_scales}};
+        for (int i = 0; i < (type == kQ6_K ? 3 : 1); i++)
+            if (ends[i][1] > ends[i][0] &&
+                (e = hipMemsetAsync(w.base + ends[i][0], 0, ends[i][1] - ends[i][0], c->stream)) != hipSuccess)
+                return bail(e, "hipMemset(weight)");
+    }
     uint16_t* scales = (uint16_t*)(w.base + off_scales);
     if (type == kQ6_K) {
         const unsigned grid = (unsigned)((total + kRepackBlocks / 2 - 1) / (kRepackBlocks / 2));
