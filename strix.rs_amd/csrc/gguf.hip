@@ -12,9 +12,11 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <thread>
 
 #include "smx_internal.h"
 
@@ -423,17 +425,41 @@ int smx_gguf_upload_as(smx_ctx* c, const smx_gguf* g, const char* tensor, const 
         return target_type == 2 ? smx_upload_q4_0(c, name, src, t.nbytes, in_dim, out_dim)
                                 : smx_upload_q8_0(c, name, src, t.nbytes, in_dim, out_dim);
     const size_t row_src = in_dim / f->elems * f->bytes, row_dst = in_dim / 32 * (target_type == 2 ? 18 : 34);
-    const size_t slab = std::max<size_t>(1, (size_t(8) << 20) / in_dim);  // rows per slab: 32 MB of floats
-    std::vector<float> tmp(std::min(slab, out_dim) * in_dim);
+    // slabs of rows (1 MB of floats each) shared out over the host's cores; every worker has its own fp32 slab
+    const size_t slab = std::max<size_t>(1, (size_t(1) << 18) / in_dim);
+    const size_t nslabs = (out_dim + slab - 1) / slab;
     std::vector<uint8_t> enc(out_dim * row_dst);
-    for (size_t r0 = 0; r0 < out_dim; r0 += slab) {
-        const size_t rows = std::min(slab, out_dim - r0);
-        int rc = smx_host_dequantize((int)t.type, src + r0 * row_src, rows * in_dim, tmp.data());
-        if (rc != SMX_OK) return smx::fail(c, rc, "gguf_upload_as: encoding %u of %s has no dequantiser", t.type, tensor);
-        rc = target_type == 2 ? smx_host_quantize_q4_0(tmp.data(), rows * in_dim, enc.data() + r0 * row_dst)
-                              : smx_host_quantize_q8_0(tmp.data(), rows * in_dim, enc.data() + r0 * row_dst);
-        if (rc != SMX_OK) return smx::fail(c, rc, "gguf_upload_as: quantiser failed on %s", tensor);
+    std::atomic<size_t> next{0};
+    std::atomic<int> err_deq{SMX_OK}, err_q{SMX_OK};
+    auto work = [&]() {
+        std::vector<float> tmp(std::min(slab, out_dim) * in_dim);
+        for (size_t i; (i = next.fetch_add(1)) < nslabs;) {
+            const size_t r0 = i * slab, rows = std::min(slab, out_dim - r0);
+            int rc = smx_host_dequantize((int)t.type, src + r0 * row_src, rows * in_dim, tmp.data());
+            if (rc != SMX_OK) { err_deq = rc; return; }
+            rc = target_type == 2 ? smx_host_quantize_q4_0(tmp.data(), rows * in_dim, enc.data() + r0 * row_dst)
+                                  : smx_host_quantize_q8_0(tmp.data(), rows * in_dim, enc.data() + r0 * row_dst);
+            if (rc != SMX_OK) { err_q = rc; return; }
+        }
+    };
+    {
+        const size_t hw = std::max(1u, std::thread::hardware_concurrency());
+        const size_t nthreads = std::min<size_t>({hw, 16, nslabs});
+        auto safe_work = [&]() {   // nothing may leave a worker thread
+            try { work(); } catch (...) { err_q = SMX_ERR_NOMEM; }
+        };
+        std::vector<std::thread> pool;
+        try {
+            pool.reserve(nthreads);
+            for (size_t i = 1; i < nthreads; i++) pool.emplace_back(safe_work);
+        } catch (...) {
+            // fewer workers than asked for: the ones that started and this thread finish the slabs
+        }
+        safe_work();
+        for (auto& th : pool) th.join();
     }
+    if (err_deq != SMX_OK) return smx::fail(c, err_deq, "gguf_upload_as: encoding %u of %s has no dequantiser", t.type, tensor);
+    if (err_q != SMX_OK) return smx::fail(c, err_q, "gguf_upload_as: quantiser failed on %s", tensor);
     return target_type == 2 ? smx_upload_q4_0(c, name, enc.data(), enc.size(), in_dim, out_dim)
                             : smx_upload_q8_0(c, name, enc.data(), enc.size(), in_dim, out_dim);
     });
