@@ -553,6 +553,9 @@ int smx_tune(smx_ctx* c, const char* knob, int value) {
     } else if (k == "gemm_splitk") {
         if (value > 16) return fail(c, SMX_ERR_ARG, "tune: gemm_splitk must be 0..16");
         c->tune_gemm_splitk = value;
+    } else if (k == "gemm_tile_m") {
+        if (value != 0 && value != 64 && value != 128) return fail(c, SMX_ERR_ARG, "tune: gemm_tile_m must be 0, 64 or 128");
+        c->tune_gemm_tile_m = value;
     } else {
         return fail(c, SMX_ERR_ARG, "tune: unknown knob %s", knob);
     }

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         const int T = p.tiles_m * p.tiles_n;
         if (p.xcd_remap) t = (t & 7) * (T >> 3) + (t >> 3);
         const int tm = t % p.tiles_m, tn = t / p.tiles_m;
-        tok0 = tm * BM; row0 = tn * BN; col0 = row0; M_end = p.M; N_end = p.N;
+        tok0 = tm * p.tile_m; row0 = tn * BN; col0 = row0; M_end = min(p.M, tok0 + p.tile_m); N_end = p.N;
     }
     const GemmOperand op = p.op[op_i];
     // Wave roles.  A full tile gives each wave 32 tokens x 128 rows (4 row tiles).  A tile with few live
@@ -479,13 +479,19 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     // (-7 %); three workgroups per CU with 2-block stages, every operand and scale staged LDS-direct and the
     // LDS reads software-pipelined (-5..-10 %: the third wave per SIMD raises the instruction issue rate,
     // and the clock the chip sustains drops by as much).
-    const int bm = 128;
-    p.tiles_m = (p.M + bm - 1) / bm;
+    const int slots = c->num_cu * 2;
     p.tiles_n = (p.N + BN - 1) / BN;
+    // Tokens per tile.  65..128 tokens make one row of 128-token tiles in which half the waves of a workgroup may idle and
+    // the K slices are long; as two rows of 64-token tiles (the waves pair up on two row tiles each) the launch has twice
+    // the workgroups at half the work each: Q8_0 2560 x 9728 and 9728 x 2560 at 96 / 128 tokens 28.2 / 29.4 -> 25.4 /
+    // 26.7 us and 25.9 / 27.3 -> 22.9 / 24.7 us, 15360 x 3840 -2..4 %, the long-K shapes and Q6_K unchanged within 2 %.
+    // From 129 tokens on the gain is erratic (-10 .. +20 % with the shape and the split-K factor it meets): 128-token tiles.
+    const int bm = (c->tune_gemm_tile_m == 64 || (c->tune_gemm_tile_m == 0 && p.M > 64 && p.M <= 128 && w.type != kQ6_K)) ? 64 : 128;
+    p.tile_m = bm;
+    p.tiles_m = (p.M + bm - 1) / bm;
     const int T = p.tiles_m * p.tiles_n;
     p.xcd_remap = (T % 8 == 0) ? 1 : 0;
     const int nstages = (p.nb + KB - 1) / KB;
-    const int slots = c->num_cu * 2;
     int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(slots, T, nstages));
     p.stages_per_slice = (nstages + Z - 1) / Z;
     Z = (nstages + p.stages_per_slice - 1) / p.stages_per_slice;

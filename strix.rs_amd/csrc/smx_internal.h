@@ -78,7 +78,7 @@ struct smx_ctx {
     hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
 
     // tuning overrides (0 = automatic)
-    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0;
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_tile_m = 0;
 
     // dynamic-LDS limit already raised on this context's device, per kernel (see set_dyn_lds): a fixed
     // open-addressing table, so that a launch never allocates host memory
@@ -190,6 +190,7 @@ struct GemmArgs {
     int* dump;              // optional [M][N][nb] (Q6_K: [M][N][2 * nb], one per 16-element sub-block)
     int M, N, nb, ldo;
     int tiles_m, tiles_n;
+    int tile_m;             // dense tiling: tokens per tile, 128 or 64 (a 64-token tile's waves pair up on two row tiles each)
     int stages_per_slice;   // stages (of 4 blocks) each grid.z slice covers
     int xcd_remap;
     int nops;               // grouped launches: operands per tile (workgroup x serves tile x / nops, operand x % nops)

@@ -55,6 +55,31 @@ def test_gemm_row_equals_gemv(accel, synth, relerr, ty):
         assert relerr(y[t], accel.gemv("t.rg", xs[t], N)) <= TOL
 
 
+@pytest.mark.parametrize("ty,M,N,K", [(8, 96, 2560, 2560), (2, 128, 300, 1280), (8, 65, 130, 288), (8, 100, 257, 96), (14, 70, 130, 512)])
+def test_gemm_64_token_tiles(accel, orc, synth, relerr, ty, M, N, K):
+    """65..128 tokens of a Q8_0 / Q4_0 weight run as two rows of 64-token tiles; the knob forces either tiling on any
+    shape.  Same integers, same fp32 association per output: the two tilings agree bit for bit."""
+    raw = synth.make_weight(ty, N, K, seed=M + N)
+    assert getattr(accel, UPLOAD[ty])("t.t64", raw, K, N)
+    xs = synth.make_acts(M + 150, K, seed=M)
+    ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
+    for m in (M, M + 150):      # the second size has three or four 64-token rows, the last one ragged
+        ys = {}
+        for tile in (0, 64, 128):
+            accel.tune("gemm_tile_m", tile)
+            ys[tile] = accel.prefill_q8_gemm("t.t64", xs[:m], m, N)
+            assert relerr(ys[tile], ref[:m]) <= TOL, (m, tile)
+        accel.tune("gemm_tile_m", 64)
+        xq, _, _ = orc.actquant(xs[:m], K)
+        dots = accel.gemm_block_dots("t.t64", xs[:m], m, N, K // (16 if ty == 14 else 32))
+        for t in (0, 63, 64, m - 1):
+            assert np.array_equal(dots[t], orc.block_dots(ty, raw, K, N, xq[t])), (m, t)
+        accel.tune("gemm_tile_m", 0)
+        if K <= 1280:   # at most 10 stages: never split over K, identical association
+            assert np.array_equal(ys[64], ys[128]) and np.array_equal(ys[0], ys[64])
+    accel.evict("t.t64")
+
+
 def test_gemm_declines_and_errors(accel, synth, pkg):
     assert accel.prefill_q8_gemm("t.absent", np.zeros((2, 64), np.float32), 2, 8) is None
     raw = synth.make_weight(8, 8, 256, seed=1)
