@@ -190,10 +190,14 @@ class Bench:
         nsrc = min(ncopies, 3)
         src = [sy.make_weight(ty, N, K, seed=1000 + i) for i in range(nsrc)]
         keys = []
+        acc.sync()
+        t_up = time.perf_counter()
         for i in range(ncopies):
             key = f"{name}.w{i}"
-            assert getattr(acc, UPLOAD[ty])(key, src[i % nsrc], K, N)
+            assert getattr(acc, UPLOAD[ty])(key, src[i % nsrc], K, N)   # raw GGUF blocks from pageable memory, repacked on the device
             keys.append(key)
+        acc.sync()
+        upload_gbps = ncopies * src[0].nbytes / (time.perf_counter() - t_up) / 1e9
         del src
         x = sy.make_acts(m, K, seed=7)
         xd = acc.dev_alloc(x.nbytes)
@@ -230,6 +234,7 @@ class Bench:
             "kernel_GBps": kgbs, "kernel_frac_hbm_peak": kgbs / HBM_PEAK_GBS,
             "kernel_timing": ("events around the timed region's back-to-back launches / launches" if single
                               else "event pair around each launch"),
+            "upload_GBps": upload_gbps,   # set-up: host call to synchronised device, raw block bytes per second
         }
 
     # ------------------------------------------------------------------ grouped GEMV (one launch, G weights)
