@@ -811,30 +811,39 @@ struct FlatXRows {
     }
 };
 
-// The same for up to MT fp32 rows that are quantised here (FQ = 1 with MT > 1): thread i takes half block i % hb of row
-// i / hb, hb = half blocks per row; MT * hb <= 1024 (the launcher's bound: 4 rows of up to 4096 elements).  Saves the
-// quantiser launch in front of a 2..4-row GEMV (2.5 of the 7.6 us Q4_0 9728 x 2560 takes at 2 rows).
+// The same for up to MT fp32 rows that are quantised here (FQ = 1 with MT > 1): item i = half block i % hb of row i / hb,
+// hb = half blocks per row; a thread takes items threadIdx.x and threadIdx.x + 1024, MT * hb <= 2048 (the launcher's
+// bound: 32768 values in all, e.g. 4 rows of up to 8192 elements).  Saves the quantiser launch in front of a 2..4-row
+// GEMV (2.5 of the 7.6 us Q4_0 9728 x 2560 takes at 2 rows).
 template <class Ops, int MT>
 struct FlatXRowsF {
-    static_assert(MT <= 4, "row = number of row boundaries at or below the thread index");
-    float4 v[4];
-    int t, h;
+    static_assert(MT <= 4, "row = number of row boundaries at or below the item index");
+    float4 v[2][4];
+    int t[2], h[2];
 
     __device__ __forceinline__ void request(const GemvX& X, int nblk, int m) {
-        const int hb = Ops::nb32(nblk) * 2, i = threadIdx.x;
-        t = (i >= hb ? 1 : 0) + (i >= 2 * hb ? 1 : 0) + (i >= 3 * hb ? 1 : 0);
-        h = i - t * hb;
+        const int hb = Ops::nb32(nblk) * 2;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (t < m && i < MT * hb) v[j] = ((const float4*)(X.x + (size_t)t * hb * 16))[h * 4 + j];
+        for (int p = 0; p < 2; p++) {
+            const int i = threadIdx.x + p * 1024;
+            t[p] = (i >= hb ? 1 : 0) + (i >= 2 * hb ? 1 : 0) + (i >= 3 * hb ? 1 : 0);
+            h[p] = i - t[p] * hb;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                v[p][j] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (t[p] < m && i < MT * hb) v[p][j] = ((const float4*)(X.x + (size_t)t[p] * hb * 16))[h[p] * 4 + j];
+            }
         }
     }
     // rows past m are staged as zeros (their results are not written)
     __device__ __forceinline__ void store(char* smem, int tokb, int nblk) {
-        const int hb = Ops::nb32(nblk) * 2, i = threadIdx.x;
-        if ((i & ~63) >= MT * hb) return;   // whole waves
-        quantize_half_block<Ops>(smem + min(t, MT - 1) * tokb, nblk, h, i < MT * hb, v);
+        const int hb = Ops::nb32(nblk) * 2;
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            const int i = threadIdx.x + p * 1024;
+            if ((i & ~63) >= MT * hb) return;   // whole waves
+            quantize_half_block<Ops>(smem + min(t[p], MT - 1) * tokb, nblk, h[p], i < MT * hb, v[p]);
+        }
     }
 };
 
