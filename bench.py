@@ -289,8 +289,9 @@ class Bench:
 
     # ------------------------------------------------------------------ dense FFN decode step (2 calls, 3 launches)
     def ffn_block(self, name, ty, H, F, min_total_bytes, steps=None, warmup=None):
-        """One token through a dense FFN: launch 1 = rmsnorm + quantiser + gate and up GEMVs, launch 2 =
-        SwiGLU + quantiser + down GEMV; rotating through >= 1 GB of (gate, up, down) sets."""
+        """One token through a dense FFN in two launches: rmsnorm + quantiser + gate and up GEMVs with the SwiGLU
+        product in the kernel's tail (smx_ffn_gate_up_dev), then quantiser + down GEMV on it; rotating through >= 1 GB
+        of (gate, up, down) sets.  `three_launch_ms_per_step`: the same step as gate/up pair, SwiGLU quantiser, down."""
         acc, sy = self.acc, self.synth
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
         a1, w1 = gemv_bytes(ty, F, H, 1)
@@ -307,12 +308,18 @@ class Bench:
         acc.h2d(xd, x)
         acc.h2d(wd, np.ones(H, np.float32))
 
-        def step(i):
+        def step3(i):
             j = i % nsets
             acc.gemv_fused_dev([f"{name}.g{j}", f"{name}.u{j}"], 1, xd, wd, [gd, ud], 1e-6)
             acc.gemv_fused_dev([f"{name}.d{j}"], 2, gd, ud, [yd])
 
+        def step(i):
+            j = i % nsets
+            acc.ffn_gate_up_dev(f"{name}.g{j}", f"{name}.u{j}", 2, xd, gd, norm=True, norm_w_dev=wd, eps=1e-6)
+            acc.gemv_dev(f"{name}.d{j}", gd, 1, yd)
+
         self._first_touch(step, nsets)
+        ms3, _ = self._timed(step3, steps, warmup)
         ms, wall_ms = self._timed(step, steps, warmup)
         for i in range(nsets):
             for t in "gud":
@@ -321,9 +328,9 @@ class Bench:
             acc.dev_free(p)
         algo = 2 * a1 + a2
         gbs = algo * steps / (ms * 1e-3) / 1e9
-        return {"workload": name, "shape": {"hidden": H, "ffn": F, "M": 1, "calls_per_step": 2, "launches_per_step": 3}, "weight_sets": nsets,
+        return {"workload": name, "shape": {"hidden": H, "ffn": F, "M": 1, "calls_per_step": 2, "launches_per_step": 2}, "weight_sets": nsets,
                 "algorithmic_bytes": algo, "steps": steps, "ms_per_step": ms / steps, "GBps": gbs,
-                "frac_hbm_peak": gbs / HBM_PEAK_GBS}
+                "frac_hbm_peak": gbs / HBM_PEAK_GBS, "three_launch_ms_per_step": ms3 / steps}
 
     # ------------------------------------------------------------------ dense FFN prefill block (3 GEMMs)
     def ffn_prefill_block(self, name, ty, H, F, M, steps=None, warmup=None):
@@ -410,7 +417,7 @@ class Bench:
     # ------------------------------------------------------------------ decode chain as one graph
     def decode_chain_graph(self, name, layers=4, hidden=2048, ffn=8192, ne=64, eff=768, k=8, steps=None, warmup=None):
         """`layers` decoder FFN halves captured once as ONE HIP graph and replayed per token, everything resident and
-        routed on the device: per layer rmsnorm + gate/up GEMVs (one launch), SwiGLU + down GEMV, router logits GEMV,
+        routed on the device: per layer rmsnorm + gate/up GEMVs + SwiGLU product (one launch), down GEMV, router logits GEMV,
         top-k router, the k routed experts' FFN (gate/up, down).  Attention is outside this path.  Q4_0 dense
         weights, Q8_0 experts and router."""
         acc, sy = self.acc, self.synth
@@ -432,8 +439,8 @@ class Bench:
         def chain():
             cur = xd
             for l in range(layers):
-                acc.gemv_fused_dev([f"{name}.g{l}", f"{name}.u{l}"], 1, cur, nw, [gd, ud], 1e-6)
-                acc.gemv_fused_dev([f"{name}.d{l}"], 2, gd, ud, [hd])
+                acc.ffn_gate_up_dev(f"{name}.g{l}", f"{name}.u{l}", 2, cur, gd, norm=True, norm_w_dev=nw, eps=1e-6)
+                acc.gemv_dev(f"{name}.d{l}", gd, 1, hd)
                 acc.gemv_dev(f"{name}.r{l}", hd, 1, ld)
                 acc.moe_route_dev(ld, ne, k, idd, wd)
                 acc.moe_ffn_routed_dev(base + l, idd, wd, k, hd, yd)
@@ -454,7 +461,7 @@ class Bench:
             acc.dev_free(p)
         wbytes = layers * (3 * gemv_bytes(Q4_0, ffn, hidden)[1] + gemv_bytes(Q8_0, ne, hidden)[1] + k * 3 * eff * (hidden // 32) * 34)
         return {"workload": name, "shape": {"layers": layers, "hidden": hidden, "ffn": ffn, "experts": ne, "eff": eff, "top_k": k,
-                                            "launches_per_token": layers * 7},
+                                            "launches_per_token": layers * 6},
                 "weight_bytes_per_token": wbytes, "steps": steps, "graph_us_per_token": graph_ms / steps * 1e3,
                 "eager_us_per_token": eager_ms / steps * 1e3, "GBps": wbytes * steps / (graph_ms * 1e-3) / 1e9,
                 "frac_hbm_peak": wbytes * steps / (graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,

@@ -190,6 +190,16 @@ int smx_gemv_fused_dev(smx_ctx* ctx, size_t n, const char* const* keys, int act,
                        const float* b_dev, float eps, float* const* ys_dev);
 int smx_gemv_fused(smx_ctx* ctx, const char* key, int act, const float* a, const float* b, size_t in_len,
                    float eps, float* y, size_t out_cap);
+
+/* The gate and up projections of a dense FFN decode step in ONE launch with the SwiGLU / GeGLU product in the kernel's
+ * tail: h[i] = act(gate_i . x') * (up_i . x') with x' = x or (norm = 1) rmsnorm(x, eps) * norm_w (norm_w may be NULL);
+ * act = SMX_ACT_SILU_MUL or SMX_ACT_GEGLU.  The reference runs q4_gemv_dp2 (kernels.rs:324-339) and then silu_xquant /
+ * geglu_xquant (:151-226) over the two outputs; here a workgroup walks the same rows of both weights and holds both dots
+ * of a row, so h leaves the first launch and the down projection (smx_gemv_dev on h) quantises it in its own staging:
+ * two launches per FFN instead of three.  Each dot is formed exactly as smx_gemv_fused_dev forms it (same bits).
+ * gate and up: same format and shape.  SMX_NOT_RESIDENT when either key is unknown. */
+int smx_ffn_gate_up_dev(smx_ctx* ctx, const char* gate_key, const char* up_key, int act, const float* x_dev, int norm,
+                        const float* norm_w_dev, float eps, float* h_dev);
 /* The prefill form (kernels.rs:1174-1187 silu_quant_rows, :1000-1013 xquant8_rows behind a norm): m rows
  * a_dev[m][in_dim] go through the producer inside the quantiser launch that feeds the int8 GEMM, so the
  * normalised / gated fp32 rows are never written.  b_dev: the norm weight [in_dim] (or NULL) for RMSNORM,

@@ -31,7 +31,7 @@ EXPORTS = [
     "smx_prof_enable", "smx_prof_reset", "smx_prof_read", "smx_prof_names", "smx_timer_begin",
     "smx_timer_end", "smx_quantize", "smx_gemv_block_dots", "smx_gemm_block_dots",
     "smx_moe_ffn_stages", "smx_tune", "smx_graph_begin", "smx_graph_end", "smx_graph_launch",
-    "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused",
+    "smx_graph_destroy", "smx_dev_copy", "smx_gemv_batch_dev", "smx_gemv_fused_dev", "smx_gemv_fused", "smx_ffn_gate_up_dev",
     "smx_upload_moe_q6", "smx_gguf_open", "smx_gguf_close", "smx_gguf_tensor_count", "smx_gguf_tensor",
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
@@ -100,6 +100,7 @@ def load_library():
     L.smx_gemv_noalloc_dev.argtypes = [vp, cp, vp, sz, vp]
     L.smx_gemv_batch_dev.argtypes = [vp, sz, vp, vp, vp]
     L.smx_gemv_fused_dev.argtypes = [vp, sz, vp, i, vp, vp, C.c_float, vp]
+    L.smx_ffn_gate_up_dev.argtypes = [vp, C.c_char_p, C.c_char_p, i, vp, i, vp, C.c_float, vp]
     L.smx_gemv_fused.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp, sz]
     L.smx_moe_ffn_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_moe_shexp_dev.argtypes = [vp, sz, C.c_float, vp, vp]
@@ -524,6 +525,11 @@ class Mi355WeightAccel:
         k = (C.c_char_p * n)(*[s.encode() for s in keys])
         yp = (C.c_void_p * n)(*ys_dev)
         return self._check(self._L.smx_gemv_fused_dev(self._h, n, k, int(act), a_dev, b_dev, float(eps), yp))
+
+    def ffn_gate_up_dev(self, gate_key, up_key, act, x_dev, h_dev, norm=False, norm_w_dev=None, eps=0.0):
+        """h = act(gate . x') * (up . x') in one launch, x' = x or rmsnorm(x) * norm_w (see smx_ffn_gate_up_dev)."""
+        return self._check(self._L.smx_ffn_gate_up_dev(self._h, gate_key.encode(), up_key.encode(), int(act), x_dev,
+                                                       1 if norm else 0, norm_w_dev, float(eps), h_dev))
 
     def gemm_fused_dev(self, key, act, a_dev, b_dev, m, y_dev, eps=0.0):
         """Prefill rows through a producer + quantiser + int8 GEMM (see smx_gemm_fused_dev)."""

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstring>
 
+#include "detmath.h"
 #include "smx_internal.h"
 
 using namespace smx;
@@ -334,6 +335,48 @@ int smx_gemv_fused_dev(smx_ctx* c, size_t n, const char* const* keys, int act, c
     }
     const ActProd prod = {act, b_dev, eps};
     return launch_gemv_group(c, ws, xs, ys_dev, (int)n, nullptr, &prod);
+}
+
+// h[i] = act(g[i]) * u[i], the arithmetic of the paired GEMV's tail (for shapes the paired launch does not serve)
+__global__ __launch_bounds__(256) void act_mul_kernel(const float* __restrict__ g, const float* __restrict__ u, float* __restrict__ h,
+                                                      int n, int act) {
+#pragma clang fp contract(off)
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) h[i] = (act == SMX_ACT_GEGLU ? det_gelu_tanh(g[i]) : det_silu(g[i])) * u[i];
+}
+
+int smx_ffn_gate_up_dev(smx_ctx* c, const char* gate_key, const char* up_key, int act, const float* x_dev, int norm,
+                        const float* norm_w_dev, float eps, float* h_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!gate_key || !up_key || !x_dev || !h_dev) return fail(c, SMX_ERR_ARG, "ffn_gate_up_dev: null argument");
+    if (act != SMX_ACT_SILU_MUL && act != SMX_ACT_GEGLU)
+        return fail(c, SMX_ERR_ARG, "ffn_gate_up_dev: activation %d (SMX_ACT_SILU_MUL or SMX_ACT_GEGLU)", act);
+    if (norm != 0 && norm != 1) return fail(c, SMX_ERR_ARG, "ffn_gate_up_dev: norm %d (0 or 1)", norm);
+    if (!norm && norm_w_dev) return fail(c, SMX_ERR_ARG, "ffn_gate_up_dev: norm weight without norm");
+    const Weight* wg = find_weight(c, gate_key);
+    const Weight* wu = find_weight(c, up_key);
+    if (!wg || !wu) return SMX_NOT_RESIDENT;
+    if (wg->type != wu->type || wg->K != wu->K || wg->N != wu->N)
+        return fail(c, SMX_ERR_ARG, "ffn_gate_up_dev: gate is %zu x %zu (type %d), up %zu x %zu (type %d)", wg->N, wg->K,
+                    (int)wg->type, wu->N, wu->K, (int)wu->type);
+    const ActProd prod = {norm ? SMX_ACT_RMSNORM : SMX_ACT_NONE, norm_w_dev, eps};
+    const float* xs[2] = {x_dev, x_dev};
+    float* hs[1] = {h_dev};
+    bool served = false;
+    int rc = launch_gemv_dual(c, &wg, &wu, xs, nullptr, nullptr, hs, 1, act, &prod, nullptr, &served);
+    if (rc != SMX_OK || served) return rc;
+    // other shapes: the pair in one launch, then the product
+    if ((rc = ensure(c, c->work2, 2 * wg->N * 4)) != SMX_OK) return rc;
+    float* g = (float*)c->work2.p;
+    float* u = g + wg->N;
+    const Weight* ws[2] = {wg, wu};
+    float* ys[2] = {g, u};
+    if ((rc = launch_gemv_group(c, ws, xs, ys, 2, nullptr, &prod)) != SMX_OK) return rc;
+    ProfScope ps(c, "act_mul");
+    hipLaunchKernelGGL(act_mul_kernel, dim3((unsigned)((wg->N + 255) / 256)), dim3(256), 0, c->stream, (const float*)g, (const float*)u,
+                       h_dev, (int)wg->N, act);
+    SMX_HIP(c, hipGetLastError());
+    return SMX_OK;
 }
 
 int smx_gemv_fused(smx_ctx* c, const char* key, int act, const float* a, const float* b, size_t in_len, float eps,

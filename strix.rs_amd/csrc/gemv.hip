@@ -43,10 +43,13 @@ struct alignas(128) GemvJob {
     int prod;           // SMX_ACT_*
     float eps;
     int m;              // activation rows
+    int act2;           // paired launch: SMX_ACT_SILU_MUL or SMX_ACT_GEGLU applied to this job's dot ...
+    float* h;           // ... times the next job's: h[r] = act2(y[r]) * y_next[r]
     __host__ __device__ GemvX X() const { return GemvX{x, xq, xd, xs, x2, prod, eps}; }
     void set_x(const GemvX& a) { x = a.x; xq = a.xq; xd = a.xd; xs = a.xs; x2 = a.x2; prod = a.prod; eps = a.eps; }
 };
 static_assert(offsetof(GemvJob, xq) == 64, "the first line ends with magic_u");
+static_assert(sizeof(GemvJob) == 128, "two lines per job: 16 jobs and the routing fit the kernel-argument segment");
 struct GemvJobs {
     GemvJob job[SMX_GEMV_GROUP_MAX];
     // expert indirection (MoE decode routed on the device): job j reads expert ids[slot[j]] of a stacked tensor
@@ -84,6 +87,16 @@ __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int* 
     const GemvJob& jb = J.job[blockIdx.y];
     gemv_body_flat<Ops, MT, PRE, GL, FQ, DUMP>(job_weight<Ops, IND>(J, blockIdx.y), jb.X(), jb.y, jb.N, jb.nblk, jb.N, MT == 1 ? 1 : jb.m,
                                                blockIdx.x, jb.n_wgs, jb.magic_u, dump, dump_per_row);
+}
+
+// Paired form: workgroup (x, p) serves jobs 2p (gate) and 2p + 1 (up) over the same rows and writes the product of the
+// activated gate dot and the up dot (gemv_body_flat, DUAL).
+template <class Ops, int PRE, int GL, int FQ>
+__global__ __launch_bounds__(1024) void gemv_flat_dual_kernel(const GemvJobs J) {
+    const GemvJob& jg = J.job[2 * blockIdx.y];
+    const GemvJob& ju = J.job[2 * blockIdx.y + 1];
+    gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(jg.W, jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1, blockIdx.x, jg.n_wgs, jg.magic_u,
+                                                      nullptr, 0, ju.W, ju.y, jg.h, jg.act2);
 }
 
 namespace {
@@ -444,6 +457,70 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
     }
     if (g.lds > 160 * 1024) return fail(c, SMX_ERR_LIMIT, "gemv: activation of %zu needs %zu bytes of LDS", w0.K, g.lds);
     return launch_jobs(c, w0.type, g, J, n, (int)w0.nblk, 1, 1, nullptr, 0, name);
+}
+
+// npairs (gate, up) pairs of one format and shape in one launch: h[p][r] = act2(gate_p[r] . x_p) * (up_p[r] . x_p), the
+// activation optionally behind rmsnorm (prod).  yg / yu (optional, per pair) also receive the two dots.  *served = false
+// (and nothing launched) when the shape does not take the flat form: the caller then runs the projections and the
+// product separately.
+int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* wu, const float* const* xs, float* const* yg,
+                     float* const* yu, float* const* hs, int npairs, int act2, const ActProd* prod, const char* name, bool* served) {
+    *served = false;
+    if (npairs < 1 || 2 * npairs > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "paired gemv of %d pairs", npairs);
+    if (act2 != SMX_ACT_SILU_MUL && act2 != SMX_ACT_GEGLU) return fail(c, SMX_ERR_ARG, "paired gemv: activation %d", act2);
+    if (prod && prod->kind != SMX_ACT_NONE && prod->kind != SMX_ACT_RMSNORM)
+        return fail(c, SMX_ERR_ARG, "paired gemv: the activation row may pass through rmsnorm only");
+    const Weight& w0 = *wg[0];
+    GemvJobs J = {};
+    for (int p = 0; p < npairs; p++) {
+        const Weight *a = wg[p], *b = wu[p];
+        if (a->type != w0.type || b->type != w0.type || a->K != w0.K || b->K != w0.K || a->N != w0.N || b->N != w0.N)
+            return fail(c, SMX_ERR_ARG, "paired gemv mixes formats or shapes");
+        GemvJob& jg = J.job[2 * p];
+        GemvJob& ju = J.job[2 * p + 1];
+        jg.W = {a->scales, (const uint4*)a->quants, (const uint4*)a->qh, (const uint2*)a->sc};
+        ju.W = {b->scales, (const uint4*)b->quants, (const uint4*)b->qh, (const uint2*)b->sc};
+        jg.x = ju.x = xs[p];
+        if (prod && prod->kind == SMX_ACT_RMSNORM) {
+            jg.x2 = prod->b;
+            jg.prod = prod->kind;
+            jg.eps = prod->eps;
+        }
+        jg.y = yg ? yg[p] : nullptr;
+        ju.y = yu ? yu[p] : nullptr;
+        jg.h = hs[p];
+        jg.act2 = act2;
+        jg.N = ju.N = (int)a->N;
+    }
+    if (w0.N > 0x7fffffffu / 4 || w0.K > (size_t(1) << 20))
+        return fail(c, SMX_ERR_LIMIT, "gemv: shape %zu x %zu exceeds the kernel's index range", w0.N, w0.K);
+    Geom g = pick_geom(c, w0.type, w0.N, w0.nblk, 1, false, npairs);
+    if (!g.flat) return SMX_OK;
+    // the group sums of both weights live in LDS side by side
+    const size_t upb = w0.type == kQ6_K ? 4 : (w0.type == kQ8_0 ? 2 : 1);
+    const size_t rows = (w0.N + g.grid - 1) / g.grid;
+    g.lds += rows * w0.nblk * upb / g.flat * 4;
+    if (g.lds > 160 * 1024) return SMX_OK;
+    const bool norm = prod && prod->kind == SMX_ACT_RMSNORM;
+    const unsigned units = (unsigned)(w0.nblk * upb);
+    const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);
+    for (int i = 0; i < 2 * npairs; i++) { J.job[i].nblk = (int)w0.nblk; J.job[i].m = 1; J.job[i].n_wgs = (int)g.grid; J.job[i].magic_u = magic; }
+    ProfScope ps(c, name ? name : "gemv_gate_up_act");
+    auto go = [&](auto kern) -> int {
+        int rc = set_dyn_lds(c, kern, g.lds);
+        if (rc != SMX_OK) return rc;
+        hipLaunchKernelGGL(kern, dim3(g.grid, (unsigned)npairs), dim3(1024), g.lds, c->stream, J);
+        SMX_HIP(c, hipGetLastError());
+        *served = true;
+        return SMX_OK;
+    };
+#define SMX_DUAL(OPS, PRE, GL) \
+    if (g.flat_pre == PRE && g.flat == GL) return norm ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1>);
+    if (w0.type == kQ4_0) { SMX_DUAL(OpsQ4_0, 3, 16) SMX_DUAL(OpsQ4_0, 3, 8) }
+    else if (w0.type == kQ8_0) { SMX_DUAL(OpsQ8_0, 3, 16) SMX_DUAL(OpsQ8_0, 3, 8) }
+    else { SMX_DUAL(OpsQ6_K, 1, 16) SMX_DUAL(OpsQ6_K, 1, 8) SMX_DUAL(OpsQ6_K, 1, 4) }
+#undef SMX_DUAL
+    return SMX_OK;   // no variant for this geometry: not served
 }
 
 }  // namespace smx

@@ -860,12 +860,20 @@ struct FlatXRowsF {
 //
 // DUMP (one activation row): every unit also writes its exact integer block dot(s) to
 // dump[row * dump_per_row + ...], the same integers that enter the fp32 combination.
-template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP = false>
+//
+// DUAL (one activation row): the workgroup walks the same rows of a second weight W1 (the `up` projection next to `gate`)
+// after those of W -- the loads of the two weights form one sequence, whole 64-unit loads each -- and its tail has both
+// dots of a row: y[r] (optional), y1[r] (optional) and hout[r] = act2(y[r]) * y1[r] (SMX_ACT_SILU_MUL / SMX_ACT_GEGLU).
+// A row's sums are formed exactly as without DUAL, so y and y1 have the bits of two separate launches.
+template <class Ops, int MT, int PRE, int GL, int FQ, bool DUMP = false, bool DUAL = false>
 __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, float* __restrict__ y, int ldy, int nblk,
                                                int N, int m, int wg, int n_wgs, unsigned magic_u,
-                                               int* __restrict__ dump = nullptr, int dump_per_row = 0) {
+                                               int* __restrict__ dump = nullptr, int dump_per_row = 0,
+                                               const GemvW W1 = GemvW{}, float* __restrict__ y1 = nullptr,
+                                               float* __restrict__ hout = nullptr, int act2 = 0) {
     static_assert(MT == 1 || FQ == 0 || FQ == 1, "several activation rows: staged from quantised rows or quantised here");
     static_assert(!DUMP || MT == 1, "the block-dot dump covers one activation row");
+    static_assert(!DUAL || (MT == 1 && !DUMP), "the paired form serves one activation row");
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int U = Ops::units_per_row(nblk);
@@ -873,9 +881,10 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     const unsigned rbase = (unsigned)N / (unsigned)n_wgs, rrem = (unsigned)N - rbase * (unsigned)n_wgs;
     const int r0 = wg * (int)rbase + min(wg, (int)rrem), r1 = r0 + (int)rbase + (wg < (int)rrem ? 1 : 0);
     const int nunits = (r1 - r0) * U;          // < 2^16 (launcher)
-    const int nloads = (nunits + 63) >> 6;
+    const int nloads1 = (nunits + 63) >> 6;          // loads per weight
+    const int nloads = DUAL ? 2 * nloads1 : nloads1;
     const int tokb = Ops::tok_bytes(nblk);
-    float* part = (float*)(smem + MT * tokb);  // [nunits / GL][MT]
+    float* part = (float*)(smem + MT * tokb);  // [nunits / GL][MT]; DUAL: the second weight's groups follow the first's
     // a job with fewer rows than the launch has workgroups leaves some without rows: their (unused)
     // loads go to the weight's first unit
     const size_t f_base = nunits > 0 ? (size_t)r0 * U : 0;
@@ -893,8 +902,9 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     auto request = [&]() {
 #pragma unroll
         for (int k = 0; k < PRE; k++) {
-            const int fl = min(l_t * 64 + lane, max(nunits - 1, 0));
-            Ops::load_flat(ring[k], W, f_base + fl);
+            const bool second = DUAL && l_t >= nloads1;   // wave-uniform
+            const int fl = min((second ? l_t - nloads1 : l_t) * 64 + lane, max(nunits - 1, 0));
+            Ops::load_flat(ring[k], second ? W1 : W, f_base + fl);
             l_t += 16;
         }
     };
@@ -902,7 +912,8 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
 #pragma unroll
         for (int k = 0; k < PRE; k++) {
             if (c_t < nloads) {   // wave-uniform
-                const int fl = c_t * 64 + lane;
+                const bool second = DUAL && c_t >= nloads1;
+                const int fl = (second ? c_t - nloads1 : c_t) * 64 + lane;
                 const bool act = fl < nunits;
                 const int flc = act ? fl : nunits - 1;
                 const int rl = (int)__umulhi((unsigned)flc, magic_u);            // flc / U: row within the workgroup
@@ -915,7 +926,7 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const float s = small_group_sum<GL>(acc[t]);
-                    if (act && (lane & (GL - 1)) == GL - 1) part[(fl / GL) * MT + t] = s;
+                    if (act && (lane & (GL - 1)) == GL - 1) part[((second ? nunits / GL : 0) + fl / GL) * MT + t] = s;
                 }
             }
             c_t += 16;
@@ -935,6 +946,26 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
     // A row's G group sums are added by 8 lanes (lane l takes groups l, l + 8, ... in ascending order, then a
     // fixed DPP tree): one thread per row would pay the LDS latency once per group, one after the other.
     const int G = U / GL;
+    if constexpr (DUAL) {
+#pragma clang fp contract(off)
+        const float* part1 = part + nunits / GL;
+        for (int i8 = threadIdx.x; i8 < (r1 - r0) * 8; i8 += 1024) {
+            const int r = i8 >> 3, l = i8 & 7;
+            float s0 = 0.f, s1 = 0.f;
+            for (int j = l; j < G; j += 8) {
+                s0 += part[r * G + j];
+                s1 += part1[r * G + j];
+            }
+            s0 = small_group_sum<8>(s0);
+            s1 = small_group_sum<8>(s1);
+            if (l == 0) {
+                if (y) y[r0 + r] = s0;
+                if (y1) y1[r0 + r] = s1;
+                hout[r0 + r] = (act2 == SMX_ACT_GEGLU ? det_gelu_tanh(s0) : det_silu(s0)) * s1;
+            }
+        }
+        return;
+    }
     for (int i8 = threadIdx.x; i8 < (r1 - r0) * MT * 8; i8 += 1024) {   // 1024: the form's workgroup size
         const int i = i8 >> 3, l = i8 & 7;
         const int r = i / MT, t = i % MT;

@@ -656,17 +656,25 @@ static int shexp_enqueue(smx_ctx* c, size_t layer, size_t hidden, float sgate, c
     float* g = (float*)(c->work2.p + o_g);
     float* u = (float*)(c->work2.p + o_u);
     float* sd = (float*)(c->work2.p + o_d);
-    {
-        const Weight* ws[2] = {w[0], w[1]};
+    {   // gate and up with the SwiGLU product in the kernel's tail (h lands in g) where the shape takes the flat form
         const float* xs[2] = {x_dev, x_dev};
-        float* ys[2] = {g, u};
-        if ((rc = launch_gemv_group(c, ws, xs, ys, 2, "shexp_gate_up")) != SMX_OK) return rc;
-    }
-    {
-        const ActProd prod = {SMX_ACT_SILU_MUL, u, 0.f};
-        const float* xs[1] = {g};
-        float* ys[1] = {sd};
-        if ((rc = launch_gemv_group(c, &w[2], xs, ys, 1, "shexp_down", &prod)) != SMX_OK) return rc;
+        float* hs[1] = {g};
+        bool served = false;
+        if ((rc = launch_gemv_dual(c, &w[0], &w[1], xs, nullptr, nullptr, hs, 1, SMX_ACT_SILU_MUL, nullptr, "shexp_gate_up", &served)) != SMX_OK)
+            return rc;
+        if (served) {
+            const float* hx[1] = {g};
+            float* ys[1] = {sd};
+            if ((rc = launch_gemv_group(c, &w[2], hx, ys, 1, "shexp_down")) != SMX_OK) return rc;
+        } else {
+            const Weight* ws[2] = {w[0], w[1]};
+            float* ys2[2] = {g, u};
+            if ((rc = launch_gemv_group(c, ws, xs, ys2, 2, "shexp_gate_up")) != SMX_OK) return rc;
+            const ActProd prod = {SMX_ACT_SILU_MUL, u, 0.f};
+            const float* gx[1] = {g};
+            float* ys[1] = {sd};
+            if ((rc = launch_gemv_group(c, &w[2], gx, ys, 1, "shexp_down", &prod)) != SMX_OK) return rc;
+        }
     }
     ProfScope ps(c, "shexp_add");
     hipLaunchKernelGGL(shexp_add_kernel, dim3((unsigned)((hidden + 255) / 256)), dim3(256), 0, c->stream, y_dev, sd, sgate,

@@ -108,3 +108,49 @@ def test_prefill_rows_through_a_producer(accel, orc, synth, relerr, ty, act):
     assert accel.gemm_fused_dev("t.absent", act, ad, bd, M, yd, eps) is False
     for p in (ad, bd, yd):
         accel.dev_free(p)
+
+
+@pytest.mark.parametrize("ty,N,K", [(2, 9728, 2560), (8, 300, 1024), (14, 130, 2560), (2, 96, 256), (8, 77, 96), (2, 40, 16384 + 512)])
+@pytest.mark.parametrize("act", [2, 3])
+@pytest.mark.parametrize("norm", [False, True])
+def test_ffn_gate_up_with_the_product_in_the_tail(accel, orc, synth, relerr, ty, N, K, act, norm):
+    """smx_ffn_gate_up_dev: gate and up in one launch, h = act(g) * u from the kernel's tail (shapes of the flat form), or
+    the pair launch followed by the product (rows of 96 and 16896 elements).  Each dot has the bits of
+    smx_gemv_fused_dev, the product those of the oracle's producer on them."""
+    if ty == 14 and K % 256:
+        pytest.skip("Q6_K rows are whole superblocks")
+    rg, ru = synth.make_weight(ty, N, K, seed=N + act), synth.make_weight(ty, N, K, seed=N + act + 7)
+    assert getattr(accel, UP[ty])("t.g", rg, K, N) and getattr(accel, UP[ty])("t.u", ru, K, N)
+    x, w = _inputs(synth, K, seed=70 + act)
+    eps = 1e-6
+    xd, wd = accel.dev_alloc(K * 4), accel.dev_alloc(K * 4)
+    gd, ud, hd = (accel.dev_alloc(N * 4) for _ in range(3))
+    accel.h2d(xd, x); accel.h2d(wd, w)
+    assert accel.ffn_gate_up_dev("t.g", "t.u", act, xd, hd, norm=norm, norm_w_dev=wd if norm else None, eps=eps)
+    h = accel.d2h(np.empty(N, np.float32), hd)
+    # the two dots through the existing pair launch
+    assert accel.gemv_fused_dev(["t.g", "t.u"], 1 if norm else 0, xd, wd if norm else None, [gd, ud], eps if norm else 0.0)
+    g, u = accel.d2h(np.empty(N, np.float32), gd), accel.d2h(np.empty(N, np.float32), ud)
+    assert np.array_equal(h, orc.act_produce(act, g, u, 0.0))
+    # and against the oracle end to end
+    xn = orc.act_produce(1, x, w, eps) if norm else x
+    g_ref = orc.matmul_q8_from_f32(ty, rg, K, N, xn)[0]
+    u_ref = orc.matmul_q8_from_f32(ty, ru, K, N, xn)[0]
+    assert relerr(g, g_ref) <= TOL and relerr(u, u_ref) <= TOL
+    assert relerr(h, orc.act_produce(act, g_ref, u_ref, 0.0)) <= 2e-5    # the product of two 1e-5 quantities
+    for p in (xd, wd, gd, ud, hd):
+        accel.dev_free(p)
+    accel.evict("t.g"); accel.evict("t.u")
+
+
+def test_ffn_gate_up_errors(accel, synth, pkg):
+    raw = synth.make_weight(2, 64, 256, seed=1)
+    assert accel.upload_q4_0("t.g", raw, 256, 64) and accel.upload_q4_0("t.u2", synth.make_weight(2, 32, 256, seed=2), 256, 32)
+    xd, hd = accel.dev_alloc(256 * 4), accel.dev_alloc(64 * 4)
+    assert accel.ffn_gate_up_dev("t.g", "t.absent", 2, xd, hd) is False     # declines: not resident
+    with pytest.raises(pkg.SmxError):   # shapes differ
+        accel.ffn_gate_up_dev("t.g", "t.u2", 2, xd, hd)
+    with pytest.raises(pkg.SmxError):   # not an activation product
+        accel.ffn_gate_up_dev("t.g", "t.g", 1, xd, hd)
+    accel.dev_free(xd); accel.dev_free(hd)
+    accel.evict("t.g"); accel.evict("t.u2")
