@@ -91,12 +91,13 @@ __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int* 
 
 // Paired form: workgroup (x, p) serves jobs 2p (gate) and 2p + 1 (up) over the same rows and writes the product of the
 // activated gate dot and the up dot (gemv_body_flat, DUAL).
-template <class Ops, int PRE, int GL, int FQ>
+template <class Ops, int PRE, int GL, int FQ, bool IND = false>
 __global__ __launch_bounds__(1024) void gemv_flat_dual_kernel(const GemvJobs J) {
     const GemvJob& jg = J.job[2 * blockIdx.y];
     const GemvJob& ju = J.job[2 * blockIdx.y + 1];
-    gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(jg.W, jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1, blockIdx.x, jg.n_wgs, jg.magic_u,
-                                                      nullptr, 0, ju.W, ju.y, jg.h, jg.act2);
+    gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(job_weight<Ops, IND>(J, 2 * blockIdx.y), jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1, blockIdx.x,
+                                                      jg.n_wgs, jg.magic_u, nullptr, 0, job_weight<Ops, IND>(J, 2 * blockIdx.y + 1), ju.y,
+                                                      jg.h, jg.act2);
 }
 
 namespace {
@@ -464,7 +465,8 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
 // (and nothing launched) when the shape does not take the flat form: the caller then runs the projections and the
 // product separately.
 int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* wu, const float* const* xs, float* const* yg,
-                     float* const* yu, float* const* hs, int npairs, int act2, const ActProd* prod, const char* name, bool* served) {
+                     float* const* yu, float* const* hs, int npairs, int act2, const ActProd* prod, const char* name, bool* served,
+                     const GemvIndirect* ind) {
     *served = false;
     if (npairs < 1 || 2 * npairs > SMX_GEMV_GROUP_MAX) return fail(c, SMX_ERR_ARG, "paired gemv of %d pairs", npairs);
     if (act2 != SMX_ACT_SILU_MUL && act2 != SMX_ACT_GEGLU) return fail(c, SMX_ERR_ARG, "paired gemv: activation %d", act2);
@@ -472,6 +474,13 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
         return fail(c, SMX_ERR_ARG, "paired gemv: the activation row may pass through rmsnorm only");
     const Weight& w0 = *wg[0];
     GemvJobs J = {};
+    if (ind) {   // experts chosen on the device: both jobs of a pair read the same routing slot
+        if (prod && prod->kind != SMX_ACT_NONE) return fail(c, SMX_ERR_ARG, "paired gemv: device-routed experts take the plain activation row");
+        J.ids = ind->ids;
+        J.ne = ind->ne;
+        J.blocks_per_expert = ind->blocks_per_expert;
+        for (int p = 0; p < npairs; p++) J.slot[2 * p] = J.slot[2 * p + 1] = ind->slot[p];
+    }
     for (int p = 0; p < npairs; p++) {
         const Weight *a = wg[p], *b = wu[p];
         if (a->type != w0.type || b->type != w0.type || a->K != w0.K || b->K != w0.K || a->N != w0.N || b->N != w0.N)
@@ -514,8 +523,10 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
         *served = true;
         return SMX_OK;
     };
-#define SMX_DUAL(OPS, PRE, GL) \
-    if (g.flat_pre == PRE && g.flat == GL) return norm ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1>);
+#define SMX_DUAL(OPS, PRE, GL)                                                                                  \
+    if (g.flat_pre == PRE && g.flat == GL)                                                                      \
+        return ind ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 1, true>)                                           \
+                   : (norm ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1>));
     if (w0.type == kQ4_0) { SMX_DUAL(OpsQ4_0, 3, 16) SMX_DUAL(OpsQ4_0, 3, 8) }
     else if (w0.type == kQ8_0) { SMX_DUAL(OpsQ8_0, 3, 16) SMX_DUAL(OpsQ8_0, 3, 8) }
     else { SMX_DUAL(OpsQ6_K, 1, 16) SMX_DUAL(OpsQ6_K, 1, 8) SMX_DUAL(OpsQ6_K, 1, 4) }

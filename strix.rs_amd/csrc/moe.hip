@@ -21,6 +21,8 @@ namespace smx {
 
 // a = silu(g)*u for 4 consecutive elements, then the activation quantiser over the 32-block that
 // 8 adjacent lanes hold (kernels.rs:879-892, 1174-1187): packed quants and the block scale.
+// the activation quantiser over the 32-block that 8 adjacent lanes hold, 4 consecutive elements per lane
+__device__ __forceinline__ void quant4(float4 v, int* packed, float* scale);
 __device__ __forceinline__ void silu_mul_quant4(float4 gv, float4 uv, int* packed, float* scale) {
     float4 v;
     {
@@ -30,6 +32,9 @@ __device__ __forceinline__ void silu_mul_quant4(float4 gv, float4 uv, int* packe
         v.z = det_silu(gv.z) * uv.z;
         v.w = det_silu(gv.w) * uv.w;
     }
+    quant4(v, packed, scale);
+}
+__device__ __forceinline__ void quant4(float4 v, int* packed, float* scale) {
     float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     a = fmaxf(a, __shfl_xor(a, 1));
     a = fmaxf(a, __shfl_xor(a, 2));
@@ -280,6 +285,8 @@ __global__ __launch_bounds__(1024) void moe_down_fused_kernel(const float* __res
 // does not wait for the weights (a wave's loads complete in order) and every later wait is exact.
 // Every GL-lane group lies inside one expert's row segment; its weighted sum goes to LDS and the groups
 // of a row are added in ascending order (expert k ascending, blocks ascending).
+// u == nullptr: g holds the finished products silu(g_k) * u_k (the paired gate/up launch wrote them) and only the
+// quantiser runs here.
 template <int GL>
 __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __restrict__ g, const float* __restrict__ u,
                                                             const uint16_t* __restrict__ scales,
@@ -306,7 +313,7 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
         gv[j] = uv[j] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (it < items) {
             gv[j] = ((const float4*)g)[it];
-            uv[j] = ((const float4*)u)[it];
+            if (u) uv[j] = ((const float4*)u)[it];
         }
     }
     if (tid < k) {
@@ -372,7 +379,8 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
         if ((it & ~63) < items) {   // whole waves are live or not together
             int packed;
             float d;
-            silu_mul_quant4(gv[j], uv[j], &packed, &d);
+            if (u) silu_mul_quant4(gv[j], uv[j], &packed, &d);   // (workgroup-uniform)
+            else quant4(gv[j], &packed, &d);
             if (it < items) {
                 sxq[it] = packed;
                 if ((it & 7) == 0) sxd[it >> 3] = d;
@@ -510,7 +518,8 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     int rc;
     Carver cv;
     const size_t o_g = cv.take(k * eff * 4), o_u = cv.take(k * eff * 4), o_aq = cv.take(k * eff),
-                 o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(L.type == kQ6_K ? k * hidden * 4 : 0);
+                 o_ad = cv.take(k * (eff / 32) * 4), o_dy = cv.take(L.type == kQ6_K ? k * hidden * 4 : 0),
+                 o_h = cv.take(k * eff * 4);
     if ((rc = ensure(c, c->work, cv.off)) != SMX_OK) return rc;
     MoeRoute route = {};
     route.ids_dev = ids_dev;
@@ -525,6 +534,7 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
     GemvIndirect ind = {};
     ind.ids = ids_dev;
     ind.ne = (int)L.ne;
+    bool paired = false;   // the gate/up launch left silu(g) * u at o_h
     MoeScratch s;
     s.g = (float*)(c->work.p + o_g);
     s.u = (float*)(c->work.p + o_u);
@@ -544,7 +554,29 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
                 ys[2 * i + z] = (z ? s.u : s.g) + i * eff;
             }
         ind.blocks_per_expert = eff * L.gate.nblk;
-        for (size_t i = 0; i < 2 * k; i += SMX_GEMV_GROUP_MAX) {
+        // Q8_0 experts: gate and up of an expert as one paired job with silu(g) * u in the kernel's tail (g and u are still
+        // written: the stage-by-stage checks read them); the down kernel then only quantises the products
+        if (L.type == kQ8_0) {
+            std::vector<const Weight*> wgp(k), wup(k);
+            std::vector<float*> ygp(k), yup(k), hp(k);
+            for (size_t i = 0; i < k; i++) {
+                wgp[i] = ws[2 * i]; wup[i] = ws[2 * i + 1];
+                ygp[i] = ys[2 * i]; yup[i] = ys[2 * i + 1];
+                hp[i] = (float*)(c->work.p + o_h) + i * eff;
+            }
+            constexpr int kPairs = SMX_GEMV_GROUP_MAX / 2;
+            paired = true;
+            for (size_t i = 0; i < k && paired; i += kPairs) {
+                const int n = (int)std::min<size_t>(kPairs, k - i);
+                for (int j = 0; j < n; j++) ind.slot[j] = (int)(i + j);
+                bool served = false;
+                rc = launch_gemv_dual(c, &wgp[i], &wup[i], &xs[i], &ygp[i], &yup[i], &hp[i], n, SMX_ACT_SILU_MUL, nullptr,
+                                      "moe_gemv_gate_up", &served, routed_on_device ? &ind : nullptr);
+                if (rc != SMX_OK) return rc;
+                if (!served) paired = false;   // (the first chunk decides: every chunk has the same shape)
+            }
+        }
+        for (size_t i = 0; i < 2 * k && !paired; i += SMX_GEMV_GROUP_MAX) {
             const int n = (int)std::min<size_t>(SMX_GEMV_GROUP_MAX, 2 * k - i);
             for (int j = 0; j < n; j++) ind.slot[j] = (int)((i + j) / 2);
             rc = launch_gemv_group(c, &ws[i], &xs[i], &ys[i], n, "moe_gemv_gate_up", nullptr, nullptr,
@@ -601,7 +633,9 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
             auto launch = [&](auto kern) -> int {
                 int rc2 = set_dyn_lds(c, kern, flds);
                 if (rc2 != SMX_OK) return rc2;
-                hipLaunchKernelGGL(kern, dim3((unsigned)fgrid), dim3(1024), flds, c->stream, s.g, s.u, L.down.scales,
+                const float* hsrc = (const float*)(c->work.p + o_h);
+                hipLaunchKernelGGL(kern, dim3((unsigned)fgrid), dim3(1024), flds, c->stream, paired ? hsrc : (const float*)s.g,
+                                   paired ? (const float*)nullptr : (const float*)s.u, L.down.scales,
                                    (const uint4*)L.down.quants, route, (int)k, (int)eff, (int)hidden, y_dev, (int*)s.aq, s.ad,
                                    m_units, m_upe, (int)fgrid);
                 SMX_HIP(c, hipGetLastError());

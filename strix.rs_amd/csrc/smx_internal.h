@@ -248,7 +248,8 @@ int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* x
 // npairs (gate, up) pairs in one launch with the activation product in the kernel's tail: hs[p][r] = act2(gate . x) * (up . x);
 // yg / yu (optional) also receive the dots.  *served = false and nothing launched when the shape does not take the flat form.
 int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* wu, const float* const* xs, float* const* yg,
-                     float* const* yu, float* const* hs, int npairs, int act2, const ActProd* prod, const char* name, bool* served);
+                     float* const* yu, float* const* hs, int npairs, int act2, const ActProd* prod, const char* name, bool* served,
+                     const GemvIndirect* ind = nullptr);
 // GEMM: y[m][N] on int8 MFMA.  dump (optional): out[m][N][K/32] i32.
 int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, size_t m, float* y,
                 int32_t* dump);
