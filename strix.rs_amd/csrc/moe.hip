@@ -410,6 +410,85 @@ __global__ __launch_bounds__(1024) void moe_down_flat_kernel(const float* __rest
     }
 }
 
+// The same for Q6_K experts, in terms of the GEMV's per-format pieces (gemv_body.h): h holds the k * eff products
+// silu(g_k) * u_k (the paired gate/up launch wrote them); every workgroup quantises them into the k experts' activation
+// areas in LDS (a half block per thread), then walks its rows' units -- k experts side by side per row, four 64-element
+// units per superblock -- one load round at a time.  A GL-lane group lies inside one expert's row segment.
+template <int GL>
+__global__ __launch_bounds__(1024) void moe_down_flat_q6_kernel(const float* __restrict__ h, const GemvW D, const MoeRoute route,
+                                                               int k, int eff, int hidden, float* __restrict__ y,
+                                                               unsigned magic_units, unsigned magic_upe, int n_wgs) {
+    extern __shared__ __align__(16) char smem[];
+    const int nsb = eff / 256, upe = nsb * 4, units = k * upe;   // superblocks and units per expert row
+    const int tokb = OpsQ6_K::tok_bytes(nsb);
+    int* sid = (int*)(smem + (size_t)k * tokb);   // [k] expert ids
+    float* sw = (float*)(sid + k);                // [k] routing weights
+    float* part = sw + k;                         // [rows * units / GL]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the products first: a 16-element half per thread (k * eff <= 16384, the launcher's bound)
+    const int hbe = eff / 16, nhb = k * hbe;
+    float4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = tid < nhb ? ((const float4*)h)[tid * 4 + j] : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (tid < k) {
+        sid[tid] = route_id(route, tid);
+        sw[tid] = route_w(route, tid);
+    }
+    __syncthreads();
+    const unsigned rbase = (unsigned)hidden / (unsigned)n_wgs, rrem = (unsigned)hidden - rbase * (unsigned)n_wgs;
+    const int r0 = blockIdx.x * (int)rbase + min((int)blockIdx.x, (int)rrem);
+    const int rows = (int)rbase + ((int)blockIdx.x < (int)rrem ? 1 : 0);
+    const int nv = rows * units;                  // < 2^16 (launcher)
+    const int nloads = (nv + 63) >> 6;
+    auto locate = [&](int vv, int& rl, int& e, int& u) {
+        rl = (int)__umulhi((unsigned)vv, magic_units);
+        const int uidx = vv - rl * units;
+        e = (int)__umulhi((unsigned)uidx, magic_upe);
+        u = uidx - e * upe;
+    };
+    OpsQ6_K::Regs regs;
+    int l_t = wave, c_t = wave;
+    auto request = [&]() {
+        int rl, e, u;
+        locate(min(l_t * 64 + lane, max(nv - 1, 0)), rl, e, u);
+        OpsQ6_K::load_flat(regs, D, ((size_t)sid[e] * hidden + min(r0 + rl, hidden - 1)) * upe + u);
+        l_t += 16;
+    };
+    auto consume = [&]() {
+        if (c_t < nloads) {   // wave-uniform
+            const int vv = c_t * 64 + lane;
+            const bool act = vv < nv;
+            int rl, e, u;
+            locate(act ? vv : nv - 1, rl, e, u);
+            float acc[1] = {0.f};
+            compute_unit<1, false>(OpsQ6_K(), regs, smem + (size_t)e * tokb, tokb, nsb, u, act, acc, nullptr);
+            const float gs = small_group_sum<GL>(act ? sw[e] * acc[0] : 0.f);
+            if (act && (lane & (GL - 1)) == GL - 1) part[vv / GL] = gs;
+        }
+        c_t += 16;
+    };
+    request();
+    if ((tid & ~63) < nhb) {   // whole waves
+        const int e = tid / hbe;
+        quantize_half_block<OpsQ6_K>(smem + (size_t)min(e, k - 1) * tokb, nsb, tid - e * hbe, tid < nhb, v);
+    }
+    __syncthreads();
+    consume();
+    while (c_t < nloads) {
+        request();
+        consume();
+    }
+    __syncthreads();
+    const int G = units / GL;
+    for (int i8 = tid; i8 < rows * 8; i8 += 1024) {
+        const int r = i8 >> 3, l = i8 & 7;
+        float s = 0.f;
+        for (int j = l; j < G; j += 8) s += part[r * G + j];
+        s = small_group_sum<8>(s);
+        if (l == 0) y[r0 + r] = s;
+    }
+}
+
 // y[t][i] = sum over the token's slots (ascending slot index) of wslot[s]*dy[s][i].  Eight slots at a
 // time: their indices, weights and rows are requested together (clamped, not conditional, so the
 // loads of a batch are in flight at once instead of one dependent round trip per slot).
@@ -554,9 +633,9 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
                 ys[2 * i + z] = (z ? s.u : s.g) + i * eff;
             }
         ind.blocks_per_expert = eff * L.gate.nblk;
-        // Q8_0 experts: gate and up of an expert as one paired job with silu(g) * u in the kernel's tail (g and u are still
+        // gate and up of an expert as one paired job with silu(g) * u in the kernel's tail (g and u are still
         // written: the stage-by-stage checks read them); the down kernel then only quantises the products
-        if (L.type == kQ8_0) {
+        {
             std::vector<const Weight*> wgp(k), wup(k);
             std::vector<float*> ygp(k), yup(k), hp(k);
             for (size_t i = 0; i < k; i++) {
@@ -584,7 +663,38 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
             if (rc != SMX_OK) return rc;
         }
     }
-    if (L.type == kQ6_K) {
+    bool q6_flat = false;
+    if (L.type == kQ6_K && paired) {
+        // Q6_K experts, second launch in the flat form: quantiser + the k down projections + the weighted sum
+        const size_t nsb = eff / 256, upe = nsb * 4, units = k * upe;
+        const size_t tokb = nsb * 2 * (OpsQ6_K::kPad * 16 + 32);
+        const size_t fgrid = std::min<size_t>(hidden, (size_t)c->num_cu);
+        const size_t frows = (hidden + fgrid - 1) / fgrid;
+        const int gl = upe % 16 == 0 ? 16 : (upe % 8 == 0 ? 8 : 4);
+        const size_t flds = k * tokb + k * 8 + frows * units / gl * 4;
+        if (k * eff <= 16384 && frows * units < 65536 && flds <= 160 * 1024) {
+            q6_flat = true;
+            ProfScope ps(c, "moe_gemv_down");
+            const GemvW D = {L.down.scales, (const uint4*)L.down.quants, (const uint4*)L.down.qh, (const uint2*)L.down.sc};
+            const unsigned m_units = (unsigned)(((1ull << 32) + units - 1) / units), m_upe = (unsigned)(((1ull << 32) + upe - 1) / upe);
+            auto launch = [&](auto kern) -> int {
+                int rc2 = set_dyn_lds(c, kern, flds);
+                if (rc2 != SMX_OK) return rc2;
+                hipLaunchKernelGGL(kern, dim3((unsigned)fgrid), dim3(1024), flds, c->stream, (const float*)(c->work.p + o_h), D, route,
+                                   (int)k, (int)eff, (int)hidden, y_dev, m_units, m_upe, (int)fgrid);
+                SMX_HIP(c, hipGetLastError());
+                return SMX_OK;
+            };
+            rc = gl == 16 ? launch(moe_down_flat_q6_kernel<16>) : (gl == 8 ? launch(moe_down_flat_q6_kernel<8>) : launch(moe_down_flat_q6_kernel<4>));
+            if (rc != SMX_OK) return rc;
+            if (out_scratch) {  // the quantised activation stays in LDS on this path: rebuild it for the checks
+                rc = silu_mul_quant(c, s.g, s.u, eff, k, eff, s.aq, s.ad);
+                if (rc != SMX_OK) return rc;
+            }
+        }
+    }
+    if (q6_flat) {
+    } else if (L.type == kQ6_K) {
         // Q6_K experts (decode.rs:2839-2852, moe6_launches): the down projections are k more jobs of the
         // grouped GEMV, each quantising silu(g_k)*u_k inside its staging; then the weighted sum
         float* dy = (float*)(c->work.p + o_dy);
