@@ -228,6 +228,48 @@ def test_ffn_block_two_launches_in_a_graph(accel, orc, synth, relerr, act):
         accel.dev_free(p)
 
 
+@pytest.mark.parametrize("act", [2, 3])
+def test_ffn_block_with_the_product_in_the_first_launch_in_a_graph(accel, orc, synth, relerr, act):
+    """The same step as smx_ffn_gate_up_dev (norm + quantiser + gate/up + activation product) and a plain GEMV on the
+    product: its quantised input has the bits of the three-launch form's, so the two forms give identical outputs;
+    captured and replayed with the activation changed between replays."""
+    H, F = 1024, 2560
+    rg, ru, rd = synth.make_weight(2, F, H, seed=31), synth.make_weight(2, F, H, seed=32), synth.make_weight(2, H, F, seed=33)
+    assert accel.upload_q4_0("t.ffn.gate", rg, H, F) and accel.upload_q4_0("t.ffn.up", ru, H, F)
+    assert accel.upload_q4_0("t.ffn.down", rd, F, H)
+    xs = synth.make_acts(3, H, seed=34) * 2.0
+    nw = synth.make_acts(1, H, seed=35)[0] * 0.1 + 1.0
+    xd, wd, gd, ud, hd, yd = (accel.dev_alloc(n * 4) for n in (H, H, F, F, F, H))
+    accel.h2d(wd, nw)
+
+    def three(out):
+        accel.gemv_fused_dev(["t.ffn.gate", "t.ffn.up"], 1, xd, wd, [gd, ud], 1e-6)
+        accel.gemv_fused_dev(["t.ffn.down"], act, gd, ud, [out])
+
+    def two(out):
+        accel.ffn_gate_up_dev("t.ffn.gate", "t.ffn.up", act, xd, hd, norm=True, norm_w_dev=wd, eps=1e-6)
+        accel.gemv_dev("t.ffn.down", hd, 1, out)
+
+    accel.h2d(xd, xs[0])
+    two(yd)
+    accel.graph_begin()
+    two(yd)
+    graph = accel.graph_end()
+    for rep in range(3):
+        accel.h2d(xd, xs[rep])
+        three(yd)
+        ref = accel.d2h(np.empty(H, np.float32), yd)
+        accel.h2d(yd, np.zeros(H, np.float32))
+        accel.graph_launch(graph)
+        accel.sync()
+        assert np.array_equal(accel.d2h(np.empty(H, np.float32), yd), ref), f"replay {rep}"
+    accel.graph_destroy(graph)
+    for p in (xd, wd, gd, ud, hd, yd):
+        accel.dev_free(p)
+    for k in ("gate", "up", "down"):
+        accel.evict("t.ffn." + k)
+
+
 def test_evict_and_reupload_keep_a_live_graph_valid(pkg, synth):
     """A captured graph holds the plane pointers of the weights it uses.  While it is alive, evicting or
     replacing such a weight must not free the device memory under it: replays keep giving the result
