@@ -183,20 +183,30 @@ static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nby
         off_scales = off_sc + align256(total * 16);
         w.bytes = off_scales + total * 2;
     }
-    // the raw blocks, padded to whole 16-byte pieces, next to the planes they are split into
-    char* raw = nullptr;
+    // The raw blocks, padded to whole 16-byte pieces, next to the planes they are split into.  The staging buffer belongs to
+    // the context and is reused by the next upload (a model's tensors arrive one after the other: no allocation and release
+    // per tensor); one of more than kRawKeepBytes is given back at once.
+    constexpr size_t kRawKeepBytes = size_t(256) << 20;
     const size_t raw_bytes = (nbytes + 15) & ~size_t(15);
-    hipError_t e = hipMalloc((void**)&raw, raw_bytes);
-    if (e == hipSuccess) e = hipMalloc((void**)&w.base, w.bytes);
+    int rc0 = ensure(c, c->raw, raw_bytes);
+    if (rc0 != SMX_OK) return rc0;
+    char* raw = c->raw.p;
+    auto drop_raw = [&]() {
+        if (c->raw.cap > kRawKeepBytes) {
+            (void)hipFree(c->raw.p);
+            c->raw.p = nullptr;
+            c->raw.cap = 0;
+        }
+    };
+    hipError_t e = hipMalloc((void**)&w.base, w.bytes);
     if (e != hipSuccess) {
         (void)hipGetLastError();
-        if (raw) (void)hipFree(raw);
-        return fail(c, SMX_ERR_NOMEM, "upload: device allocation of %zu + %zu bytes failed: %s", w.bytes, raw_bytes,
-                    hipGetErrorString(e));
+        drop_raw();
+        return fail(c, SMX_ERR_NOMEM, "upload: device allocation of %zu bytes failed: %s", w.bytes, hipGetErrorString(e));
     }
     auto bail = [&](hipError_t err, const char* what) {
         (void)hipStreamSynchronize(c->stream);
-        (void)hipFree(raw);
+        drop_raw();
         (void)hipFree(w.base);
         return hip_fail(c, err, what);
     };
@@ -226,7 +236,7 @@ static int build_weight(smx_ctx* c, QType type, const uint8_t* bytes, size_t nby
     }
     if ((e = hipGetLastError()) != hipSuccess) return bail(e, "repack launch");
     if ((e = hipStreamSynchronize(c->stream)) != hipSuccess) return bail(e, "repack");
-    (void)hipFree(raw);
+    drop_raw();
     w.scales = scales;
     w.quants = w.base + off_quants;
     w.qh = type == kQ6_K ? w.base + off_qh : nullptr;
@@ -322,7 +332,7 @@ void smx_destroy(smx_ctx* c) {
         free_weight(kv.second.up);
         free_weight(kv.second.down);
     }
-    for (DevBuf* b : {&c->xf32, &c->xq, &c->xd, &c->xs, &c->yf32, &c->work, &c->work2, &c->tab})
+    for (DevBuf* b : {&c->xf32, &c->xq, &c->xd, &c->xs, &c->yf32, &c->work, &c->work2, &c->tab, &c->raw})
         if (b->p) (void)hipFree(b->p);
     for (char* p : c->retired) (void)hipFree(p);
     for (DevBuf* b : {&c->hx, &c->hy, &c->htab})

@@ -73,6 +73,7 @@ struct smx_ctx {
     smx::DevBuf work;   // split-K partials, MoE intermediates, dumps
     smx::DevBuf work2;
     smx::DevBuf tab;    // small tables (ids, weights, tile tables)
+    smx::DevBuf raw;    // upload staging: the raw GGUF blocks of the tensor being repacked (kept up to kRawKeepBytes between uploads)
     smx::DevBuf hx, hy; // pinned HOST staging of the host-pointer calls' activations and results
     smx::DevBuf htab;   // pinned HOST staging of the small tables of enqueue-only calls
     hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
