@@ -206,7 +206,31 @@ class Bench:
         return (ms / n * 1e3 if n else float("nan")), n
 
     # ------------------------------------------------------------------ GEMV
-    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False):
+    def _trait_calls(self, keys, x, N, calls=200):
+        """What a drop-in caller of the accelerator trait gets: host-pointer calls (activation in, result out, one stream
+        synchronisation per call; PCIe-inclusive, never `value`), against the rotating weight copies.  us per call of
+        smx_gemv (int8 activations), smx_gemv_f32 (the reference's per-weight gemv arithmetic) and smx_gemv_batch of 8."""
+        acc = self.acc
+        out = {}
+        for label, fn in (("gemv", lambda i: acc.gemv(keys[i % len(keys)], x, N)),
+                          ("gemv_f32", lambda i: acc.gemv_f32(keys[i % len(keys)], x, N))):
+            for i in range(10):
+                fn(i)
+            t0 = time.perf_counter()
+            for i in range(calls):
+                fn(10 + i)
+            out[label] = (time.perf_counter() - t0) / calls * 1e6
+        nb = max(1, calls // 8)
+        batch = lambda i: acc.gemv_batch([(keys[(8 * i + j) % len(keys)], x) for j in range(8)], [N] * 8)
+        batch(0)
+        t0 = time.perf_counter()
+        for i in range(nb):
+            batch(1 + i)
+        out["gemv_batch_of_8"] = (time.perf_counter() - t0) / nb * 1e6
+        out["note"] = "host-pointer trait calls, PCIe and one sync per call included"
+        return out
+
+    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False, trait=False):
         """m rows against rotating weight copies.  m <= 4: the dot4 GEMV (quantiser fused for m = 1); 5..32 rows of a
         Q8_0 / Q4_0 weight: the small-batch kernel on the matrix cores; f32: the fp32-activation GEMV (no quantiser)."""
         acc, sy = self.acc, self.synth
@@ -241,6 +265,7 @@ class Bench:
         kname = ("gemv_f32_" + KERNEL[ty][5:]) if f32 else (KERNEL[ty] if m <= 4 or ty == Q6_K else "skinny_" + KERNEL[ty][5:])
         ms, wall_ms, queued = self._timed_queued(step, steps, warmup)
         kus, nk = self._kernel_avg_us(step, steps, warmup, kname)
+        trait_us = self._trait_calls(keys, x[0], N) if trait and m == 1 else None
         for k in keys:
             acc.evict(k)
         acc.dev_free(xd)
@@ -262,7 +287,7 @@ class Bench:
             "kernel_timing": ("events around the timed region's back-to-back launches / launches" if single
                               else "event pair around each launch"),
             "upload_GBps": upload_gbps,   # set-up: host call to synchronised device, raw block bytes per second
-            **queued,
+            **queued, **({"trait_call_us": trait_us} if trait_us else {}),
         }
 
     # ------------------------------------------------------------------ grouped GEMV (one launch, G weights)
@@ -647,7 +672,7 @@ def main():
     if a.no_headline and only:
         head = None
     else:
-        head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB))
+        head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB), trait=True)
         work[head["workload"]] = head
         b.log(json.dumps(head))
     plans = [

@@ -111,6 +111,10 @@ int smx_gemv_rows(smx_ctx* ctx, const char* key, const float* xs, size_t m, size
  * pairs, one device job, one sync.  status[i] receives the per-item code. */
 int smx_gemv_batch(smx_ctx* ctx, size_t n, const char* const* keys, const float* const* xs,
                    const size_t* in_lens, float* const* ys, const size_t* out_caps, int* status);
+/* The same batch in the arithmetic of smx_gemv_f32 (what the reference's gemv_batch launches,
+ * decode.rs:3227-3255 over the fp32-activation kernels): one launch per item, back to back, one sync. */
+int smx_gemv_f32_batch(smx_ctx* ctx, size_t n, const char* const* keys, const float* const* xs,
+                       const size_t* in_lens, float* const* ys, const size_t* out_caps, int* status);
 
 /* ---- prefill GEMM ---- */
 /* WeightAccel::prefill_q8_gemm, accel.rs:213; decode.rs:3257-3297 (and the

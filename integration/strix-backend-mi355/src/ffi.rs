@@ -112,6 +112,16 @@ extern "C" {
         out_caps: *const usize,
         status: *mut c_int,
     ) -> c_int;
+    pub fn smx_gemv_f32_batch(
+        ctx: *mut SmxCtx,
+        n: usize,
+        keys: *const *const c_char,
+        xs: *const *const c_float,
+        in_lens: *const usize,
+        ys: *const *mut c_float,
+        out_caps: *const usize,
+        status: *mut c_int,
+    ) -> c_int;
     pub fn smx_gemm(
         ctx: *mut SmxCtx,
         key: *const c_char,

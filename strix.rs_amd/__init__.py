@@ -36,7 +36,7 @@ EXPORTS = [
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
     "smx_weight_dims", "smx_moe_layer_stages", "smx_gemv_noalloc_dev",
-    "smx_gemv_f32", "smx_gemv_f32_dev", "smx_moe_route_dev", "smx_moe_route", "smx_moe_ffn_routed_dev",
+    "smx_gemv_f32", "smx_gemv_f32_dev", "smx_gemv_f32_batch", "smx_moe_route_dev", "smx_moe_route", "smx_moe_ffn_routed_dev",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -82,6 +82,7 @@ def load_library():
     L.smx_gemv_f32_dev.argtypes = [vp, cp, vp, vp]
     L.smx_gemv_rows.argtypes = [vp, cp, vp, sz, sz, vp, sz]
     L.smx_gemv_batch.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp]
+    L.smx_gemv_f32_batch.argtypes = [vp, sz, vp, vp, vp, vp, vp, vp]
     L.smx_gemm.argtypes = [vp, cp, vp, sz, sz, vp, sz]
     L.smx_lm_head_argmax_rows.argtypes = [vp, cp, vp, sz, sz, vp]
     L.smx_moe_ffn.argtypes = [vp, sz, vp, vp, sz, vp, sz, C.c_float, vp, sz]
@@ -365,8 +366,8 @@ class Mi355WeightAccel:
         ok = self._check(self._L.smx_gemv_rows(self._h, key.encode(), _p(xs), m, k, _p(y), y.size))
         return y if ok else None
 
-    def gemv_batch(self, calls, out_dims):
-        """calls: [(key, x)], out_dims: [out_dim]; returns [array | None] (accel.rs:397)."""
+    def gemv_batch(self, calls, out_dims, f32=False):
+        """calls: [(key, x)], out_dims: [out_dim]; returns [array | None] (accel.rs:397).  f32: the arithmetic of gemv_f32."""
         n = len(calls)
         xs = [_c(x, np.float32).reshape(-1) for _, x in calls]
         ys = [np.empty(d, np.float32) for d in out_dims]
@@ -376,7 +377,8 @@ class Mi355WeightAccel:
         il = (C.c_size_t * n)(*[x.size for x in xs])
         oc = (C.c_size_t * n)(*[y.size for y in ys])
         st = (C.c_int * n)()
-        self._check(self._L.smx_gemv_batch(self._h, n, keys, xp, il, yp, oc, st))
+        fn = self._L.smx_gemv_f32_batch if f32 else self._L.smx_gemv_batch
+        self._check(fn(self._h, n, keys, xp, il, yp, oc, st))
         out = []
         for i in range(n):
             if st[i] < 0:

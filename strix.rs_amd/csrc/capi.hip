@@ -176,8 +176,10 @@ int smx_gemm(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_d
     return matmul_host(c, key, xs, m, in_dim, y, y_cap, true, "gemm");
 }
 
-int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs, const size_t* in_lens,
-                   float* const* ys, const size_t* out_caps, int* status) {
+// One device job and one synchronisation for n host-pointer GEMVs.  f32: every item runs the fp32-activation kernel
+// (one launch per item, back to back); otherwise consecutive items of one format and row length share a launch.
+static int gemv_batch_host(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs, const size_t* in_lens,
+                           float* const* ys, const size_t* out_caps, int* status, bool f32) {
     if (!c) return SMX_ERR_ARG;
     if (!keys || !xs || !in_lens || !ys || !out_caps || !status) return fail(c, SMX_ERR_ARG, "gemv_batch: null argument");
     return guarded(c, "gemv_batch", [&]() -> int {
@@ -235,6 +237,11 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
     // consecutive items of one format and row length share a launch (up to 8 per launch)
     for (size_t i = 0; i < n;) {
         if (!ws[i]) { i++; continue; }
+        if (f32) {
+            status[i] = launch_gemv_f32(c, *ws[i], xdev[i], ydev[i]);
+            i++;
+            continue;
+        }
         const Weight* gw[8];
         const float* gx[8];
         float* gy[8];
@@ -262,6 +269,16 @@ int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* c
             if (ws[i] && status[i] == SMX_OK) memcpy(ys[i], c->hy.p + yoff[i], ws[i]->N * 4);
     return SMX_OK;
     });
+}
+
+int smx_gemv_batch(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs, const size_t* in_lens,
+                   float* const* ys, const size_t* out_caps, int* status) {
+    return gemv_batch_host(c, n, keys, xs, in_lens, ys, out_caps, status, false);
+}
+
+int smx_gemv_f32_batch(smx_ctx* c, size_t n, const char* const* keys, const float* const* xs, const size_t* in_lens,
+                       float* const* ys, const size_t* out_caps, int* status) {
+    return gemv_batch_host(c, n, keys, xs, in_lens, ys, out_caps, status, true);
 }
 
 int smx_lm_head_argmax_rows(smx_ctx* c, const char* key, const float* xs, size_t m, size_t in_dim, uint32_t* out) {

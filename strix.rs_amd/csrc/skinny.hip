@@ -274,8 +274,8 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         };
 #pragma unroll
         for (int bi = 0; bi < 4; bi++) {
-            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero scale
-            const float dxv = __uint_as_float(dxs[bi]);
+            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, both scales zero
+            const float dxv = live ? __uint_as_float(dxs[bi]) : 0.f;  // (whatever an earlier call left in the scale slots past K)
             if constexpr (Q6) {
                 const float d6 = h2f_s(r.d6), d6m128 = -128.f * d6;
 #pragma unroll
@@ -390,7 +390,11 @@ __global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restri
         w[i] = pk;
     }
     if (gid < nchunks) xq[gid] = make_uint4(w[0], w[1], w[2], w[3]);
-    if (live && h == 0) xd[((b >> 2) * tslots + t) * 4 + (b & 3)] = d;
+    if (live && h == 0) {
+        xd[((b >> 2) * tslots + t) * 4 + (b & 3)] = d;
+        if (b == (size_t)nb - 1)   // the scale slots of the last piece past K: zero, not what an earlier call left there
+            for (size_t bb = b + 1; bb < (((size_t)nb + 3) & ~(size_t)3); bb++) xd[((bb >> 2) * tslots + t) * 4 + (bb & 3)] = 0.f;
+    }
 }
 
 }  // namespace

@@ -102,7 +102,7 @@ SMALL_BATCH = [(8, 96, 256), (8, 130, 2560), (8, 37, 9728), (2, 130, 2560), (2, 
 def test_small_batch_matches_oracle(accel, orc, synth, relerr, ty, N, K):
     raw = synth.make_weight(ty, N, K, seed=N + K)
     assert getattr(accel, UPLOAD[ty])("t.sb", raw, K, N)
-    for m in (5, 8, 9, 16, 17, 32):
+    for m in (5, 6, 7, 8, 9, 16, 17, 32):
         xs = synth.make_acts(m, K, seed=m + N)
         ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
         y = accel.prefill_q8_gemm("t.sb", xs, m, N)               # WeightAccel::prefill_q8_gemm with a short chunk
@@ -115,6 +115,27 @@ def test_small_batch_matches_oracle(accel, orc, synth, relerr, ty, N, K):
             for t in range(m):
                 assert np.array_equal(dots[t], orc.block_dots(ty, raw, K, N, xq[t])), (m, t)
     accel.evict("t.sb")
+
+
+@pytest.mark.parametrize("ty", [8, 2])
+def test_small_batch_ignores_stale_scales_past_k(accel, orc, synth, relerr, ty):
+    """The activation scales of a call's last 4-block piece have slots past K when K is not a multiple of 128.  An earlier
+    call leaves its own scales there (here: infinite ones, from infinite activations on a longer row); the next call's
+    outputs must not see them (0 * inf would be NaN in every output)."""
+    N = 64
+    for m in (5, 12, 20):
+        k_long, k_short = 2688, 2592          # 21 whole pieces / 20 pieces + 1 block
+        raw_long = synth.make_weight(ty, N, k_long, seed=1)
+        raw = synth.make_weight(ty, N, k_short, seed=2)
+        assert getattr(accel, UPLOAD[ty])("t.stale.a", raw_long, k_long, N)
+        assert getattr(accel, UPLOAD[ty])("t.stale.b", raw, k_short, N)
+        accel.gemv_rows("t.stale.a", np.full((m, k_long), np.inf, np.float32), N)
+        xs = synth.make_acts(m, k_short, seed=m)
+        y = accel.gemv_rows("t.stale.b", xs, N)
+        assert np.isfinite(y).all()
+        assert relerr(y, orc.matmul_q8_from_f32(ty, raw, k_short, N, xs)) <= TOL
+    accel.evict("t.stale.a")
+    accel.evict("t.stale.b")
 
 
 def test_small_batch_rows_equal_single_rows(accel, synth, relerr):

@@ -121,7 +121,7 @@ def test_gemv_group_with_more_workgroups_than_cus(accel, orc, synth, relerr):
 
 
 @pytest.mark.parametrize("ty", [2, 8])
-@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemv_rows_batched(accel, orc, synth, relerr, ty, m):
     N, K = 200, 2560
     raw = synth.make_weight(ty, N, K, seed=31 + m)
@@ -301,6 +301,26 @@ def test_gemv_f32_matches_f32_oracle(accel, orc, synth, relerr, ty, N, K):
     for order in (0, 1):      # both summation orders of strix-backend-cpu (gemma.rs:323-326, mellum.rs:278-293)
         assert relerr(y, orc.matmul_f32(ty, raw, K, N, x, order=order)[0]) <= 1e-5
     accel.evict("t.f32")
+
+
+def test_gemv_f32_batch_equals_single_calls(accel, orc, synth, relerr):
+    """gemv_batch in the fp32-activation arithmetic (what the trait's default binding calls): one device job, one sync,
+    every item the bits of its single call; items that are not resident decline, the others still run."""
+    K, Ns = 2560, (64, 200, 96)
+    raws = [synth.make_weight(ty, n, K, seed=ty + n) for ty, n in zip((2, 8, 14), Ns)]
+    for ty, raw, n in zip((2, 8, 14), raws, Ns):
+        _up(accel, ty, f"t.fb{ty}", raw, K, n)
+    xs = [synth.make_acts(1, K, seed=60 + i)[0] for i in range(4)]
+    calls = [("t.fb2", xs[0]), ("t.fb8", xs[1]), ("t.nope", xs[2]), ("t.fb14", xs[3]), ("t.fb2", xs[3])]
+    dims = [Ns[0], Ns[1], 7, Ns[2], Ns[0]]
+    out = accel.gemv_batch(calls, dims, f32=True)
+    assert out[2] is None
+    for i, (key, x) in enumerate(calls):
+        if i != 2:
+            assert np.array_equal(out[i], accel.gemv_f32(key, x, dims[i])), i
+    assert relerr(out[1], orc.matmul_f32(8, raws[1], K, Ns[1], xs[1])[0]) <= 1e-5
+    for ty in (2, 8, 14):
+        accel.evict(f"t.fb{ty}")
 
 
 def test_gemv_f32_limits(accel, synth, pkg):
