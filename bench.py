@@ -468,57 +468,72 @@ class Bench:
         }
 
     # ------------------------------------------------------------------ decode chain as one graph
-    def decode_chain_graph(self, name, layers=4, hidden=2048, ffn=8192, ne=64, eff=768, k=8, steps=None, warmup=None):
-        """`layers` decoder FFN halves captured once as ONE HIP graph and replayed per token, everything resident and
-        routed on the device: per layer rmsnorm + gate/up GEMVs + SwiGLU product (one launch), down GEMV, router logits GEMV,
-        top-k router, the k routed experts' FFN (gate/up, down).  Attention is outside this path.  Q4_0 dense
-        weights, Q8_0 experts and router."""
+    def decode_chain_graph(self, name, layers=4, hidden=2048, ffn=8192, ne=64, eff=768, k=8, nsets=4, steps=None, warmup=None):
+        """`layers` decoder FFN halves per token, everything resident and routed on the device (strix.rs_amd/chain.py, the
+        sequence tests/test_gpu_chain.py checks against the oracle): per layer rmsnorm + gate/up GEMVs + SwiGLU product
+        (one launch), down GEMV, router logits + top-k (one launch), the k routed experts' FFN (two launches).  Attention
+        is outside this path.  Q4_0 dense weights, Q8_0 experts and router.  Cache-cold: `nsets` complete weight sets
+        (every layer's dense weights and expert tensors) are resident and ONE captured graph runs one token through each
+        set in turn, so a token's weights were last read nsets - 1 tokens (> 1 GB of other weights) ago."""
         acc, sy = self.acc, self.synth
+        chain_mod = _load("strix_rs_amd_chain", os.path.join(ROOT, "strix.rs_amd", "chain.py"))
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
         base = 50
-        for l in range(layers):
-            assert acc.upload_q4_0(f"{name}.g{l}", sy.make_weight(Q4_0, ffn, hidden, seed=4000 + l), hidden, ffn)
-            assert acc.upload_q4_0(f"{name}.u{l}", sy.make_weight(Q4_0, ffn, hidden, seed=4100 + l), hidden, ffn)
-            assert acc.upload_q4_0(f"{name}.d{l}", sy.make_weight(Q4_0, hidden, ffn, seed=4200 + l), ffn, hidden)
-            assert acc.upload_q8_0(f"{name}.r{l}", sy.make_weight(Q8_0, ne, hidden, seed=4300 + l), hidden, ne)
-            gate, up, down = sy.make_moe_q8(ne, hidden, eff, seed=4400 + l)
+        nl = layers * nsets
+        dense = [(sy.make_weight(Q4_0, ffn, hidden, seed=4000 + i), sy.make_weight(Q4_0, hidden, ffn, seed=4200 + i)) for i in range(2)]
+        router = sy.make_weight(Q8_0, ne, hidden, seed=4300)
+        gate, up, down = sy.make_moe_q8(ne, hidden, eff, seed=4400)
+        for l in range(nl):
+            assert acc.upload_q4_0(f"{name}.g{l}", dense[l % 2][0], hidden, ffn)
+            assert acc.upload_q4_0(f"{name}.u{l}", dense[(l + 1) % 2][0], hidden, ffn)
+            assert acc.upload_q4_0(f"{name}.d{l}", dense[l % 2][1], ffn, hidden)
+            assert acc.upload_q8_0(f"{name}.r{l}", router, hidden, ne)
             assert acc.upload_moe_q8(base + l, gate, up, down, hidden, eff, ne)
+        del dense, gate, up, down
         x = sy.make_acts(1, hidden, seed=11)
-        xd, nw, gd, ud, hd, ld, yd = (acc.dev_alloc(n * 4) for n in (hidden, hidden, ffn, ffn, hidden, ne, hidden))
-        idd, wd = acc.dev_alloc(k * 4), acc.dev_alloc(k * 4)
+        xd, nw = acc.dev_alloc(hidden * 4), acc.dev_alloc(hidden * 4)
         acc.h2d(xd, x)
         acc.h2d(nw, np.ones(hidden, np.float32))
+        keys = lambda l: tuple(f"{name}.{t}{l}" for t in "gudr")
 
-        def chain():
-            cur = xd
-            for l in range(layers):
-                acc.ffn_gate_up_dev(f"{name}.g{l}", f"{name}.u{l}", 2, cur, gd, norm=True, norm_w_dev=nw, eps=1e-6)
-                acc.gemv_dev(f"{name}.d{l}", gd, 1, hd)
-                acc.gemv_dev(f"{name}.r{l}", hd, 1, ld)
-                acc.moe_route_dev(ld, ne, k, idd, wd)
-                acc.moe_ffn_routed_dev(base + l, idd, wd, k, hd, yd)
-                cur = yd
+        def measure(fused_router, sets):
+            ch = chain_mod.FfnMoeChain(acc, layers, hidden, ffn, ne, k, keys, lambda l: base + l, nw, fused_router=fused_router)
 
-        chain()
-        acc.sync()
-        acc.graph_begin()
-        chain()
-        g = acc.graph_end()
-        eager_ms, _ = self._timed(lambda i: chain(), steps, warmup)
-        graph_ms, _ = self._timed(lambda i: acc.graph_launch(g), steps, warmup)
-        acc.graph_destroy(g)
-        for l in range(layers):
+            def tokens():   # one token through each weight set
+                for s_ in range(sets):
+                    ch.enqueue(xd, layer_offset=s_ * layers)
+
+            tokens()        # also the first read of every set's weights
+            acc.sync()
+            acc.graph_begin()
+            tokens()
+            g = acc.graph_end()
+            reps = max(1, steps // sets)
+            eager_ms, _ = self._timed(lambda i: tokens(), reps, max(1, warmup // sets))
+            graph_ms, _ = self._timed(lambda i: acc.graph_launch(g), reps, max(1, warmup // sets))
+            acc.graph_destroy(g)
+            n_launch = ch.launches_per_token()
+            ch.close()
+            return graph_ms / (reps * sets) * 1e3, eager_ms / (reps * sets) * 1e3, n_launch
+
+        cold_us, cold_eager_us, n_launch = measure(True, nsets)
+        two_launch_router_us, _, _ = measure(False, nsets)
+        hot_us, _, _ = measure(True, 1)
+        for l in range(nl):
             for t in "gudr":
                 acc.evict(f"{name}.{t}{l}")
-        for p in (xd, nw, gd, ud, hd, ld, yd, idd, wd):
-            acc.dev_free(p)
+        acc.dev_free(xd)
+        acc.dev_free(nw)
         wbytes = layers * (3 * gemv_bytes(Q4_0, ffn, hidden)[1] + gemv_bytes(Q8_0, ne, hidden)[1] + k * 3 * eff * (hidden // 32) * 34)
+        gbs = wbytes / (cold_us * 1e-6) / 1e9
         return {"workload": name, "shape": {"layers": layers, "hidden": hidden, "ffn": ffn, "experts": ne, "eff": eff, "top_k": k,
-                                            "launches_per_token": layers * 6},
-                "weight_bytes_per_token": wbytes, "steps": steps, "graph_us_per_token": graph_ms / steps * 1e3,
-                "eager_us_per_token": eager_ms / steps * 1e3, "GBps": wbytes * steps / (graph_ms * 1e-3) / 1e9,
-                "frac_hbm_peak": wbytes * steps / (graph_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                "note": "weights (304 MB) stay in the 256 MB Infinity Cache in part: not a cache-cold figure"}
+                                            "launches_per_token": n_launch, "weight_sets_rotated": nsets},
+                "weight_bytes_per_token": wbytes, "bytes_between_two_reads_of_a_weight": wbytes * (nsets - 1),
+                "steps": max(1, steps // nsets) * nsets, "graph_us_per_token": cold_us, "eager_us_per_token": cold_eager_us,
+                "router_as_two_launches_us_per_token": two_launch_router_us, "one_weight_set_us_per_token": hot_us,
+                "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
+                "note": "graph_us_per_token is cache-cold (weight sets rotate); one_weight_set_us_per_token re-reads one 274 MB "
+                        "set, partly from the 256 MB Infinity Cache"}
 
     # ------------------------------------------------------------------ MoE
     def moe(self, name, ne, hidden, eff, k, m, layers, steps=None, warmup=None, ty=Q8_0):
@@ -588,6 +603,13 @@ class Bench:
             acc.dev_free(xd)
             acc.dev_free(yd)
             ops = 2 * slot_tok.size * 3 * eff * hidden
+            # This configuration is HBM-bound, not MFMA-bound: 38.65 GOP over the weights of every expert that got a token
+            # (302 MB when all 64 did) is 128 op/B, far left of the 625 op/B ridge of 5 POP/s over 8 TB/s.
+            active = sum(1 for e_, _, cnt in plan if cnt > 0)
+            wbytes = active * 3 * eff * (hidden // 256 * 210 if ty == Q6_K else hidden // 32 * 34)
+            out.update({"bound": "hbm", "active_experts": active, "expert_weight_bytes": wbytes,
+                        "GBps": wbytes * steps / (all_ms * 1e-3) / 1e9,
+                        "frac_hbm_peak": wbytes * steps / (all_ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
             out.update({"resident_ms_per_step": res_ms / steps, "resident_TOPS": ops * steps / (res_ms * 1e-3) / 1e12})
             out.update({"slots": int(slot_tok.size), "ops": ops, "steps": steps,
                         "device_ms_per_step": all_ms / steps, "host_call_ms_per_step": wall_ms / steps,

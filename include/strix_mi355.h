@@ -222,6 +222,13 @@ int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float*
  * same with host buffers (one sync). */
 int smx_moe_route_dev(smx_ctx* ctx, const float* logits_dev, size_t ne, size_t k, int32_t* ids_dev, float* w_dev);
 int smx_moe_route(smx_ctx* ctx, const float* logits, size_t ne, size_t k, int32_t* ids, float* w);
+/* Router logits and routing in ONE launch: logits = W_router . x for the resident router weight `key` (out_dim = number of
+ * experts; the reference launches f32_gemv on its router weight and then topk_router, decode.rs:1136-1166), then the routing
+ * of smx_moe_route_dev on them.  One workgroup serves a router of up to 256 experts whose rows take the flat GEMV form
+ * (64 x 2048 Q8_0 = 139 KB); other shapes run as the two launches.  The logits have the bits of smx_gemv_dev, the routing
+ * those of smx_moe_route_dev on them.  logits_dev (optional, [out_dim]) also receives the logits. */
+int smx_moe_router_dev(smx_ctx* ctx, const char* key, const float* x_dev, size_t k, int32_t* ids_dev, float* w_dev,
+                       float* logits_dev);
 /* smx_moe_ffn_dev with the routing read from device memory when the kernels run (what smx_moe_route_dev
  * wrote): router + expert FFN of a decode token can be captured once and replayed with every token's own
  * routing (decode.rs:1923-2128 reads the router's device output the same way).  Ids outside 0 .. ne - 1

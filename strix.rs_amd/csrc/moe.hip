@@ -95,18 +95,19 @@ __device__ __forceinline__ float route_w(const MoeRoute& r, int i) { return r.w_
 // lane l holds experts l, l + 64, ... (PL of them: 1 for up to 64 experts, which keeps the k selection
 // rounds at one compare each).  The softmax denominator is summed in double in a fixed order.
 constexpr int kRouterPerLane = 16;   // ne <= 1024
+// The router's arithmetic, run by ONE wave: v[j] = logit of expert lane + 64 j (-FLT_MAX past ne); sel: 64 floats of LDS.
 template <int PL>
-__global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict__ logits, int ne, int k,
-                                                         int* __restrict__ ids, float* __restrict__ w) {
+__device__ __forceinline__ void topk_router_wave(float (&v)[PL], int ne, int k, int* __restrict__ ids, float* __restrict__ w,
+                                                 float* sel) {
 #pragma clang fp contract(off)
     constexpr int kRouterPerLane = PL;
-    const int lane = threadIdx.x;
-    if (PL == 1) {
+    const int lane = threadIdx.x & 63;
+    if constexpr (PL == 1) {
         // Up to 64 experts, one per lane: every cross-lane step is a lane read into a scalar register (no
         // LDS round trips, which dominate the time of this one-wave kernel).  A lane's rank = the number
         // of experts that precede it in (probability descending, index ascending) order; rank r < k is pick r.
         const bool live = lane < ne;
-        const float x = live ? logits[lane] : -3.40282347e+38f;
+        const float x = v[0];
         float mx = -3.40282347e+38f;
 #pragma unroll
         for (int j = 0; j < 64; j++) mx = fmaxf(mx, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j)));
@@ -121,25 +122,22 @@ __global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict
             const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), j));
             rank += (pj > p || (pj == p && j < lane)) ? 1 : 0;
         }
-        __shared__ float sel[64];
         if (live && rank < k) {
             sel[rank] = p;
             ids[rank] = lane;
         }
-        __syncthreads();
+        // one wave: its own LDS writes, read back by its other lanes
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         float wsum = 0.f;   // in pick order, as the reference sums the chosen probabilities
         for (int i = 0; i < k; i++) wsum += sel[i];
         if (lane < k) w[lane] = sel[lane] / wsum;
         return;
     }
-    float v[kRouterPerLane];
     float mx = -3.40282347e+38f;
 #pragma unroll
-    for (int j = 0; j < kRouterPerLane; j++) {
-        const int e = lane + 64 * j;
-        v[j] = e < ne ? logits[e] : -3.40282347e+38f;
-        mx = fmaxf(mx, v[j]);
-    }
+    for (int j = 0; j < kRouterPerLane; j++) mx = fmaxf(mx, v[j]);
     for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
     double sum = 0.0;
 #pragma unroll
@@ -174,6 +172,43 @@ __global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict
         wsum += b;   // in pick order, as the reference sums the chosen probabilities
     }
     if (lane < k) w[lane] = mine / wsum;
+}
+
+template <int PL>
+__global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict__ logits, int ne, int k,
+                                                         int* __restrict__ ids, float* __restrict__ w) {
+    __shared__ float sel[64];
+    float v[PL];
+#pragma unroll
+    for (int j = 0; j < PL; j++) {
+        const int e = (int)threadIdx.x + 64 * j;
+        v[j] = e < ne ? logits[e] : -3.40282347e+38f;
+    }
+    topk_router_wave<PL>(v, ne, k, ids, w, sel);
+}
+
+// Router logits + routing in ONE launch (the reference's f32_gemv of the router weight followed by topk_router,
+// decode.rs:1136-1166): one 16-wave workgroup runs the flat GEMV over all ne rows of the (small) router weight -- 64 x 2048
+// Q8_0 is 139 KB -- writes the logits, and its first wave then routes them.  The logits have the bits of a separate GEMV
+// launch (a row's sum does not depend on how rows are shared out), the routing those of topk_router_kernel on them.
+template <class Ops, int PRE, int GL, int PL>
+__global__ __launch_bounds__(1024) void moe_router_fused_kernel(const GemvW W, const float* __restrict__ x, float* logits, int nblk,
+                                                                int ne, unsigned magic_u, int k, int* __restrict__ ids,
+                                                                float* __restrict__ w) {
+    extern __shared__ __align__(16) char router_smem[];
+    gemv_body_flat<Ops, 1, PRE, GL, 1>(W, GemvX{x, nullptr, nullptr, nullptr, nullptr, SMX_ACT_NONE, 0.f}, logits, ne, nblk, ne, 1, 0, 1,
+                                       magic_u);
+    __threadfence_block();   // the logits the other waves stored are read back by the first wave
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float v[PL];
+#pragma unroll
+        for (int j = 0; j < PL; j++) {
+            const int e = (int)threadIdx.x + 64 * j;
+            v[j] = e < ne ? *(const volatile float*)(logits + e) : -3.40282347e+38f;
+        }
+        topk_router_wave<PL>(v, ne, k, ids, w, (float*)router_smem);
+    }
 }
 
 // Decode, second half, in one launch: a_k = quantised silu(g_k)*u_k is rebuilt in LDS by every
@@ -926,6 +961,53 @@ int smx_moe_route_dev(smx_ctx* c, const float* logits_dev, size_t ne, size_t k, 
     hipLaunchKernelGGL(kern, dim3(1), dim3(64), 0, c->stream, logits_dev, (int)ne, (int)k, ids_dev, w_dev);
     SMX_HIP(c, hipGetLastError());
     return SMX_OK;
+}
+
+int smx_moe_router_dev(smx_ctx* c, const char* key, const float* x_dev, size_t k, int32_t* ids_dev, float* w_dev, float* logits_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!key || !x_dev || !ids_dev || !w_dev) return fail(c, SMX_ERR_ARG, "moe_router_dev: null argument");
+    return guarded(c, "moe_router_dev", [&]() -> int {
+        auto it = c->weights.find(key);
+        if (it == c->weights.end()) return SMX_NOT_RESIDENT;
+        const Weight& w = it->second;
+        const size_t ne = w.N;
+        if (ne > 64 * (size_t)kRouterPerLane || k == 0 || k > 64 || k > ne)
+            return fail(c, SMX_ERR_LIMIT, "moe_router_dev: %zu experts, top %zu (up to %d experts, top 64)", ne, k, 64 * kRouterPerLane);
+        int rc;
+        if (!logits_dev) {   // the logits still pass through memory: the context's own room when the caller does not want them
+            if ((rc = ensure(c, c->yf32, ne * 4)) != SMX_OK) return rc;
+            logits_dev = (float*)c->yf32.p;
+        }
+        // one workgroup serves the whole weight when its rows take the flat form and fit one workgroup's unit index and LDS
+        const size_t upb = w.type == kQ6_K ? 4 : (w.type == kQ8_0 ? 2 : 1);
+        const size_t units = w.nblk * upb;
+        const size_t tokb = w.type == kQ4_0 ? ((w.nblk * 40 + 15) & ~size_t(15))
+                                             : (w.type == kQ8_0 ? ((w.nblk * 36 + 15) & ~size_t(15)) : w.nblk * 2 * (OpsQ6_K::kPad * 16 + 32));
+        const int gl = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : ((w.type == kQ6_K && (units % 4) == 0) ? 4 : 0));
+        const size_t lds = gl ? tokb + ne * units / gl * 4 : 0;
+        if (gl && w.K <= 16384 && ne <= 256 && ne * units < 65536 && lds <= 160 * 1024) {
+            const GemvW W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
+            const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);
+            ProfScope ps(c, "moe_router_fused");
+            auto go = [&](auto kern) -> int {
+                int rc2 = set_dyn_lds(c, kern, lds);
+                if (rc2 != SMX_OK) return rc2;
+                hipLaunchKernelGGL(kern, dim3(1), dim3(1024), lds, c->stream, W, x_dev, logits_dev, (int)w.nblk, (int)ne, magic, (int)k,
+                                   ids_dev, w_dev);
+                SMX_HIP(c, hipGetLastError());
+                return SMX_OK;
+            };
+#define SMX_ROUTER(OPS, PRE, GL) \
+    if (gl == GL) return ne <= 64 ? go(moe_router_fused_kernel<OPS, PRE, GL, 1>) : go(moe_router_fused_kernel<OPS, PRE, GL, 4>);
+            if (w.type == kQ4_0) { SMX_ROUTER(OpsQ4_0, 3, 16) SMX_ROUTER(OpsQ4_0, 3, 8) }
+            else if (w.type == kQ8_0) { SMX_ROUTER(OpsQ8_0, 3, 16) SMX_ROUTER(OpsQ8_0, 3, 8) }
+            else { SMX_ROUTER(OpsQ6_K, 1, 16) SMX_ROUTER(OpsQ6_K, 1, 8) SMX_ROUTER(OpsQ6_K, 1, 4) }
+#undef SMX_ROUTER
+        }
+        // other shapes: the two launches
+        if ((rc = launch_gemv(c, w, x_dev, 1, logits_dev, nullptr)) != SMX_OK) return rc;
+        return smx_moe_route_dev(c, logits_dev, ne, k, ids_dev, w_dev);
+    });
 }
 
 int smx_moe_route(smx_ctx* c, const float* logits, size_t ne, size_t k, int32_t* ids, float* w) {

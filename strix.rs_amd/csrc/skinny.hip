@@ -274,8 +274,11 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         };
 #pragma unroll
         for (int bi = 0; bi < 4; bi++) {
-            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, both scales zero
-            const float dxv = live ? __uint_as_float(dxs[bi]) : 0.f;  // (whatever an earlier call left in the scale slots past K)
+            const bool live = blk0 + bi < p.nb;                       // blocks past K: clamped loads, zero weight scale
+            // The activation scale is used as it was loaded: the quantiser launch writes zeros into the scale slots past K, and a
+            // select here would be a vector write of the register the hand-written DPP multiply-adds below read through DPP
+            // (two wait states the compiler's hazard recogniser does not insert for inline assembly).
+            const float dxv = __uint_as_float(dxs[bi]);
             if constexpr (Q6) {
                 const float d6 = h2f_s(r.d6), d6m128 = -128.f * d6;
 #pragma unroll

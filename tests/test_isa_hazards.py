@@ -1,7 +1,8 @@
-"""The Q6_K GEMM epilogue reads its activation scale through hand-written `v_fmac_f32_dpp` instructions
-(inline assembly, so the compiler's hazard recogniser does not see them).  CDNA requires two wait states
-between a VALU write of a register and a DPP read of it: compile the kernel to assembly and check that
-no VALU instruction writes the DPP source register within the two instructions before each use."""
+"""The Q6_K GEMM epilogue, the small-batch kernel and the grouped MoE GEMM read their activation scale through hand-written
+`v_fmac_f32_dpp` instructions (inline assembly, so the compiler's hazard recogniser does not see them).  CDNA requires two
+wait states between a VALU write of a register and a DPP read of it: compile every source file that holds such an
+instruction to assembly and check that no VALU instruction writes the DPP source register within the two instructions
+before each use."""
 import os
 import re
 import shutil
@@ -13,11 +14,25 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
+def _dpp_sources():
+    """Source files of the library with a hand-written DPP multiply-add."""
+    csrc = os.path.join(ROOT, "strix.rs_amd", "csrc")
+    headers = [n for n in os.listdir(csrc) if n.endswith(".h") and "v_fmac_f32_dpp" in open(os.path.join(csrc, n)).read()]
+    names = []
+    for n in sorted(os.listdir(csrc)):
+        text = open(os.path.join(csrc, n)).read() if n.endswith(".hip") else ""
+        if "v_fmac_f32_dpp" in text or any(f'"{h}"' in text for h in headers):
+            names.append(n)
+    assert "gemm.hip" in names and "skinny.hip" in names
+    return names
+
+
 @pytest.mark.skipif(not os.path.exists(HIPCC) and not shutil.which("hipcc"), reason="hipcc not available")
-def test_no_valu_write_right_before_a_dpp_read(tmp_path):
-    out = tmp_path / "gemm.s"
+@pytest.mark.parametrize("source", _dpp_sources())
+def test_no_valu_write_right_before_a_dpp_read(tmp_path, source):
+    out = tmp_path / (source + ".s")
     cmd = [HIPCC if os.path.exists(HIPCC) else "hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
-           "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only", os.path.join(ROOT, "strix.rs_amd", "csrc", "gemm.hip"), "-o", str(out)]
+           "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only", os.path.join(ROOT, "strix.rs_amd", "csrc", source), "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True, timeout=600)
     lines = [l.strip() for l in out.read_text().splitlines()]
     lines = [l for l in lines if l and not l.startswith((";", ".")) and not l.endswith(":")]
