@@ -166,8 +166,8 @@ int smx_gemv_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, f
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same kernels and results
  * as smx_gemv_dev; the rows quantised for m >= 2 live in a static device array of the library (160 KB per
  * GPU, held until the process ends) instead of the context's growable scratch, so the call never
- * allocates or frees device or host memory.  Limits: m <= SMX_NOALLOC_MAX_ROWS, in_dim <= SMX_NOALLOC_MAX_IN_DIM
- * (SMX_ERR_LIMIT beyond).  All contexts of one GPU share the array: calls that overlap on one GPU race. */
+ * allocates or frees device or host memory.  Limits: m <= SMX_NOALLOC_MAX_ROWS, and for m >= 2 in_dim <= SMX_NOALLOC_MAX_IN_DIM
+ * (SMX_ERR_LIMIT beyond; a single row is quantised inside the GEMV and does not use the array).  All contexts of one GPU share the array: calls that overlap on one GPU race. */
 #define SMX_NOALLOC_MAX_IN_DIM 16384
 #define SMX_NOALLOC_MAX_ROWS 8
 int smx_gemv_noalloc_dev(smx_ctx* ctx, const char* key, const float* xs_dev, size_t m, float* y_dev);
@@ -222,11 +222,10 @@ int smx_moe_ffn_dev(smx_ctx* ctx, size_t layer, const int32_t* ids, const float*
  * same with host buffers (one sync). */
 int smx_moe_route_dev(smx_ctx* ctx, const float* logits_dev, size_t ne, size_t k, int32_t* ids_dev, float* w_dev);
 int smx_moe_route(smx_ctx* ctx, const float* logits, size_t ne, size_t k, int32_t* ids, float* w);
-/* Router logits and routing in ONE launch: logits = W_router . x for the resident router weight `key` (out_dim = number of
+/* Router logits and routing in one call: logits = W_router . x for the resident router weight `key` (out_dim = number of
  * experts; the reference launches f32_gemv on its router weight and then topk_router, decode.rs:1136-1166), then the routing
- * of smx_moe_route_dev on them.  One workgroup serves a router of up to 256 experts whose rows take the flat GEMV form
- * (64 x 2048 Q8_0 = 139 KB); other shapes run as the two launches.  The logits have the bits of smx_gemv_dev, the routing
- * those of smx_moe_route_dev on them.  logits_dev (optional, [out_dim]) also receives the logits. */
+ * of smx_moe_route_dev on them (two launches; capturable).  The logits have the bits of smx_gemv_dev, the routing those of
+ * smx_moe_route_dev on them.  logits_dev (optional, [out_dim]) also receives the logits. */
 int smx_moe_router_dev(smx_ctx* ctx, const char* key, const float* x_dev, size_t k, int32_t* ids_dev, float* w_dev,
                        float* logits_dev);
 /* smx_moe_ffn_dev with the routing read from device memory when the kernels run (what smx_moe_route_dev

@@ -556,7 +556,7 @@ class Mi355WeightAccel:
         return self._check(self._L.smx_moe_route_dev(self._h, logits_dev, ne, k, ids_dev, w_dev))
 
     def moe_router_dev(self, key, x_dev, k, ids_dev, w_dev, logits_dev=None):
-        """Router logits (GEMV of the resident router weight) + softmax + top-k in one launch."""
+        """Router logits (GEMV of the resident router weight) + softmax + top-k in one call."""
         return self._check(self._L.smx_moe_router_dev(self._h, key.encode(), x_dev, k, ids_dev, w_dev, logits_dev))
 
     def moe_ffn_routed_dev(self, layer, ids_dev, w_dev, k, x_dev, y_dev):

@@ -2,10 +2,10 @@
 as a HIP graph and replays per token (the reference's captured token, crates/strix-backend-rocm/src/decode.rs:3053-3203,
 and its per-layer launch sequence, decode.rs:1136-1180: router logits -> topk_router -> moe_launches).
 
-Per layer, five calls / five launches:
+Per layer, four calls / six launches:
     1. smx_ffn_gate_up_dev   rmsnorm + quantiser + gate and up GEMVs + SwiGLU product   x -> h[ffn]
     2. smx_gemv_dev          quantiser + down GEMV                                      h -> d[hidden]
-    3. smx_moe_router_dev    router logits + softmax + top-k                            d -> ids[k], w[k] (+ logits[ne])
+    3. smx_moe_router_dev    router logits GEMV, then softmax + top-k (two launches)    d -> ids[k], w[k] (+ logits[ne])
     4. smx_moe_ffn_routed_dev  the k routed experts' gate/up (one launch) and down (one launch)   d -> y[hidden]
 Attention, RoPE and the KV cache are outside this path.  The benchmark (bench.py) and the parity test
 (tests/test_gpu_chain.py) both run this class, so what is measured is what is checked.
@@ -19,10 +19,10 @@ class FfnMoeChain:
     otherwise the layers share one set (what a decode loop does)."""
 
     def __init__(self, acc, layers, hidden, ffn, ne, k, keys, moe_layer, norm_w_dev, eps=1e-6, keep_stages=False,
-                 fused_router=True):
+                 router_call=True):
         self.acc, self.layers, self.hidden, self.ffn, self.ne, self.k = acc, layers, hidden, ffn, ne, k
         self.keys, self.moe_layer, self.norm_w_dev, self.eps = keys, moe_layer, norm_w_dev, eps
-        self.fused_router = fused_router
+        self.router_call = router_call   # False: the router as smx_gemv_dev + smx_moe_route_dev (same launches, same bits)
         self._bufs = []
         nsets = layers if keep_stages else 1
         self.stage = []
@@ -51,7 +51,7 @@ class FfnMoeChain:
             gate, up, down, router = self.keys(l + layer_offset)
             ok = acc.ffn_gate_up_dev(gate, up, 2, cur, b["h"], norm=True, norm_w_dev=self.norm_w_dev, eps=self.eps)
             ok = ok and acc.gemv_dev(down, b["h"], 1, b["d"])
-            if self.fused_router:
+            if self.router_call:
                 ok = ok and acc.moe_router_dev(router, b["d"], self.k, b["ids"], b["w"], b["logits"])
             else:
                 ok = ok and acc.gemv_dev(router, b["d"], 1, b["logits"])
@@ -63,7 +63,7 @@ class FfnMoeChain:
         return cur
 
     def launches_per_token(self):
-        return self.layers * (5 if self.fused_router else 6)
+        return self.layers * 6
 
     def close(self):
         for p in self._bufs:

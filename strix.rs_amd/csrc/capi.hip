@@ -103,10 +103,9 @@ namespace smx {
 int run_matmul_dev(smx_ctx* c, const Weight& w, const float* xs_dev, size_t m, float* y_dev, bool force_gemm,
                    int32_t* dump, const ActScratch* sc) {
     const bool skinny = skinny_serves(w, m);
-    // Q6_K with 5..8 rows where the small-batch kernel does not serve (none today; kept for weights it declines): the dot4
-    // GEMV runs its 8-row variant there (35 us on 15360 x 3840, 440 us on a 262144-row head, LDS- and VALU-bound), the tiled
-    // GEMM, whose sparse tiles share their rows out over the waves, 29 / 290 us for any row count up to 32.
-    // (A caller that brings its own scratch keeps the GEMV: the GEMM sizes its scratch itself.)
+    // Q6_K with 5..8 rows of a weight the small-batch kernel declines (rows shorter than 128 elements): the tiled GEMM, whose
+    // sparse tiles share their rows out over the waves; a caller that brings its own scratch keeps the dot4 GEMV there (the
+    // GEMM sizes its scratch itself).
     const bool gemv_rows = m <= SMX_GEMV_MAX_M && (w.type != kQ6_K || m <= 4 || sc != nullptr);
     if (!skinny && gemv_rows && !force_gemm) return launch_gemv(c, w, xs_dev, m, y_dev, dump, sc);  // quantiser fused
     if (sc && !skinny) return fail(c, SMX_ERR_LIMIT, "%zu rows of this weight need the tiled GEMM, which sizes its scratch from the call", m);

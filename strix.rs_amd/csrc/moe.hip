@@ -187,30 +187,6 @@ __global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict
     topk_router_wave<PL>(v, ne, k, ids, w, sel);
 }
 
-// Router logits + routing in ONE launch (the reference's f32_gemv of the router weight followed by topk_router,
-// decode.rs:1136-1166): one 16-wave workgroup runs the flat GEMV over all ne rows of the (small) router weight -- 64 x 2048
-// Q8_0 is 139 KB -- writes the logits, and its first wave then routes them.  The logits have the bits of a separate GEMV
-// launch (a row's sum does not depend on how rows are shared out), the routing those of topk_router_kernel on them.
-template <class Ops, int PRE, int GL, int PL>
-__global__ __launch_bounds__(1024) void moe_router_fused_kernel(const GemvW W, const float* __restrict__ x, float* logits, int nblk,
-                                                                int ne, unsigned magic_u, int k, int* __restrict__ ids,
-                                                                float* __restrict__ w) {
-    extern __shared__ __align__(16) char router_smem[];
-    gemv_body_flat<Ops, 1, PRE, GL, 1>(W, GemvX{x, nullptr, nullptr, nullptr, nullptr, SMX_ACT_NONE, 0.f}, logits, ne, nblk, ne, 1, 0, 1,
-                                       magic_u);
-    __threadfence_block();   // the logits the other waves stored are read back by the first wave
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        float v[PL];
-#pragma unroll
-        for (int j = 0; j < PL; j++) {
-            const int e = (int)threadIdx.x + 64 * j;
-            v[j] = e < ne ? *(const volatile float*)(logits + e) : -3.40282347e+38f;
-        }
-        topk_router_wave<PL>(v, ne, k, ids, w, (float*)router_smem);
-    }
-}
-
 // Decode, second half, in one launch: a_k = quantised silu(g_k)*u_k is rebuilt in LDS by every
 // workgroup (k*eff elements; measured faster than a launch of its own), then each wave computes
 // output rows y[r] = sum_k w_k * sum_b dw*dx*I over the k routed experts' down-projection rows,
@@ -978,33 +954,11 @@ int smx_moe_router_dev(smx_ctx* c, const char* key, const float* x_dev, size_t k
             if ((rc = ensure(c, c->yf32, ne * 4)) != SMX_OK) return rc;
             logits_dev = (float*)c->yf32.p;
         }
-        // one workgroup serves the whole weight when its rows take the flat form and fit one workgroup's unit index and LDS
-        const size_t upb = w.type == kQ6_K ? 4 : (w.type == kQ8_0 ? 2 : 1);
-        const size_t units = w.nblk * upb;
-        const size_t tokb = w.type == kQ4_0 ? ((w.nblk * 40 + 15) & ~size_t(15))
-                                             : (w.type == kQ8_0 ? ((w.nblk * 36 + 15) & ~size_t(15)) : w.nblk * 2 * (OpsQ6_K::kPad * 16 + 32));
-        const int gl = (units % 16) == 0 ? 16 : ((units % 8) == 0 ? 8 : ((w.type == kQ6_K && (units % 4) == 0) ? 4 : 0));
-        const size_t lds = gl ? tokb + ne * units / gl * 4 : 0;
-        if (gl && w.K <= 16384 && ne <= 256 && ne * units < 65536 && lds <= 160 * 1024) {
-            const GemvW W = {w.scales, (const uint4*)w.quants, (const uint4*)w.qh, (const uint2*)w.sc};
-            const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);
-            ProfScope ps(c, "moe_router_fused");
-            auto go = [&](auto kern) -> int {
-                int rc2 = set_dyn_lds(c, kern, lds);
-                if (rc2 != SMX_OK) return rc2;
-                hipLaunchKernelGGL(kern, dim3(1), dim3(1024), lds, c->stream, W, x_dev, logits_dev, (int)w.nblk, (int)ne, magic, (int)k,
-                                   ids_dev, w_dev);
-                SMX_HIP(c, hipGetLastError());
-                return SMX_OK;
-            };
-#define SMX_ROUTER(OPS, PRE, GL) \
-    if (gl == GL) return ne <= 64 ? go(moe_router_fused_kernel<OPS, PRE, GL, 1>) : go(moe_router_fused_kernel<OPS, PRE, GL, 4>);
-            if (w.type == kQ4_0) { SMX_ROUTER(OpsQ4_0, 3, 16) SMX_ROUTER(OpsQ4_0, 3, 8) }
-            else if (w.type == kQ8_0) { SMX_ROUTER(OpsQ8_0, 3, 16) SMX_ROUTER(OpsQ8_0, 3, 8) }
-            else { SMX_ROUTER(OpsQ6_K, 1, 16) SMX_ROUTER(OpsQ6_K, 1, 8) SMX_ROUTER(OpsQ6_K, 1, 4) }
-#undef SMX_ROUTER
-        }
-        // other shapes: the two launches
+        // Two launches: the GEMV over all CUs (2.4 us back to back for a 64 x 2048 Q8_0 router, launch-bound) and the one-wave
+        // routing kernel (3.2 us).  ONE launch -- a single 16-wave workgroup running the flat GEMV over the whole router weight,
+        // then routing the logits it just stored -- was built and gave the same bits, but took 6.6-6.9 us against 5.7-5.9 us:
+        // on one CU the activation fetch, the 139 KB of weights, the row sums, the store and the routing run one after the
+        // other, and together they cost more than the second launch.
         if ((rc = launch_gemv(c, w, x_dev, 1, logits_dev, nullptr)) != SMX_OK) return rc;
         return smx_moe_route_dev(c, logits_dev, ne, k, ids_dev, w_dev);
     });

@@ -58,9 +58,10 @@ extern "C" int smx_gemv_noalloc_dev(smx_ctx* c, const char* key, const float* xs
     if (!w) return SMX_NOT_RESIDENT;
     if (m == 0 || m > kNoallocMaxRows)
         return fail(c, SMX_ERR_LIMIT, "gemv_noalloc_dev: %zu rows (1..%zu supported)", m, kNoallocMaxRows);
-    if (w->K > kNoallocMaxK)
-        return fail(c, SMX_ERR_LIMIT, "gemv_noalloc_dev: in_dim %zu exceeds the static scratch (rows of at most %zu elements)",
-                    w->K, kNoallocMaxK);
+    // one row is quantised inside the GEMV's staging and never touches the scratch: rows of any length the GEMV serves
+    if (m >= 2 && w->K > kNoallocMaxK)
+        return fail(c, SMX_ERR_LIMIT, "gemv_noalloc_dev: in_dim %zu exceeds the static scratch (%zu rows of at most %zu elements)",
+                    w->K, m, kNoallocMaxK);
     if (!c->static_scratch) return fail(c, SMX_ERR_HIP, "gemv_noalloc_dev: the static scratch was not located on device %d", c->device);
     unsigned char* base = (unsigned char*)c->static_scratch;   // the device pointer, never the array's name
     const ActScratch sc = {(int8_t*)base, (float*)(base + kScratchQ), (int32_t*)(base + kScratchQ + kScratchD)};

@@ -1,6 +1,6 @@
 """The decode chain that bench.py times (strix.rs_amd/chain.py: per layer rmsnorm + gate/up + SwiGLU product, down GEMV,
-fused router, routed expert FFN; the reference's captured token, decode.rs:3053-3203) against the oracle, stage by stage,
-eager and as a replayed graph, and the fused router launch on its own."""
+router, routed expert FFN; the reference's captured token, decode.rs:3053-3203) against the oracle, stage by stage,
+eager and as a replayed graph, and the router call on its own."""
 import importlib.util
 import os
 import sys
@@ -44,10 +44,9 @@ def _read(accel, ptr, n, dtype=np.float32):
 
 @pytest.mark.parametrize("ty,ne,K,k", [(8, 64, 2048, 8), (8, 16, 512, 4), (2, 64, 1024, 8), (14, 64, 2048, 6), (8, 200, 512, 5),
                                        (8, 300, 256, 3), (8, 33, 4128, 4), (8, 64, 32768, 2)])
-def test_fused_router_equals_gemv_then_route(accel, orc, synth, relerr, ty, ne, K, k):
+def test_router_call_equals_gemv_then_route(accel, orc, synth, relerr, ty, ne, K, k):
     """smx_moe_router_dev: logits with the bits of smx_gemv_dev, routing with the bits of smx_moe_route_dev on them, experts
-    as the oracle routes the oracle-checked logits.  Shapes: one workgroup (up to 256 experts, flat-form rows) and the
-    two-launch route (300 experts; rows of 4128 and 32768 elements)."""
+    as the oracle routes the oracle-checked logits; all three formats, 16..300 experts, flat-form and other row lengths."""
     raw = _router_weight(synth, ty, ne, K, ne + K, 0.05 if ty != 14 else 0.1)
     assert {2: accel.upload_q4_0, 8: accel.upload_q8_0, 14: accel.upload_q6_k}[ty]("t.router", raw, K, ne)
     xd, ld, l2 = accel.dev_alloc(K * 4), accel.dev_alloc(ne * 4), accel.dev_alloc(ne * 4)
@@ -96,7 +95,7 @@ def test_decode_chain_stage_by_stage_eager_and_replayed(accel, orc, synth, reler
     accel.h2d(nwd, nw)
     ch = chain_mod.FfnMoeChain(accel, layers, H, F, ne, k, lambda l: tuple(f"t.ch.{t}{l}" for t in "gudr"), lambda l: base + l,
                                nwd, eps=1e-6, keep_stages=True)
-    assert ch.launches_per_token() == 10
+    assert ch.launches_per_token() == 12
     toks = synth.make_acts(4, H, seed=77) * np.float32(1.5)
 
     def run_eager(x):
@@ -151,9 +150,9 @@ def test_decode_chain_stage_by_stage_eager_and_replayed(accel, orc, synth, reler
         assert np.array_equal(_read(accel, out, H), want[t]), f"replay of token {t}"
     accel.graph_destroy(g)
 
-    # the chain with the router as two launches gives the same bits
+    # the chain with the router as two calls gives the same bits
     ch2 = chain_mod.FfnMoeChain(accel, layers, H, F, ne, k, lambda l: tuple(f"t.ch.{t}{l}" for t in "gudr"), lambda l: base + l,
-                                nwd, eps=1e-6, fused_router=False)
+                                nwd, eps=1e-6, router_call=False)
     accel.h2d(xd, toks[3])
     out2 = ch2.enqueue(xd)
     accel.sync()
