@@ -566,6 +566,9 @@ int smx_tune(smx_ctx* c, const char* knob, int value) {
     } else if (k == "gemm_tile_m") {
         if (value != 0 && value != 64 && value != 128) return fail(c, SMX_ERR_ARG, "tune: gemm_tile_m must be 0, 64 or 128");
         c->tune_gemm_tile_m = value;
+    } else if (k == "gemm_walk") {
+        if (value > 64) return fail(c, SMX_ERR_ARG, "tune: gemm_walk must be 0..64");
+        c->tune_gemm_walk = value;   // token-tile groups of the GEMM's tile walk (0: chosen from the L2 size)
     } else {
         return fail(c, SMX_ERR_ARG, "tune: unknown knob %s", knob);
     }

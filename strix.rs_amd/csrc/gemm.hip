@@ -81,7 +81,10 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     } else {
         const int T = p.tiles_m * p.tiles_n;
         if (p.xcd_remap) t = (t & 7) * (T >> 3) + (t >> 3);
-        const int tm = t % p.tiles_m, tn = t / p.tiles_m;
+        // logical order: token-tile group (walk_gm token tiles), weight strip, token tile inside the group
+        const int per_group = p.walk_gm * p.tiles_n;
+        const int grp = t / per_group, in_grp = t - grp * per_group;
+        const int tn = in_grp / p.walk_gm, tm = grp * p.walk_gm + (in_grp - tn * p.walk_gm);
         tok0 = tm * p.tile_m; row0 = tn * BN; col0 = row0; M_end = min(p.M, tok0 + p.tile_m); N_end = p.N;
     }
     const GemmOperand op = p.op[op_i];
@@ -491,6 +494,19 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     p.tiles_m = (p.M + bm - 1) / bm;
     const int T = p.tiles_m * p.tiles_n;
     p.xcd_remap = (T % 8 == 0) ? 1 : 0;
+    // Tile walk.  Workgroup t runs on XCD t % 8 and each XCD gets a contiguous eighth of the logical tile order, so the order
+    // decides which operand bytes an XCD's 4 MB L2 must see.  Token tiles are taken in groups of walk_gm (up to 8): an XCD then
+    // works on walk_gm token tiles x (tiles_n * tiles_m / walk_gm / 8) weight strips instead of all token tiles x an eighth of
+    // the strips, whose activations (7.9 MB at M = 2048, K = 3840) it fetched again for every strip.  Measured L2 fills per
+    // launch at M = 2048 (rocprofv3 FETCH_SIZE, Q8_0): K 3840 x N 15360 540 -> 341 MB, K 15360 x N 3840 580 -> 366 MB with groups
+    // of 8; groups of 4: 360 / 363 MB; of 1 (ffn_down): 947 MB.  The launch time does not move (the kernel is bound by
+    // instruction issue, and these fetches are served by the Infinity Cache).
+    {
+        int gm = std::min(p.tiles_m, 8);
+        if (c->tune_gemm_walk > 0) gm = std::max(1, p.tiles_m / c->tune_gemm_walk);
+        while (p.tiles_m % gm != 0) gm--;   // whole groups
+        p.walk_gm = gm;
+    }
     const int nstages = (p.nb + KB - 1) / KB;
     int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(slots, T, nstages));
     p.stages_per_slice = (nstages + Z - 1) / Z;

@@ -384,9 +384,9 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
     J.job[0].x = x;
     J.job[0].y = y;
     J.job[0].N = (int)w.N;
-    // 2..4 rows of at most 32768 values in all: the flat kernel quantises them itself (one or two half blocks per thread), which
+    // 2..4 rows of at most 49152 values in all: the flat kernel quantises them itself (up to three half blocks per thread), which
     // saves the quantiser launch; longer rows are quantised once for all workgroups by their own launch
-    g.rowsf = mt > 1 && mt <= 4 && g.flat && !dump && (size_t)mt * w.K <= 32768;
+    g.rowsf = mt > 1 && mt <= 4 && g.flat && !dump && (size_t)mt * w.K <= 49152;
     if (mt > 1 && !g.rowsf) {
         // each of the persistent workgroups would repeat the quantiser for all m rows: do it once instead
         int rc;

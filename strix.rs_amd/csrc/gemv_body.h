@@ -812,19 +812,20 @@ struct FlatXRows {
 };
 
 // The same for up to MT fp32 rows that are quantised here (FQ = 1 with MT > 1): item i = half block i % hb of row i / hb,
-// hb = half blocks per row; a thread takes items threadIdx.x and threadIdx.x + 1024, MT * hb <= 2048 (the launcher's
-// bound: 32768 values in all, e.g. 4 rows of up to 8192 elements).  Saves the quantiser launch in front of a 2..4-row
-// GEMV (2.5 of the 7.6 us Q4_0 9728 x 2560 takes at 2 rows).
+// hb = half blocks per row; a thread takes items threadIdx.x, threadIdx.x + 1024 and threadIdx.x + 2048, MT * hb <= 3072 (the
+// launcher's bound: 49152 values in all, e.g. 4 rows of up to 12288 elements).  Saves the quantiser launch in front of a
+// 2..4-row GEMV (2.5 of the 7.6 us Q4_0 9728 x 2560 takes at 2 rows).
 template <class Ops, int MT>
 struct FlatXRowsF {
     static_assert(MT <= 4, "row = number of row boundaries at or below the item index");
-    float4 v[2][4];
-    int t[2], h[2];
+    static constexpr int NP = 3;   // items per thread
+    float4 v[NP][4];
+    int t[NP], h[NP];
 
     __device__ __forceinline__ void request(const GemvX& X, int nblk, int m) {
         const int hb = Ops::nb32(nblk) * 2;
 #pragma unroll
-        for (int p = 0; p < 2; p++) {
+        for (int p = 0; p < NP; p++) {
             const int i = threadIdx.x + p * 1024;
             t[p] = (i >= hb ? 1 : 0) + (i >= 2 * hb ? 1 : 0) + (i >= 3 * hb ? 1 : 0);
             h[p] = i - t[p] * hb;
@@ -839,7 +840,7 @@ struct FlatXRowsF {
     __device__ __forceinline__ void store(char* smem, int tokb, int nblk) {
         const int hb = Ops::nb32(nblk) * 2;
 #pragma unroll
-        for (int p = 0; p < 2; p++) {
+        for (int p = 0; p < NP; p++) {
             const int i = threadIdx.x + p * 1024;
             if ((i & ~63) >= MT * hb) return;   // whole waves
             quantize_half_block<Ops>(smem + min(t[p], MT - 1) * tokb, nblk, h[p], i < MT * hb, v[p]);

@@ -56,8 +56,9 @@ struct SkinnyArgs {
     const float* xd;          // [pieces][tslots][4]: the four block scales of a piece side by side per token slot
     float* y;                 // [m][N]
     int* dump;                // optional [m][N][nb] i32 block dots (Q6_K: [m][N][2 nb] sub-block dots)
+    size_t xq_tile, xd_tile;  // two token tiles (33..64 rows): bytes from tile 0's quants to tile 1's, floats between their scales
     int m, N, nb;
-    int tslots;               // token slots of the fragment-ordered activations: 8, 16 or 32
+    int tslots;               // token slots of the fragment-ordered activations: 8, 16 or 32 (per token tile)
     int ksplit;               // K slices per row group (1 or 2)
     int pieces_per_slice;     // 4-block pieces in a slice
     int rows_per_group;       // weight rows a workgroup owns (<= 32): chosen so that the workgroups fill whole rounds of CUs
@@ -67,7 +68,7 @@ __device__ __forceinline__ float h2f_s(uint16_t h) { return __half2float(__ushor
 __device__ __forceinline__ unsigned sub8s(unsigned x) { return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u; }
 
 #define SMX_SK_FMAC(I)                                                                      \
-    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I " row_mask:0xf bank_mask:0xf" : "+v"(acc[I]) : "v"(dxv), "v"(t[I]))
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:" #I " row_mask:0xf bank_mask:0xf" : "+v"(av[I]) : "v"(dxv), "v"(t[I]))
 
 // 64 lanes x 16 bytes from global memory straight into LDS (no register round trip): lane i's bytes land at
 // LDS byte address lds_base + 16 * i; lds_base is wave-uniform (M0).  Completion is counted by vmcnt.
@@ -100,6 +101,8 @@ struct PieceRegs {
     uint2 dw;              // four f16 scales of this lane's weight row; Q6_K: the eight int8 sub-block scales of the piece
     uint16_t d6;           // Q6_K: d of the row's superblock
     uint4 dx;              // four f32 scales (one per block) of the token whose accumulators this lane feeds by row broadcast
+    v4i c0, c1, c2, c3;    // second token tile (33..64 rows): its fragments ...
+    uint4 dx1;             // ... and scales
 };
 // vector-memory loads per piece: 6 that return into registers, then up to 4 (Q8_0: 8 rows x 128 B each)
 // or 2 (Q4_0: 16 rows x 64 B of nibbles each) LDS-direct ones
@@ -115,10 +118,14 @@ struct PieceRegs {
 // NACC: accumulators per lane that hold live tokens (accumulator i of lane half h is token (i / 4) * 8 + 4 h + i % 4: 4 for up
 // to 8 token slots, 8 for 16); only those are rescaled -- with all 16 the Q6_K variant would be bound by its vector ALU work,
 // and Q4_0 9728 x 2560 takes 1.3 us longer at 5..16 rows.
-template <int FMT, bool DUMP, int NW, bool ALDS, int NACC = 16>
+// TT = 2 (33..64 rows of a Q8_0 / Q4_0 weight): two 32-token tiles share every weight piece -- two MFMAs per block on the same
+// weight fragment, 32 accumulators per lane -- so the weight is still read once (the tiled GEMM takes 22 us where 32 rows
+// take 14: 128-row strips leave it 20 tiles to split over K, and a reduction launch behind them).
+template <int FMT, bool DUMP, int NW, bool ALDS, int NACC = 16, int TT = 1>
 __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
     constexpr bool Q4 = FMT == FMT_Q4, Q6 = FMT == FMT_Q6;
     static_assert(!Q6 || ALDS, "the Q6_K variant reads its activation fragments from LDS");
+    static_assert(TT == 1 || (!ALDS && !Q6 && NACC == 16), "two token tiles: fragments through registers, all accumulators live");
     constexpr int kWaves = NW;
     constexpr int kWaveLds = wave_lds(FMT, ALDS);
     extern __shared__ __align__(16) char smem[];
@@ -138,9 +145,13 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
 
     // loop-invariant lane roles
     const int wrow = min(r0 + col, r_last);                         // this lane's weight row (MFMA operand and scales)
-    const int atok = min(col, p.m - 1);                             // this lane's token as the other MFMA operand
+    const int m0 = TT == 2 ? 32 : p.m, m1 = p.m - 32;                // rows of the first / second token tile
+    const int atok = min(col, m0 - 1);                              // this lane's token as the other MFMA operand
+    const int atok1 = min(col, max(m1, 1) - 1);
     const int nrows = r_last - r0 + 1;                              // rows of this group: load instructions past them are not issued
-    const int dx_tok = min(((lane & 15) >> 2) * 8 + half * 4 + (lane & 3), p.m - 1);   // token of accumulator lane % 16 in this lane half
+    const int dx_slot = ((lane & 15) >> 2) * 8 + half * 4 + (lane & 3);
+    const int dx_tok = min(dx_slot, m0 - 1);   // token of accumulator lane % 16 in this lane half
+    const int dx_tok1 = min(dx_slot, max(m1, 1) - 1);
     const bool vec_sc = (p.nb & 3) == 0;
     // Q8_0 landing: lane = [row:3][slot:3] of an 8-row group; the lane fetches chunk (slot - row) % 8 of its row, so
     // chunk c of row r sits in slot (c + r) % 8 and the transposed fragment reads spread over the banks
@@ -161,9 +172,16 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
                 return *(const v4i*)(p.xq + ((size_t)(min(blk0 + bi, p.nb - 1) * 2 + half) * p.tslots + atok) * 16);
             };
             r.a0 = la(0); r.a1 = la(1); r.a2 = la(2); r.a3 = la(3);
+            if constexpr (TT == 2) {
+                auto lc = [&](int bi) {
+                    return *(const v4i*)(p.xq + p.xq_tile + ((size_t)(min(blk0 + bi, p.nb - 1) * 2 + half) * p.tslots + atok1) * 16);
+                };
+                r.c0 = lc(0); r.c1 = lc(1); r.c2 = lc(2); r.c3 = lc(3);
+            }
         }
         const uint16_t* ws = p.wscales + (size_t)wrow * p.nb;
         r.dx = *(const uint4*)(p.xd + ((size_t)piece * p.tslots + dx_tok) * 4);   // 16 contiguous bytes per token slot
+        if constexpr (TT == 2) r.dx1 = *(const uint4*)(p.xd + p.xd_tile + ((size_t)piece * p.tslots + dx_tok1) * 4);
         r.d6 = 0;
         if (Q6) {
             const size_t sb = (size_t)wrow * (p.nb >> 3) + (piece >> 1);
@@ -203,9 +221,11 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         return r;
     };
 
-    float acc[16];
+    float acc[16], acc1[TT == 2 ? 16 : 1];
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < (TT == 2 ? 16 : 1); i++) acc1[i] = 0.f;
     v16i cmagic;
 #pragma unroll
     for (int i = 0; i < 16; i++) cmagic[i] = kMagicI;
@@ -261,7 +281,7 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         const unsigned dwh[4] = {r.dw.x & 0xffffu, r.dw.x >> 16, r.dw.y & 0xffffu, r.dw.y >> 16};
         const unsigned dxs[4] = {r.dx.x, r.dx.y, r.dx.z, r.dx.w};
         // acc[i] += dx(token of accumulator i) * fl(dw * I) for the live accumulators, I the exact i32 of MFMA result d
-        auto rescale = [&](const v16i& d, float dw, float dxv) {
+        auto rescale = [&](float (&av)[16], const v16i& d, float dw, float dxv) {
             const float ndw = -dw * kMagicF;   // exact: dw has at most 18 significant bits (f16, or f16 x int8)
             float t[16];
 #pragma unroll
@@ -289,7 +309,7 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
                     // d * sc, exact in fp32 (11 x 8 significant bits): sc + 128 as an unsigned byte -> float, then one FMA
                     const unsigned scw = ((2 * bi + jj) < 4 ? r.dw.x : r.dw.y) ^ 0x80808080u;
                     const float dw = fmaf((float)((scw >> (8 * ((2 * bi + jj) & 3))) & 0xffu), d6, d6m128);
-                    rescale(d, dw, dxv);
+                    rescale(acc, d, dw, dxv);
                     if (DUMP) {
                         const int row = r0 + col;
 #pragma unroll
@@ -305,13 +325,27 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
                                        : (bi == 0 ? r.a0 : (bi == 1 ? r.a1 : (bi == 2 ? r.a2 : r.a3)));
                 const v16i d = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, bfrag, cmagic, 0, 0, 0);
                 const float dw = live ? h2f_s((uint16_t)dwh[bi]) : 0.f;
-                rescale(d, dw, dxv);
+                rescale(acc, d, dw, dxv);
                 if (DUMP) {
                     const int row = r0 + col;
 #pragma unroll
                     for (int i = 0; i < NACC; i++) {
                         const int tok = (i >> 2) * 8 + half * 4 + (i & 3);
                         if (live && tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d[i] - kMagicI;
+                    }
+                }
+                if constexpr (TT == 2) {   // the second token tile on the same weight fragment
+                    const v4i cfrag = bi == 0 ? r.c0 : (bi == 1 ? r.c1 : (bi == 2 ? r.c2 : r.c3));
+                    const v16i d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(cfrag, bfrag, cmagic, 0, 0, 0);
+                    const unsigned dxs1[4] = {r.dx1.x, r.dx1.y, r.dx1.z, r.dx1.w};
+                    rescale(acc1, d1, dw, __uint_as_float(dxs1[bi]));
+                    if (DUMP) {
+                        const int row = r0 + col;
+#pragma unroll
+                        for (int i = 0; i < 16; i++) {
+                            const int tok = 32 + (i >> 2) * 8 + half * 4 + (i & 3);
+                            if (live && tok < p.m && row <= r_last) p.dump[((size_t)tok * p.N + row) * p.nb + blk0 + bi] = d1[i] - kMagicI;
+                        }
                     }
                 }
             }
@@ -331,22 +365,26 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
         for (int pc = pc0; pc < my_end; pc++) consume(request(pc), pc);
     }
 
-    // the waves' partial tiles, added in wave order
-    __syncthreads();
+    // the waves' partial tiles, added in wave order (one token tile after the other through the same LDS)
     float* red = (float*)smem;   // [wave][16][64]
 #pragma unroll
-    for (int i = 0; i < NACC; i++) red[(wave * 16 + i) * 64 + lane] = acc[i];
-    __syncthreads();
+    for (int tile = 0; tile < TT; tile++) {
+        __syncthreads();
+        const float* av = (TT == 2 && tile == 1) ? acc1 : acc;
 #pragma unroll
-    for (int i = wave; i < NACC; i += kWaves) {   // accumulator index; lane as above
-        float s = 0.f;
+        for (int i = 0; i < NACC; i++) red[(wave * 16 + i) * 64 + lane] = av[i];
+        __syncthreads();
 #pragma unroll
-        for (int w = 0; w < kWaves; w++) s += red[(w * 16 + i) * 64 + lane];
-        const int tok = (i >> 2) * 8 + half * 4 + (i & 3), row = r0 + col;
-        if (tok < p.m && row <= r_last) {
-            float* o = p.y + (size_t)tok * p.N + row;
-            if (p.ksplit == 1) *o = s;
-            else atomicAdd(o, s);   // two addends onto a zeroed output: the sum does not depend on their order
+        for (int i = wave; i < NACC; i += kWaves) {   // accumulator index; lane as above
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < kWaves; w++) s += red[(w * 16 + i) * 64 + lane];
+            const int tok = tile * 32 + (i >> 2) * 8 + half * 4 + (i & 3), row = r0 + col;
+            if (tok < p.m && row <= r_last) {
+                float* o = p.y + (size_t)tok * p.N + row;
+                if (p.ksplit == 1) *o = s;
+                else atomicAdd(o, s);   // two addends onto a zeroed output: the sum does not depend on their order
+            }
         }
     }
 }
@@ -360,18 +398,23 @@ __global__ __launch_bounds__(64 * NW) void skinny_kernel(const SkinnyArgs p) {
 // scales go out as [piece = b / 4][token slot][b % 4].  The same launch zeroes the output when two K slices are going to add into it.
 __global__ __launch_bounds__(256) void skinny_quant_kernel(const float* __restrict__ x, int m, int nb, int tslots,
                                                            uint4* __restrict__ xq, float* __restrict__ xd,
-                                                           float4* __restrict__ zero, size_t zero_n4) {
+                                                           float4* __restrict__ zero, size_t zero_n4, size_t xq_tile16,
+                                                           size_t xd_tile) {
     const size_t gid = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (gid < zero_n4) zero[gid] = make_float4(0.f, 0.f, 0.f, 0.f);
+    const int tile = blockIdx.y;   // token tile: rows 32 * tile .. (its quants xq_tile16 chunks, its scales xd_tile floats further on)
+    if (tile == 0 && gid < zero_n4) zero[gid] = make_float4(0.f, 0.f, 0.f, 0.f);
+    xq += tile * xq_tile16;
+    xd += tile * xd_tile;
     const size_t nchunks = (size_t)nb * 2 * tslots;
     const int t = (int)(gid % tslots), h = (int)((gid / tslots) & 1);
     const size_t b = gid / (2 * (size_t)tslots);
-    const bool live = gid < nchunks && t < m;
+    const int row = tile * 32 + t;
+    const bool live = gid < nchunks && row < m;
     float v[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) v[i] = 0.f;
     if (live) {
-        const float4* src = (const float4*)(x + ((size_t)t * nb + b) * 32 + h * 16);
+        const float4* src = (const float4*)(x + ((size_t)row * nb + b) * 32 + h * 16);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const float4 f = src[i];
@@ -411,11 +454,13 @@ bool skinny_serves(const Weight& w, size_t m) {
     // 58.3 / 61.8, at 8 rows the dot4 GEMV 68.2 / 57.6 us; 262144 x 2560: 174.5 / 169.6, 159.2 / 155.5, 171.6 / 139.0 us)
     if (m < SMX_SKINNY_MIN_M || m > SMX_SKINNY_MAX_M || w.K < 128) return false;
     if (w.type == kQ6_K) return m <= 16;   // its activation fragments travel through LDS: up to 16 token slots
+    // 33..64 rows: two token tiles per weight piece
     return (w.type == kQ8_0 || w.type == kQ4_0) && (m <= 16 || w.N <= 32768);
 }
 
-size_t skinny_xq_bytes(size_t m, size_t K) { return (K / 32) * 2 * (m <= 8 ? 8 : (m <= 16 ? 16 : 32)) * 16; }
-size_t skinny_xd_bytes(size_t m, size_t K) { return ((K / 32 + 3) / 4) * (m <= 8 ? 8 : (m <= 16 ? 16 : 32)) * 16; }
+static size_t skinny_slots(size_t m) { return m <= 8 ? 8 : (m <= 16 ? 16 : (m <= 32 ? 32 : 64)); }   // 64: two tiles of 32
+size_t skinny_xq_bytes(size_t m, size_t K) { return (K / 32) * 2 * skinny_slots(m) * 16; }
+size_t skinny_xd_bytes(size_t m, size_t K) { return ((K / 32 + 3) / 4) * skinny_slots(m) * 16; }
 
 // y[m][N] for m <= 32 fp32 rows x[m][K]: quantiser launch (fragment-ordered quants into sc.xq, skinny_xq_bytes(m, K)
 // bytes; scales into sc.xd) and the matmul launch.  dump (optional): out[m][N][K/32].
@@ -437,6 +482,9 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
     p.nb = (int)(w.K / 32);   // 32-blocks per row in every format
     p.tslots = m <= 8 ? 8 : (m <= 16 ? 16 : 32);
     const int npieces = (p.nb + 3) / 4;
+    const int ntiles = m > 32 ? 2 : 1;   // token tiles
+    p.xq_tile = (size_t)p.nb * 2 * 32 * 16;
+    p.xd_tile = (size_t)npieces * 32 * 4;
     // Rows per workgroup and K slices: one workgroup per CU, so the launch takes ceil(workgroups / CUs) rounds.  Two K
     // slices when a single round of 32-row groups would leave CUs without work (and every wave still gets a piece);
     // then as few rows per group as keep the number of rounds (a last round of a few 32-row workgroups costs
@@ -457,13 +505,13 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
         const size_t threads = (size_t)p.nb * 2 * p.tslots, zero_n4 = ksplit > 1 ? m * w.N / 4 : 0;
         const size_t grid = (std::max(threads, zero_n4) + 255) / 256;
         ProfScope ps(c, "skinny_quant");
-        hipLaunchKernelGGL(skinny_quant_kernel, dim3((unsigned)grid), dim3(256), 0, c->stream, x, (int)m, p.nb, p.tslots,
-                           (uint4*)sc.xq, sc.xd, (float4*)y, zero_n4);
+        hipLaunchKernelGGL(skinny_quant_kernel, dim3((unsigned)grid, (unsigned)ntiles), dim3(256), 0, c->stream, x, (int)m, p.nb, p.tslots,
+                           (uint4*)sc.xq, sc.xd, (float4*)y, zero_n4, p.xq_tile / 16, p.xd_tile);
         SMX_HIP(c, hipGetLastError());
     }
     const int fmt = w.type == kQ4_0 ? FMT_Q4 : (w.type == kQ6_K ? FMT_Q6 : FMT_Q8);
     const int nwg = nrg * ksplit;
-    const int nw = nwg <= c->num_cu ? 16 : 8;   // waves per workgroup (see the kernel)
+    const int nw = (nwg <= c->num_cu && ntiles == 1) ? 16 : 8;   // waves per workgroup (see the kernel; two token tiles: 32 more accumulators per lane)
     const bool alds = p.tslots <= 16;
     const size_t lds = (size_t)nw * wave_lds(fmt, alds);   // the reduction reuses the first nw * 4 KB
     const dim3 grid((unsigned)nwg);
@@ -483,6 +531,10 @@ int launch_skinny(smx_ctx* c, const Weight& w, const float* x, size_t m, float* 
     // live accumulators per lane: 4 with up to 8 token slots, 8 with 16, all 16 with 32
 #define SMX_SK_ROWS(F_, NW_)                                                                      \
     (p.tslots == 8 ? SMX_SK_GO(F_, NW_, true, 4) : (p.tslots == 16 ? SMX_SK_GO(F_, NW_, true, 8) : SMX_SK_GO(F_, NW_, false, 16)))
+    if (ntiles == 2) {
+        if (fmt == FMT_Q4) return dump ? go(skinny_kernel<FMT_Q4, true, 8, false, 16, 2>) : go(skinny_kernel<FMT_Q4, false, 8, false, 16, 2>);
+        return dump ? go(skinny_kernel<FMT_Q8, true, 8, false, 16, 2>) : go(skinny_kernel<FMT_Q8, false, 8, false, 16, 2>);
+    }
     if (nw == 16) return fmt == FMT_Q4 ? SMX_SK_ROWS(FMT_Q4, 16) : SMX_SK_ROWS(FMT_Q8, 16);
     return fmt == FMT_Q4 ? SMX_SK_ROWS(FMT_Q4, 8) : SMX_SK_ROWS(FMT_Q8, 8);
 #undef SMX_SK_ROWS

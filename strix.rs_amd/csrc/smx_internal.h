@@ -79,7 +79,7 @@ struct smx_ctx {
     hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
 
     // tuning overrides (0 = automatic)
-    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_tile_m = 0;
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_tile_m = 0, tune_gemm_walk = 0;
 
     // dynamic-LDS limit already raised on this context's device, per kernel (see set_dyn_lds): a fixed
     // open-addressing table, so that a launch never allocates host memory
@@ -194,6 +194,7 @@ struct GemmArgs {
     int tile_m;             // dense tiling: tokens per tile, 128 or 64 (a 64-token tile's waves pair up on two row tiles each)
     int stages_per_slice;   // stages (of 4 blocks) each grid.z slice covers
     int xcd_remap;
+    int walk_gm;            // dense tiling: token tiles per group of the tile walk (see launch_gemm)
     int nops;               // grouped launches: operands per tile (workgroup x serves tile x / nops, operand x % nops)
 };
 
@@ -257,7 +258,7 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
 
 // Small-batch matmul on the matrix cores (skinny.hip): m <= SMX_SKINNY_MAX_M fp32 rows against a Q8_0 / Q4_0
 // weight read once (its own quantiser launch + the matmul launch).  dump (optional): out[m][N][K/32] i32.
-#define SMX_SKINNY_MAX_M 32
+#define SMX_SKINNY_MAX_M 64
 #define SMX_SKINNY_MIN_M 5
 bool skinny_serves(const Weight& w, size_t m);
 // bytes of sc.xq the call needs (quants in MFMA fragment order, 8, 16 or 32 token slots)

@@ -151,11 +151,13 @@ def test_gemv_rows_q6k(accel, orc, synth, relerr, m):
 
 
 @pytest.mark.parametrize("ty,N,K", [(2, 130, 256), (8, 96, 4096), (14, 200, 4096), (2, 64, 4128), (8, 300, 8192), (14, 40, 8192), (2, 9728, 2560),
-                                    (8, 2560, 9728), (2, 77, 16384), (14, 33, 10240), (8, 50, 8224), (2, 40, 16416)])
+                                    (8, 2560, 9728), (2, 77, 16384), (14, 33, 10240), (8, 50, 8224), (2, 40, 16416), (8, 90, 12288),
+                                    (2, 70, 12320), (14, 35, 12288), (8, 64, 10240)])
 def test_gemv_rows_quantised_in_kernel(accel, orc, synth, relerr, ty, N, K):
-    # 2..4 fp32 rows of at most 32768 values in all (counting 4 rows for 3) are quantised by the GEMV kernel itself, one or
-    # two half blocks per thread; longer ones by a quantiser launch of their own: both sides of the bound (8192 / 8224 and
-    # 16384 / 16416 elements per row), a row of eight blocks, three rows in the four-row variant (its fourth row is staged as zeros)
+    # 2..4 fp32 rows of at most 49152 values in all (counting 4 rows for 3) are quantised by the GEMV kernel itself, one to
+    # three half blocks per thread; longer ones by a quantiser launch of their own: both sides of the bound (12288 / 12320
+    # elements per row at 4 rows, 16384 / 16416 at 2), one, two and three items per thread (4096, 8192, 9728..12288 elements
+    # at 4 rows), a row of eight blocks, three rows in the four-row variant (its fourth row is staged as zeros)
     raw = synth.make_weight(ty, N, K, seed=N + K)
     _up(accel, ty, "t.rq", raw, K, N)
     for m in (2, 3, 4):
