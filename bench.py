@@ -114,6 +114,8 @@ def machine_floors(log):
     out["mfma_plus_rescale_fma"] = f.mfma_valu(2, 4, 2)
     out["mfma_plus_rescale_fma_plus_lds_fragment_reads"] = f.mfma_valu(3, 4, 2)
     out["mfma_plus_rescale_fma_three_waves_per_simd"] = f.mfma_valu(2, 4, 3)
+    # Q6_K: two K = 16 MFMAs per 32-block and row tile, each with its own weight scale: four vector operations per output
+    out["mfma_plus_rescale_fma_q6_k"] = f.mfma_valu(6, 4, 2)
     out["note"] = ("mfma_only runs at the clock the chip sustains under matrix load; with the two FMAs per output that exact "
                    "per-block rescaling needs, the vector ALU bounds the rate: mfma_plus_rescale_fma is the ceiling of this arithmetic")
     log(json.dumps(out))
@@ -731,6 +733,12 @@ def main():
             r = fn()
             work[name] = r
             b.log(json.dumps(r))
+    if floors:   # every GEMM against the measured ceiling of its own arithmetic (MFMA + the rescale operations its format needs)
+        for n, w in work.items():
+            if n.startswith("gemm_") and "kernel_TOPS" in w:
+                ceil = floors["mfma_plus_rescale_fma_q6_k" if "q6_k" in n else "mfma_plus_rescale_fma"]["TOPS"]
+                w["rescale_ceiling_TOPS"], w["kernel_over_ceiling"] = ceil, w["kernel_TOPS"] / ceil
+                b.log(f"{n}: kernel {w['kernel_TOPS']:.0f} TOPS = {w['kernel_over_ceiling']:.2f} of its arithmetic's ceiling ({ceil:.0f} TOPS)")
     if head is None:  # sweep mode: per-workload records only, no headline line
         print(json.dumps({"workloads": work}), flush=True)
         return

@@ -140,12 +140,12 @@ __global__ __launch_bounds__(256, OCC) void mfma_valu_kernel(const float* __rest
     const int dx_tok = ((lane & 15) >> 2) * 8 + half * 4 + (lane & 3);
     const v4i* ag = aglob + ((size_t)(blockIdx.x * 4 + wave) * 64) * 64 + lane;   // 64 blocks of 1 KB per wave, reused
     v4i fa_next = fa;
-    if (MODE >= 4) fa_next = ag[0];
+    if (MODE == 4 || MODE == 5) fa_next = ag[0];
     for (int b = 0; b < nblocks; b++) {
         const int bs = b & 15;
         float dxr[16], dw[NT];
         float dxv = 0.f;
-        if (MODE != 0) {
+        if (MODE != 0 && MODE != 6) {
             if (MODE == 4) {
                 dxv = sdx[bs * 128 + wave * 32 + dx_tok];
             } else {
@@ -157,6 +157,40 @@ __global__ __launch_bounds__(256, OCC) void mfma_valu_kernel(const float* __rest
             }
 #pragma unroll
             for (int nt = 0; nt < NT; nt++) dw[nt] = sdw[bs * 128 + nt * 32 + col];
+        }
+        if constexpr (MODE == 6) {
+            // Q6_K arithmetic: the format scales 16-element sub-blocks, so a 32-block of a row tile is two K = 16 MFMAs, each
+            // rescaled by its own weight scale: four vector operations per output per 32-block (the activation scale through a
+            // DPP row broadcast, as the Q6_K GEMM reads it)
+            dxv = sdx[bs * 128 + wave * 32 + dx_tok];
+            float dw2[NT];
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                dw[nt] = sdw[bs * 128 + nt * 32 + col];
+                dw2[nt] = sdw[((bs + 1) & 15) * 128 + nt * 32 + col];
+            }
+            auto unit = [&](int v) -> v16i {
+                const int nt = v >> 1, jj = v & 1;
+                const long a = ((long)(unsigned)fa[2 * jj]) | ((long)fa[2 * jj + 1] << 32);
+                const long bq = ((long)(unsigned)fb[nt][2 * jj]) | ((long)fb[nt][2 * jj + 1] << 32);
+                return __builtin_amdgcn_mfma_i32_32x32x16_i8(a, bq, cmagic, 0, 0, 0);
+            };
+            d[0] = unit(0);
+#pragma unroll
+            for (int v = 0; v < 2 * NT; v++) {
+                if (v + 1 < 2 * NT) {
+                    d[(v + 1) & 1] = unit(v + 1);
+                    asm volatile("" : "+v"(d[(v + 1) & 1]));
+                }
+                const int u = v >> 1;
+                const float dwv = (v & 1) ? dw2[u] : dw[u];
+                scale_accumulate_dpp(acc[u], d[v & 1], dwv, -dwv * kMagicF, dxv);
+                asm volatile("" : "+v"(acc[u][0]), "+v"(acc[u][1]), "+v"(acc[u][2]), "+v"(acc[u][3]), "+v"(acc[u][4]),
+                                  "+v"(acc[u][5]), "+v"(acc[u][6]), "+v"(acc[u][7]), "+v"(acc[u][8]), "+v"(acc[u][9]),
+                                  "+v"(acc[u][10]), "+v"(acc[u][11]), "+v"(acc[u][12]), "+v"(acc[u][13]),
+                                  "+v"(acc[u][14]), "+v"(acc[u][15]));
+            }
+            continue;
         }
         if (MODE >= 4) {
             fa = fa_next;
@@ -313,7 +347,7 @@ int sbk_copy(size_t bytes, int launches, double* us_per_launch) {
 // `warm_launches` untimed launches come first: under matrix load the chip takes some 20 ms to settle at the clock it
 // then sustains (the first launches after idle run 15 % slower), and a prefill is hundreds of such launches.
 int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, int warm_launches, double* us, double* tops, double* cycles_per_unit) {
-    if (!us || !tops || !cycles_per_unit || mode < 0 || mode > 5 || wgs_per_cu < 1 || wgs_per_cu > 4 || nblocks <= 0 || warm_launches < 1) return SBK_ERR;
+    if (!us || !tops || !cycles_per_unit || mode < 0 || mode > 6 || wgs_per_cu < 1 || wgs_per_cu > 4 || nblocks <= 0 || warm_launches < 1) return SBK_ERR;
     if ((row_tiles != 4 && row_tiles != 2) || (row_tiles == 4 && wgs_per_cu > 3)) return SBK_ERR;
     Timer t;
     if (!t.ok) return SBK_ERR;
@@ -334,12 +368,12 @@ int sbk_mfma_valu(int mode, int row_tiles, int wgs_per_cu, int nblocks, int warm
         (void)hipMemcpy(scales, h.data(), 1024 * 4, hipMemcpyHostToDevice);
         typedef void (*kern_t)(const float*, int, float*, unsigned long long*, const v4i*);
         // [mode][tile 4/2][occupancy class: waves per SIMD the register budget is set for]
-        static const kern_t k4lo[6] = {mfma_valu_kernel<0, 4, 2>, mfma_valu_kernel<1, 4, 2>, mfma_valu_kernel<2, 4, 2>, mfma_valu_kernel<3, 4, 2>,
-                                       mfma_valu_kernel<4, 4, 2>, mfma_valu_kernel<5, 4, 2>};
-        static const kern_t k4hi[6] = {mfma_valu_kernel<0, 4, 3>, mfma_valu_kernel<1, 4, 3>, mfma_valu_kernel<2, 4, 3>, mfma_valu_kernel<3, 4, 3>,
-                                       mfma_valu_kernel<4, 4, 3>, mfma_valu_kernel<5, 4, 3>};
-        static const kern_t k2[6] = {mfma_valu_kernel<0, 2, 4>, mfma_valu_kernel<1, 2, 4>, mfma_valu_kernel<2, 2, 4>, mfma_valu_kernel<3, 2, 4>,
-                                     mfma_valu_kernel<4, 2, 4>, mfma_valu_kernel<5, 2, 4>};
+        static const kern_t k4lo[7] = {mfma_valu_kernel<0, 4, 2>, mfma_valu_kernel<1, 4, 2>, mfma_valu_kernel<2, 4, 2>, mfma_valu_kernel<3, 4, 2>,
+                                       mfma_valu_kernel<4, 4, 2>, mfma_valu_kernel<5, 4, 2>, mfma_valu_kernel<6, 4, 2>};
+        static const kern_t k4hi[7] = {mfma_valu_kernel<0, 4, 3>, mfma_valu_kernel<1, 4, 3>, mfma_valu_kernel<2, 4, 3>, mfma_valu_kernel<3, 4, 3>,
+                                       mfma_valu_kernel<4, 4, 3>, mfma_valu_kernel<5, 4, 3>, mfma_valu_kernel<6, 4, 3>};
+        static const kern_t k2[7] = {mfma_valu_kernel<0, 2, 4>, mfma_valu_kernel<1, 2, 4>, mfma_valu_kernel<2, 2, 4>, mfma_valu_kernel<3, 2, 4>,
+                                     mfma_valu_kernel<4, 2, 4>, mfma_valu_kernel<5, 2, 4>, mfma_valu_kernel<6, 2, 4>};
         const kern_t kern = row_tiles == 2 ? k2[mode] : (wgs_per_cu <= 2 ? k4lo[mode] : k4hi[mode]);
         auto launch = [&]() { hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, t.s, (const float*)scales, nblocks, out, cyc, (const v4i*)aglob); };
         if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) rc = SBK_ERR;
