@@ -233,7 +233,7 @@ class Bench:
         return out
 
     def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False, trait=False):
-        """m rows against rotating weight copies.  m <= 4: the dot4 GEMV (quantiser fused for m = 1); 5..32 rows of a
+        """m rows against rotating weight copies.  m <= 4: the dot4 GEMV (quantiser fused for m = 1); 5..64 rows of a
         Q8_0 / Q4_0 weight: the small-batch kernel on the matrix cores; f32: the fp32-activation GEMV (no quantiser)."""
         acc, sy = self.acc, self.synth
         steps, warmup = steps or self.steps, warmup if warmup is not None else self.warmup
@@ -260,6 +260,8 @@ class Bench:
         def step(i):
             if f32:
                 acc.gemv_f32_dev(keys[i % ncopies], xd, yd)
+            elif m > 32:    # a short prefill chunk: the GEMM entry point (33..64 rows: the small-batch kernel with two token tiles)
+                acc.gemm_dev(keys[i % ncopies], xd, m, yd)
             else:
                 acc.gemv_dev(keys[i % ncopies], xd, m, yd)
 
@@ -709,6 +711,7 @@ def main():
         ("q8_0_gemv_2560x9728_m8", lambda: b.gemv("q8_0_gemv_2560x9728_m8", Q8_0, 2560, 9728, 8, int(1.1 * GB))),
         ("q8_0_small_batch_2560x9728_m16", lambda: b.gemv("q8_0_small_batch_2560x9728_m16", Q8_0, 2560, 9728, 16, int(1.1 * GB))),
         ("q8_0_small_batch_2560x9728_m32", lambda: b.gemv("q8_0_small_batch_2560x9728_m32", Q8_0, 2560, 9728, 32, int(1.1 * GB))),
+        ("q8_0_small_batch_2560x9728_m64", lambda: b.gemv("q8_0_small_batch_2560x9728_m64", Q8_0, 2560, 9728, 64, int(1.1 * GB))),
         ("q4_0_gemv_f32_9728x2560", lambda: b.gemv("q4_0_gemv_f32_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB), f32=True)),
         ("q8_0_gemv_f32_2560x9728", lambda: b.gemv("q8_0_gemv_f32_2560x9728", Q8_0, 2560, 9728, 1, int(1.1 * GB), f32=True)),
         ("q6_k_gemv_f32_15360x3840", lambda: b.gemv("q6_k_gemv_f32_15360x3840", Q6_K, 15360, 3840, 1, int(1.1 * GB), f32=True)),

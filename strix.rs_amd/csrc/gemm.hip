@@ -243,10 +243,12 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
                 *(uint4*)(sB + off + ((2 * q_bi + 1 + r) & 7) * 16) = hi;  // elements 16..31
             }
         }
-        if (!Q6 && role_w) {
+        if (!Q6 && role_w) {   // the four block scales of a row side by side: one 16-byte write here, one 16-byte read per row tile and stage
             const unsigned h[4] = {rsv.x & 0xffffu, rsv.x >> 16, rsv.y & 0xffffu, rsv.y >> 16};
+            float v[KB];
 #pragma unroll
-            for (int j = 0; j < KB; j++) sdw[j * 128 + wr] = (w_valid && blk0 + j < p.nb) ? h2f_((uint16_t)h[j]) : 0.f;
+            for (int j = 0; j < KB; j++) v[j] = (w_valid && blk0 + j < p.nb) ? h2f_((uint16_t)h[j]) : 0.f;
+            *(float4*)(sdw + wr * 4) = make_float4(v[0], v[1], v[2], v[3]);
         }
         if (role_x) {
             const unsigned v[4] = {rsv.x, rsv.y, rsv.z, rsv.w};
@@ -275,6 +277,16 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     const int dx_tok = ((lane & 15) >> 2) * 8 + half * 4 + (lane & 3);  // token of accumulator lane % 16 in this lane's half
     const int frag6 = (col >> 3) * GRP + (col & 7) * 128 + half * 8;
 
+    float4 stage_dw[4];   // Q8_0 / Q4_0: the weight scales of this lane's row in each row tile, four blocks of the stage
+    auto read_stage_scales = [&](int buf) {
+        if (Q6) return;
+        const float* sdw = (const float*)(smem + buf * STAGE_BYTES + A_BYTES + B_BYTES);
+#pragma unroll
+        for (int nt = 0; nt < 4; nt++) {
+            if (nt >= nt_cnt) break;
+            stage_dw[nt] = *(const float4*)(sdw + ((nt_base + nt) * 32 + col) * 4);
+        }
+    };
     auto read_frag = [&](GemmFrag<SUB>& f, int buf, int bi) {
         const char* sA = smem + buf * STAGE_BYTES;
         const char* sB = sA + A_BYTES;
@@ -306,7 +318,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
             for (int nt = 0; nt < 4; nt++) {
                 if (nt >= nt_cnt) break;
                 f.b[nt] = *(const v4i*)(sBw + nt * 4 * GRP + frag_lane[bi]);
-                f.dw[nt][0] = sdww[bi * 128 + nt * 32 + col];
+                f.dw[nt][0] = bi == 0 ? stage_dw[nt].x : (bi == 1 ? stage_dw[nt].y : (bi == 2 ? stage_dw[nt].z : stage_dw[nt].w));
             }
         }
     };
@@ -383,6 +395,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         if (more && (my_slot == 0 || !wave_live)) issue_stage(buf ^ 1, s + 1);
         if (wave_live) {
         GemmFrag<SUB> f0, f1;
+        read_stage_scales(buf);
         read_frag(f0, buf, 0);
         read_frag(f1, buf, 1);
         __builtin_amdgcn_sched_barrier(0);
