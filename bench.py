@@ -278,7 +278,7 @@ class Bench:
         # With one activation row the quantiser is fused: a step is exactly one launch of the GEMV
         # kernel, so the timed region's events give that kernel's average launch duration directly
         # (an event pair per launch adds about 2 us of its own and is reported separately).
-        single = m == 1 or f32
+        single = m == 1 or f32 or len(set(self.last_names)) == 1   # (2..4 rows may be quantised inside the GEMV: one launch)
         launch_us = ms / steps * 1e3 if single else kus
         kgbs = algo / (launch_us * 1e-6) / 1e9
         return {
@@ -675,6 +675,8 @@ def main():
     ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-floors", action="store_true", help="skip the measurement-only kernels (empty launch, read floor, MFMA+FMA ceiling)")
+    ap.add_argument("--no-trait", action="store_true", help="skip the host-pointer trait-call timing of the headline workload (keeps a kernel trace of the run to the timed launches)")
+    ap.add_argument("--records", default=os.path.join(ROOT, "bench_workloads.json"), help="where the per-workload records are written")
     ap.add_argument("--no-headline", action="store_true", help="skip the headline GEMV when --only names other workloads")
     ap.add_argument("--tune", default="", help="launch-geometry overrides for sweeps, e.g. gemm_nw=4,gemm_splitk=2")
     a = ap.parse_args()
@@ -697,7 +699,7 @@ def main():
     if a.no_headline and only:
         head = None
     else:
-        head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB), trait=True)
+        head = b.gemv("q4_0_gemv_9728x2560", Q4_0, 9728, 2560, 1, int(1.1 * GB), trait=not a.no_trait)
         work[head["workload"]] = head
         b.log(json.dumps(head))
     plans = [
@@ -743,11 +745,16 @@ def main():
                 w["rescale_ceiling_TOPS"], w["kernel_over_ceiling"] = ceil, w["kernel_TOPS"] / ceil
                 b.log(f"{n}: kernel {w['kernel_TOPS']:.0f} TOPS = {w['kernel_over_ceiling']:.2f} of its arithmetic's ceiling ({ceil:.0f} TOPS)")
     if head is None:  # sweep mode: per-workload records only, no headline line
-        print(json.dumps({"workloads": work}), flush=True)
+        try:
+            with open(a.records, "w") as f:
+                json.dump({"workloads": work}, f, indent=1)
+        except OSError as e:
+            b.log(f"could not write {a.records}: {e}")
+        print(json.dumps({"workloads": sorted(work)}), flush=True)
         return
     cpu = None if a.no_cpu else cpu_baseline()
     b.acc.close()
-    wpath = os.path.join(ROOT, "bench_workloads.json")
+    wpath = a.records
     try:
         with open(wpath, "w") as f:
             json.dump({"workloads": work}, f, indent=1)

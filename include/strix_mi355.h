@@ -253,9 +253,11 @@ int smx_graph_end(smx_ctx* ctx, smx_graph** out);
 int smx_graph_launch(smx_ctx* ctx, smx_graph* g);   /* enqueue one replay on the context's stream */
 void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
 
-/* Launch-geometry overrides for measurement sweeps; value 0 restores the built-in choice.  They shape
+/* Measurement hook, not part of the operator surface (no counterpart in the reference; a binding has no reason to
+ * call it): launch-geometry overrides for sweeps; value 0 restores the built-in choice.  They shape
  * a kernel's launch, never which kernel a shape is served by.
- * Knobs: "gemm_splitk" (K slices of the GEMM), "gemm_tile_m" (tokens per GEMM tile: 64 or 128); for shapes served by the row-per-wavefront GEMV (rows that
+ * Knobs: "gemm_splitk" (K slices of the GEMM), "gemm_tile_m" (tokens per GEMM tile: 64 or 128), "gemm_walk" (token-tile
+ * groups of the GEMM's tile walk); for shapes served by the row-per-wavefront GEMV (rows that
  * are not a whole number of 16-byte unit groups, or longer than 16384 elements): "gemv_rpw" (rows per
  * wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4), "gemv_lpr" (lanes per row: 16, 32,
  * 64), "gemv_wpc" (workgroups per CU).  Results do not depend on them beyond fp32 summation order. */
