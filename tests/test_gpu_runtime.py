@@ -126,13 +126,24 @@ def test_tuning_knobs_keep_results(accel, orc, synth, relerr, pkg):
             for k in knobs:
                 accel.tune(k, 0)
     raw = synth.make_weight(8, 256, 4096, seed=11)
-    xs = synth.make_acts(64, 4096, seed=12)
+    xs = synth.make_acts(96, 4096, seed=12)             # 96 rows: the tiled GEMM (up to 64 run in the small-batch kernel)
     assert accel.upload_q8_0("t.tune", raw, 4096, 256)
     ref = orc.matmul_q8_from_f32(8, raw, 4096, 256, xs)
-    for sk in (1, 2, 4, 8):
+    for sk in (1, 2, 4, 8, 16):
         accel.tune("gemm_splitk", sk)
-        assert relerr(accel.prefill_q8_gemm("t.tune", xs, 64, 256), ref) <= 1e-5
+        assert relerr(accel.prefill_q8_gemm("t.tune", xs, 96, 256), ref) <= 1e-5
+        assert relerr(accel.prefill_q8_gemm("t.tune", xs[:40], 40, 256), ref[:40]) <= 1e-5   # small-batch kernel: one or two K slices
     accel.tune("gemm_splitk", 0)
+    # the GEMM's tile walk only renumbers tiles: every grouping of the token tiles gives the same bits
+    raw = synth.make_weight(2, 1000, 512, seed=13)
+    xs = synth.make_acts(1100, 512, seed=14)            # 9 token tiles x 8 weight strips
+    assert accel.upload_q4_0("t.tune", raw, 512, 1000)
+    base = accel.prefill_q8_gemm("t.tune", xs, 1100, 1000)
+    assert relerr(base, orc.matmul_q8_from_f32(2, raw, 512, 1000, xs)) <= 1e-5
+    for walk in (1, 2, 3, 9, 64):
+        accel.tune("gemm_walk", walk)
+        assert np.array_equal(accel.prefill_q8_gemm("t.tune", xs, 1100, 1000), base), walk
+    accel.tune("gemm_walk", 0)
     with pytest.raises(pkg.SmxError):
         accel.tune("gemv_flat", 1)          # no knob re-routes a shape to another kernel
     with pytest.raises(pkg.SmxError):
