@@ -475,7 +475,7 @@ class Bench:
     def decode_chain_graph(self, name, layers=4, hidden=2048, ffn=8192, ne=64, eff=768, k=8, nsets=4, steps=None, warmup=None):
         """`layers` decoder FFN halves per token, everything resident and routed on the device (strix.rs_amd/chain.py, the
         sequence tests/test_gpu_chain.py checks against the oracle): per layer rmsnorm + gate/up GEMVs + SwiGLU product
-        (one launch), down GEMV, router logits and top-k (two launches), the k routed experts' FFN (two launches).  Attention
+        (one launch), down GEMV, router logits GEMV, the k routed experts' FFN (two launches, the routing in the prologue of the first).  Attention
         is outside this path.  Q4_0 dense weights, Q8_0 experts and router.  Cache-cold: `nsets` complete weight sets
         (every layer's dense weights and expert tensors) are resident and ONE captured graph runs one token through each
         set in turn, so a token's weights were last read nsets - 1 tokens (> 1 GB of other weights) ago."""
@@ -500,8 +500,8 @@ class Bench:
         acc.h2d(nw, np.ones(hidden, np.float32))
         keys = lambda l: tuple(f"{name}.{t}{l}" for t in "gudr")
 
-        def measure(sets):
-            ch = chain_mod.FfnMoeChain(acc, layers, hidden, ffn, ne, k, keys, lambda l: base + l, nw)
+        def measure(sets, route="in_launch"):
+            ch = chain_mod.FfnMoeChain(acc, layers, hidden, ffn, ne, k, keys, lambda l: base + l, nw, route=route)
 
             def tokens():   # one token through each weight set
                 for s_ in range(sets):
@@ -521,6 +521,7 @@ class Bench:
             return graph_ms / (reps * sets) * 1e3, eager_ms / (reps * sets) * 1e3, n_launch
 
         cold_us, cold_eager_us, n_launch = measure(nsets)
+        routed_by_a_launch_us, _, _ = measure(nsets, route="launches")
         hot_us, _, _ = measure(1)
         for l in range(nl):
             for t in "gudr":
@@ -533,7 +534,7 @@ class Bench:
                                             "launches_per_token": n_launch, "weight_sets_rotated": nsets},
                 "weight_bytes_per_token": wbytes, "bytes_between_two_reads_of_a_weight": wbytes * (nsets - 1),
                 "steps": max(1, steps // nsets) * nsets, "graph_us_per_token": cold_us, "eager_us_per_token": cold_eager_us,
-                "one_weight_set_us_per_token": hot_us,
+                "routing_as_a_launch_of_its_own_us_per_token": routed_by_a_launch_us, "one_weight_set_us_per_token": hot_us,
                 "GBps": gbs, "frac_hbm_peak": gbs / HBM_PEAK_GBS,
                 "note": "graph_us_per_token is cache-cold (weight sets rotate); one_weight_set_us_per_token re-reads one 274 MB "
                         "set, partly from the 256 MB Infinity Cache"}

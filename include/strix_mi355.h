@@ -234,6 +234,14 @@ int smx_moe_router_dev(smx_ctx* ctx, const char* key, const float* x_dev, size_t
  * are clamped. */
 int smx_moe_ffn_routed_dev(smx_ctx* ctx, size_t layer, const int32_t* ids_dev, const float* w_dev, size_t k,
                            const float* x_dev, float* y_dev);
+/* The routed expert FFN of a decode token straight from the router logits (topk_router followed by moe_launches,
+ * decode.rs:1154-1180, as ONE call): y_dev = sum_k w_k * expert_{id_k}(x_dev) with (ids, w) = the routing of
+ * smx_moe_route_dev on logits_dev[ne], ne = the layer's expert count.  For up to 64 experts and k <= 8 the routing runs in the
+ * prologue of the experts' gate/up launch (every workgroup repeats the 64-logit top-k; no routing launch: two launches per
+ * token instead of three); other shapes run the routing launch first.  ids_dev[k] / w_dev[k] receive the routing (the down
+ * launch reads them).  Same bits as smx_moe_route_dev + smx_moe_ffn_routed_dev.  Capturable. */
+int smx_moe_ffn_logits_dev(smx_ctx* ctx, size_t layer, const float* logits_dev, size_t k, const float* x_dev, float* y_dev,
+                           int32_t* ids_dev, float* w_dev);
 /* smx_moe_layer with the activations and the result on the device (y_dev: m x hidden floats); the
  * routing tables still come from the host at every call, so it cannot be captured in a graph. */
 int smx_moe_layer_dev(smx_ctx* ctx, size_t layer, const float* xs_dev, size_t m, const size_t* plan,

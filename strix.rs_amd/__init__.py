@@ -36,7 +36,7 @@ EXPORTS = [
     "smx_gguf_find", "smx_gguf_meta_u64", "smx_gguf_meta_f32", "smx_gguf_meta_str", "smx_gguf_attach", "smx_gguf_upload_as",
     "smx_host_quantize_q8_0", "smx_host_quantize_q4_0", "smx_host_dequantize", "smx_moe_layer_dev",
     "smx_weight_dims", "smx_moe_layer_stages", "smx_gemv_noalloc_dev",
-    "smx_gemv_f32", "smx_gemv_f32_dev", "smx_gemv_f32_batch", "smx_moe_route_dev", "smx_moe_route", "smx_moe_ffn_routed_dev", "smx_moe_router_dev",
+    "smx_gemv_f32", "smx_gemv_f32_dev", "smx_gemv_f32_batch", "smx_moe_route_dev", "smx_moe_route", "smx_moe_ffn_routed_dev", "smx_moe_router_dev", "smx_moe_ffn_logits_dev",
 ]
 ACT_NONE, ACT_RMSNORM, ACT_SILU_MUL, ACT_GEGLU = 0, 1, 2, 3
 
@@ -108,6 +108,7 @@ def load_library():
     L.smx_moe_route_dev.argtypes = [vp, vp, sz, sz, vp, vp]
     L.smx_moe_route.argtypes = [vp, vp, sz, sz, vp, vp]
     L.smx_moe_router_dev.argtypes = [vp, cp, vp, sz, vp, vp, vp]
+    L.smx_moe_ffn_logits_dev.argtypes = [vp, sz, vp, sz, vp, vp, vp, vp]
     L.smx_moe_ffn_routed_dev.argtypes = [vp, sz, vp, vp, sz, vp, vp]
     L.smx_gemm_fused_dev.argtypes = [vp, cp, i, vp, vp, sz, C.c_float, vp]
     L.smx_moe_layer_ffn.argtypes = [vp, sz, vp, sz, vp, sz, vp, sz]
@@ -558,6 +559,10 @@ class Mi355WeightAccel:
     def moe_router_dev(self, key, x_dev, k, ids_dev, w_dev, logits_dev=None):
         """Router logits (GEMV of the resident router weight) + softmax + top-k in one call."""
         return self._check(self._L.smx_moe_router_dev(self._h, key.encode(), x_dev, k, ids_dev, w_dev, logits_dev))
+
+    def moe_ffn_logits_dev(self, layer, logits_dev, k, x_dev, y_dev, ids_dev, w_dev):
+        """Routed expert FFN of a decode token from the router logits (routing inside the gate/up launch where it serves)."""
+        return self._check(self._L.smx_moe_ffn_logits_dev(self._h, layer, logits_dev, k, x_dev, y_dev, ids_dev, w_dev))
 
     def moe_ffn_routed_dev(self, layer, ids_dev, w_dev, k, x_dev, y_dev):
         """moe_ffn_dev reading the routing from device memory at run time (capturable with new routing)."""

@@ -16,6 +16,7 @@
 #include <type_traits>
 
 #include "gemv_body.h"
+#include "router_body.h"
 #include "smx_internal.h"
 
 namespace smx {
@@ -57,6 +58,12 @@ struct GemvJobs {
     int ne;
     unsigned long long blocks_per_expert;
     int slot[SMX_GEMV_GROUP_MAX];
+    // routing inside the launch (paired form only): every workgroup routes the ne <= 64 router logits itself (top route_k) and
+    // workgroup (0, 0) writes the routing out for the launches behind this one
+    const float* logits;
+    int route_k;
+    int* ids_out;
+    float* w_out;
 };
 
 // The planes of a job's weight; IND: moved to the expert the device-side routing names.  The indirection is
@@ -69,6 +76,13 @@ __device__ __forceinline__ GemvW job_weight(const GemvJobs& J, int j) {
         const size_t b0 = (size_t)min(max(J.ids[J.slot[j]], 0), J.ne - 1) * J.blocks_per_expert;
         Ops::advance(W, b0);
     }
+    return W;
+}
+// the same with the expert given (routing computed inside the launch)
+template <class Ops>
+__device__ __forceinline__ GemvW job_weight_at(const GemvJobs& J, int j, int expert) {
+    GemvW W = J.job[j].W;
+    Ops::advance(W, (size_t)min(max(expert, 0), J.ne - 1) * J.blocks_per_expert);
     return W;
 }
 
@@ -91,13 +105,50 @@ __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int* 
 
 // Paired form: workgroup (x, p) serves jobs 2p (gate) and 2p + 1 (up) over the same rows and writes the product of the
 // activated gate dot and the up dot (gemv_body_flat, DUAL).
-template <class Ops, int PRE, int GL, int FQ, bool IND = false>
+// IND: 0 = the jobs' weights as given, 1 = experts read from device memory (J.ids), 2 = experts routed here: the first wave of
+// every workgroup runs the router (softmax + top route_k of the ne <= 64 logits, the arithmetic of topk_router_kernel) before the
+// workgroup requests its weights, which saves the routing launch in front of a decode token's expert FFN (3.2 us for about
+// 1.3 us of prologue); workgroup (0, 0) writes ids and weights out for the down launch.
+template <class Ops, int PRE, int GL, int FQ, int IND = 0>
 __global__ __launch_bounds__(1024) void gemv_flat_dual_kernel(const GemvJobs J) {
     const GemvJob& jg = J.job[2 * blockIdx.y];
     const GemvJob& ju = J.job[2 * blockIdx.y + 1];
-    gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(job_weight<Ops, IND>(J, 2 * blockIdx.y), jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1, blockIdx.x,
-                                                      jg.n_wgs, jg.magic_u, nullptr, 0, job_weight<Ops, IND>(J, 2 * blockIdx.y + 1), ju.y,
-                                                      jg.h, jg.act2);
+    if constexpr (IND == 2) {
+        __shared__ int r_ids[64];
+        __shared__ float r_w[64];
+        __shared__ float r_sel[64];
+        if (threadIdx.x >= 64 && threadIdx.x < 576) {
+            // while the first wave routes, eight others pull the activation row through this CU's cache: the staging that
+            // follows the routing then finds it there instead of waiting for it after the routing
+            float keep = 0.f;
+            for (int i = threadIdx.x - 64; i < Ops::nb32(jg.nblk) * 8; i += 512) {
+                const float4 t = ((const float4*)jg.x)[i];
+                keep += t.x + t.y + t.z + t.w;
+            }
+            if (J.route_k < 0) r_sel[threadIdx.x & 63] = keep;   // (never: keeps the loads)
+        }
+        if (threadIdx.x < 64) {
+            float v[1];
+            v[0] = (int)threadIdx.x < J.ne ? J.logits[threadIdx.x] : -3.40282347e+38f;
+            topk_router_wave<1>(v, J.ne, J.route_k, r_ids, r_w, r_sel);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            if (blockIdx.x == 0 && blockIdx.y == 0 && (int)threadIdx.x < J.route_k) {
+                J.ids_out[threadIdx.x] = r_ids[threadIdx.x];
+                J.w_out[threadIdx.x] = r_w[threadIdx.x];
+            }
+        }
+        __syncthreads();
+        const int e = r_ids[J.slot[2 * blockIdx.y]];
+        gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(job_weight_at<Ops>(J, 2 * blockIdx.y, e), jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1,
+                                                          blockIdx.x, jg.n_wgs, jg.magic_u, nullptr, 0,
+                                                          job_weight_at<Ops>(J, 2 * blockIdx.y + 1, e), ju.y, jg.h, jg.act2);
+    } else {
+        gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(job_weight<Ops, IND == 1>(J, 2 * blockIdx.y), jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1,
+                                                          blockIdx.x, jg.n_wgs, jg.magic_u, nullptr, 0,
+                                                          job_weight<Ops, IND == 1>(J, 2 * blockIdx.y + 1), ju.y, jg.h, jg.act2);
+    }
 }
 
 namespace {
@@ -480,6 +531,14 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
         J.ne = ind->ne;
         J.blocks_per_expert = ind->blocks_per_expert;
         for (int p = 0; p < npairs; p++) J.slot[2 * p] = J.slot[2 * p + 1] = ind->slot[p];
+        if (ind->logits) {   // routed inside this launch
+            if (ind->ne > 64 || ind->route_k < 1 || ind->route_k > ind->ne || !ind->ids_out || !ind->w_out)
+                return fail(c, SMX_ERR_ARG, "paired gemv: in-launch routing takes up to 64 experts and buffers for the routing");
+            J.logits = ind->logits;
+            J.route_k = ind->route_k;
+            J.ids_out = ind->ids_out;
+            J.w_out = ind->w_out;
+        }
     }
     for (int p = 0; p < npairs; p++) {
         const Weight *a = wg[p], *b = wu[p];
@@ -509,7 +568,7 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
     const size_t upb = w0.type == kQ6_K ? 4 : (w0.type == kQ8_0 ? 2 : 1);
     const size_t rows = (w0.N + g.grid - 1) / g.grid;
     g.lds += rows * w0.nblk * upb / g.flat * 4;
-    if (g.lds > 160 * 1024) return SMX_OK;
+    if (g.lds + (ind && ind->logits ? 1024 : 0) > 160 * 1024) return SMX_OK;   // (in-launch routing keeps 768 bytes of LDS of its own)
     const bool norm = prod && prod->kind == SMX_ACT_RMSNORM;
     const unsigned units = (unsigned)(w0.nblk * upb);
     const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);
@@ -525,7 +584,7 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
     };
 #define SMX_DUAL(OPS, PRE, GL)                                                                                  \
     if (g.flat_pre == PRE && g.flat == GL)                                                                      \
-        return ind ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 1, true>)                                           \
+        return ind ? (ind->logits ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 1, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1, 1>)) \
                    : (norm ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1>));
     if (w0.type == kQ4_0) { SMX_DUAL(OpsQ4_0, 3, 16) SMX_DUAL(OpsQ4_0, 3, 8) }
     else if (w0.type == kQ8_0) { SMX_DUAL(OpsQ8_0, 3, 16) SMX_DUAL(OpsQ8_0, 3, 8) }

@@ -15,6 +15,7 @@
 
 #include "detmath.h"
 #include "gemv_body.h"
+#include "router_body.h"
 #include "smx_internal.h"
 
 namespace smx {
@@ -94,86 +95,6 @@ __device__ __forceinline__ float route_w(const MoeRoute& r, int i) { return r.w_
 // argument) and tie to the lowest index; their weight is below 2e-38 either way.  One wave;
 // lane l holds experts l, l + 64, ... (PL of them: 1 for up to 64 experts, which keeps the k selection
 // rounds at one compare each).  The softmax denominator is summed in double in a fixed order.
-constexpr int kRouterPerLane = 16;   // ne <= 1024
-// The router's arithmetic, run by ONE wave: v[j] = logit of expert lane + 64 j (-FLT_MAX past ne); sel: 64 floats of LDS.
-template <int PL>
-__device__ __forceinline__ void topk_router_wave(float (&v)[PL], int ne, int k, int* __restrict__ ids, float* __restrict__ w,
-                                                 float* sel) {
-#pragma clang fp contract(off)
-    constexpr int kRouterPerLane = PL;
-    const int lane = threadIdx.x & 63;
-    if constexpr (PL == 1) {
-        // Up to 64 experts, one per lane: every cross-lane step is a lane read into a scalar register (no
-        // LDS round trips, which dominate the time of this one-wave kernel).  A lane's rank = the number
-        // of experts that precede it in (probability descending, index ascending) order; rank r < k is pick r.
-        const bool live = lane < ne;
-        const float x = v[0];
-        float mx = -3.40282347e+38f;
-#pragma unroll
-        for (int j = 0; j < 64; j++) mx = fmaxf(mx, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), j)));
-        const float e = live ? det_expf(x - mx) : 0.f;
-        double sum = 0.0;   // ascending expert index
-#pragma unroll
-        for (int j = 0; j < 64; j++) sum += (double)__int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), j));
-        const float p = live ? e / (float)sum : -1.f;
-        int rank = 0;
-#pragma unroll
-        for (int j = 0; j < 64; j++) {
-            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), j));
-            rank += (pj > p || (pj == p && j < lane)) ? 1 : 0;
-        }
-        if (live && rank < k) {
-            sel[rank] = p;
-            ids[rank] = lane;
-        }
-        // one wave: its own LDS writes, read back by its other lanes
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        float wsum = 0.f;   // in pick order, as the reference sums the chosen probabilities
-        for (int i = 0; i < k; i++) wsum += sel[i];
-        if (lane < k) w[lane] = sel[lane] / wsum;
-        return;
-    }
-    float mx = -3.40282347e+38f;
-#pragma unroll
-    for (int j = 0; j < kRouterPerLane; j++) mx = fmaxf(mx, v[j]);
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    double sum = 0.0;
-#pragma unroll
-    for (int j = 0; j < kRouterPerLane; j++) {
-        const int e = lane + 64 * j;
-        v[j] = e < ne ? det_expf(v[j] - mx) : -1.f;   // probabilities are >= 0: -1 marks "absent or taken"
-        if (e < ne) sum += (double)v[j];
-    }
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
-    const float fsum = (float)sum;
-#pragma unroll
-    for (int j = 0; j < kRouterPerLane; j++)
-        if (v[j] >= 0.f) v[j] = v[j] / fsum;
-    float wsum = 0.f;
-    float mine = 0.f;   // lane i keeps the probability of pick i (k <= 64)
-    for (int i = 0; i < k; i++) {
-        float b = -1.f;
-        int bi = 1 << 30;
-#pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++)
-            if (v[j] > b) { b = v[j]; bi = lane + 64 * j; }   // ascending index within the lane: '>' keeps the lowest
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ob = __shfl_xor(b, off);
-            const int oi = __shfl_xor(bi, off);
-            if (ob > b || (ob == b && oi < bi)) { b = ob; bi = oi; }
-        }
-#pragma unroll
-        for (int j = 0; j < kRouterPerLane; j++)
-            if (lane + 64 * j == bi) v[j] = -1.f;
-        if (lane == i) mine = b;
-        if (lane == 0) ids[i] = bi;
-        wsum += b;   // in pick order, as the reference sums the chosen probabilities
-    }
-    if (lane < k) w[lane] = mine / wsum;
-}
-
 template <int PL>
 __global__ __launch_bounds__(64) void topk_router_kernel(const float* __restrict__ logits, int ne, int k,
                                                          int* __restrict__ ids, float* __restrict__ w) {
@@ -595,12 +516,15 @@ struct MoeScratch {
     float* ad;
 };
 
-// ids / wexp: the routing on the host; or, with ids_dev / w_dev, device memory read when the kernels run.
+// ids / wexp: the routing on the host; or, with ids_dev / w_dev, device memory read when the kernels run; or, with logits_dev
+// as well, the routing is computed from the router logits by the gate/up launch itself (which writes ids_dev / w_dev for
+// the down launch), or by a routing launch in front where that form does not serve.
 static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, const float* wexp, size_t k,
                            const float* x_dev, float* y_dev, MoeScratch* out_scratch, const int32_t* ids_dev = nullptr,
-                           const float* w_dev = nullptr) {
+                           const float* w_dev = nullptr, const float* logits_dev = nullptr) {
     if (k == 0 || k > 64) return fail(c, SMX_ERR_LIMIT, "moe_ffn: %zu routed experts (1..64 supported)", k);
     const bool routed_on_device = ids_dev != nullptr;
+    bool route_pending = logits_dev != nullptr;   // the routing has not been computed yet
     for (size_t i = 0; i < k && !routed_on_device; i++)
         if (ids[i] < 0 || (size_t)ids[i] >= L.ne)
             return fail(c, SMX_ERR_ARG, "moe_ffn: expert id %d outside 0..%zu", ids[i], L.ne - 1);
@@ -656,14 +580,32 @@ static int moe_ffn_enqueue(smx_ctx* c, const MoeLayer& L, const int32_t* ids, co
             }
             constexpr int kPairs = SMX_GEMV_GROUP_MAX / 2;
             paired = true;
+            // the routing inside the gate/up launch: one launch of all k pairs, up to 64 experts
+            const bool route_here = route_pending && k <= (size_t)kPairs && L.ne <= 64 && k <= L.ne;
+            if (route_pending && !route_here) {
+                if ((rc = smx_moe_route_dev(c, logits_dev, L.ne, k, (int32_t*)ids_dev, (float*)w_dev)) != SMX_OK) return rc;
+                route_pending = false;
+            }
             for (size_t i = 0; i < k && paired; i += kPairs) {
                 const int n = (int)std::min<size_t>(kPairs, k - i);
                 for (int j = 0; j < n; j++) ind.slot[j] = (int)(i + j);
                 bool served = false;
+                GemvIndirect ind2 = ind;
+                if (route_pending) {
+                    ind2.logits = logits_dev;
+                    ind2.route_k = (int)k;
+                    ind2.ids_out = (int*)ids_dev;
+                    ind2.w_out = (float*)w_dev;
+                }
                 rc = launch_gemv_dual(c, &wgp[i], &wup[i], &xs[i], &ygp[i], &yup[i], &hp[i], n, SMX_ACT_SILU_MUL, nullptr,
-                                      "moe_gemv_gate_up", &served, routed_on_device ? &ind : nullptr);
+                                      "moe_gemv_gate_up", &served, routed_on_device ? &ind2 : nullptr);
                 if (rc != SMX_OK) return rc;
                 if (!served) paired = false;   // (the first chunk decides: every chunk has the same shape)
+                else route_pending = false;
+            }
+            if (route_pending) {   // the paired form does not serve this shape: the routing launch, then the grouped launch below
+                if ((rc = smx_moe_route_dev(c, logits_dev, L.ne, k, (int32_t*)ids_dev, (float*)w_dev)) != SMX_OK) return rc;
+                route_pending = false;
             }
         }
         for (size_t i = 0; i < 2 * k && !paired; i += SMX_GEMV_GROUP_MAX) {
@@ -989,6 +931,20 @@ int smx_moe_ffn_routed_dev(smx_ctx* c, size_t layer, const int32_t* ids_dev, con
         auto it = c->moe.find(layer);
         if (it == c->moe.end()) return SMX_NOT_RESIDENT;
         return moe_ffn_enqueue(c, it->second, nullptr, nullptr, k, x_dev, y_dev, nullptr, ids_dev, w_dev);
+    });
+}
+
+int smx_moe_ffn_logits_dev(smx_ctx* c, size_t layer, const float* logits_dev, size_t k, const float* x_dev, float* y_dev,
+                           int32_t* ids_dev, float* w_dev) {
+    if (!c) return SMX_ERR_ARG;
+    if (!logits_dev || !ids_dev || !w_dev || !x_dev || !y_dev) return fail(c, SMX_ERR_ARG, "moe_ffn_logits_dev: null argument");
+    return guarded(c, "moe_ffn_logits_dev", [&]() -> int {
+        auto it = c->moe.find(layer);
+        if (it == c->moe.end()) return SMX_NOT_RESIDENT;
+        const MoeLayer& L = it->second;
+        if (L.ne > 64 * (size_t)kRouterPerLane || k == 0 || k > 64 || k > L.ne)
+            return fail(c, SMX_ERR_LIMIT, "moe_ffn_logits_dev: %zu experts, top %zu (up to %d experts, top 64)", L.ne, k, 64 * kRouterPerLane);
+        return moe_ffn_enqueue(c, L, nullptr, nullptr, k, x_dev, y_dev, nullptr, ids_dev, w_dev, logits_dev);
     });
 }
 

@@ -242,6 +242,12 @@ struct GemvIndirect {
     int ne;
     size_t blocks_per_expert;
     int slot[SMX_GEMV_GROUP_MAX];
+    // paired launches only: route inside the launch from the ne <= 64 router logits (top route_k); ids_out / w_out
+    // receive the routing for the launches behind it (ids may then be null)
+    const float* logits = nullptr;
+    int route_k = 0;
+    int* ids_out = nullptr;
+    float* w_out = nullptr;
 };
 // x2s (optional, with prod): a second operand per job instead of prod->b.
 int launch_gemv_group(smx_ctx* c, const Weight* const* ws, const float* const* xs, float* const* ys, int n,

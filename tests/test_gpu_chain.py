@@ -1,5 +1,5 @@
 """The decode chain that bench.py times (strix.rs_amd/chain.py: per layer rmsnorm + gate/up + SwiGLU product, down GEMV,
-router, routed expert FFN; the reference's captured token, decode.rs:3053-3203) against the oracle, stage by stage,
+router logits, routed expert FFN with the routing in its gate/up launch; the reference's captured token, decode.rs:3053-3203) against the oracle, stage by stage,
 eager and as a replayed graph, and the router call on its own."""
 import importlib.util
 import os
@@ -95,7 +95,7 @@ def test_decode_chain_stage_by_stage_eager_and_replayed(accel, orc, synth, reler
     accel.h2d(nwd, nw)
     ch = chain_mod.FfnMoeChain(accel, layers, H, F, ne, k, lambda l: tuple(f"t.ch.{t}{l}" for t in "gudr"), lambda l: base + l,
                                nwd, eps=1e-6, keep_stages=True)
-    assert ch.launches_per_token() == 12
+    assert ch.launches_per_token() == 10
     toks = synth.make_acts(4, H, seed=77) * np.float32(1.5)
 
     def run_eager(x):
@@ -150,14 +150,16 @@ def test_decode_chain_stage_by_stage_eager_and_replayed(accel, orc, synth, reler
         assert np.array_equal(_read(accel, out, H), want[t]), f"replay of token {t}"
     accel.graph_destroy(g)
 
-    # the chain with the router as two calls gives the same bits
-    ch2 = chain_mod.FfnMoeChain(accel, layers, H, F, ne, k, lambda l: tuple(f"t.ch.{t}{l}" for t in "gudr"), lambda l: base + l,
-                                nwd, eps=1e-6, router_call=False)
-    accel.h2d(xd, toks[3])
-    out2 = ch2.enqueue(xd)
-    accel.sync()
-    assert np.array_equal(_read(accel, out2, H), want[3])
-    ch2.close()
+    # the chain with the routing as a launch of its own (router call, or GEMV + routing) gives the same bits
+    for route in ("call", "launches"):
+        ch2 = chain_mod.FfnMoeChain(accel, layers, H, F, ne, k, lambda l: tuple(f"t.ch.{t}{l}" for t in "gudr"), lambda l: base + l,
+                                    nwd, eps=1e-6, route=route)
+        assert ch2.launches_per_token() == 12
+        accel.h2d(xd, toks[3])
+        out2 = ch2.enqueue(xd)
+        accel.sync()
+        assert np.array_equal(_read(accel, out2, H), want[3]), route
+        ch2.close()
     ch.close()
     accel.dev_free(nwd)
     accel.dev_free(xd)

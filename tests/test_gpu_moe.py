@@ -302,3 +302,51 @@ def test_moe_decode_graph_serves_each_tokens_own_routing(accel, orc, synth, ty):
     for p in (ld, xd, yd, idd, wd):
         accel.dev_free(p)
     assert accel.moe_ffn_routed_dev(999, idd, wd, k, xd, yd) is False
+
+
+@pytest.mark.parametrize("ty,ne,hidden,eff,k", [(8, 64, 2048, 768, 8), (8, 16, 512, 256, 4), (14, 16, 512, 256, 4), (8, 64, 512, 256, 12),
+                                                (8, 128, 256, 128, 6), (8, 8, 256, 96, 2), (8, 5, 256, 64, 5)])
+def test_moe_ffn_from_router_logits(accel, orc, synth, ty, ne, hidden, eff, k):
+    """smx_moe_ffn_logits_dev: the routing of a decode token computed in the prologue of the experts' gate/up launch (up to 64
+    experts, k <= 8, paired flat-form expert rows), or by a routing launch in front of it (the other shapes here: 12 routed
+    experts, 128 experts, expert rows of 96 elements): the routing and the output have the bits of smx_moe_route_dev +
+    smx_moe_ffn_routed_dev, the experts are those the oracle routes; captured once and replayed with other logits."""
+    layer = 45
+    gate, up, down = (synth.make_moe_q8 if ty == 8 else synth.make_moe_q6)(ne, hidden, eff, seed=ne + eff)
+    assert (accel.upload_moe_q8 if ty == 8 else accel.upload_moe_q6)(layer, gate, up, down, hidden, eff, ne)
+    rng = np.random.default_rng(ne + k)
+    ld, xd, yd, y2 = accel.dev_alloc(ne * 4), accel.dev_alloc(hidden * 4), accel.dev_alloc(hidden * 4), accel.dev_alloc(hidden * 4)
+    idd, wd, id2, w2 = (accel.dev_alloc(k * 4) for _ in range(4))
+    toks = []
+    for t in range(4):
+        logits = (rng.standard_normal(ne) * 2.5).astype(np.float32)
+        if t == 2:
+            logits = np.round(logits)                      # exact ties: the lowest index first
+        toks.append((logits, synth.make_acts(1, hidden, seed=200 + t)[0]))
+    want = []
+    for logits, x in toks:
+        accel.h2d(ld, logits)
+        accel.h2d(xd, x)
+        assert accel.moe_route_dev(ld, ne, k, id2, w2) and accel.moe_ffn_routed_dev(layer, id2, w2, k, xd, y2)
+        assert accel.moe_ffn_logits_dev(layer, ld, k, xd, yd, idd, wd)
+        ids = accel.d2h(np.empty(k, np.int32), idd).copy()
+        assert np.array_equal(ids, accel.d2h(np.empty(k, np.int32), id2)) and np.array_equal(ids, orc.route_topk(logits, k)[0])
+        assert np.array_equal(accel.d2h(np.empty(k, np.float32), wd), accel.d2h(np.empty(k, np.float32), w2))
+        y = accel.d2h(np.empty(hidden, np.float32), yd).copy()
+        assert np.array_equal(y, accel.d2h(np.empty(hidden, np.float32), y2))
+        want.append(y)
+    accel.graph_begin()
+    assert accel.moe_ffn_logits_dev(layer, ld, k, xd, yd, idd, wd)
+    g = accel.graph_end()
+    for t in (1, 3, 0, 2):
+        accel.h2d(ld, toks[t][0])
+        accel.h2d(xd, toks[t][1])
+        accel.h2d(yd, np.zeros(hidden, np.float32))
+        accel.h2d(idd, np.full(k, -1, np.int32))
+        accel.graph_launch(g)
+        accel.sync()
+        assert np.array_equal(accel.d2h(np.empty(hidden, np.float32), yd), want[t]), f"token {t}"
+    accel.graph_destroy(g)
+    assert accel.moe_ffn_logits_dev(998, ld, k, xd, yd, idd, wd) is False
+    for p in (ld, xd, yd, y2, idd, wd, id2, w2):
+        accel.dev_free(p)
