@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 # the same counter's reading for a 256 MiB copy (profiles/gemv_q4_0_9728x2560_hbm_traffic.md)
 HEADLINE_TRAFFIC_BYTES = 14232463
 # the same for the Q8_0 ffn_up GEMM launch (profiles/gemm_i8_q8_0_ffn_up_counters.md): L2 fills + writes
-GEMM_TRAFFIC_BYTES = {"gemm_q8_0_ffn_up": 667380565}
+GEMM_TRAFFIC_BYTES = {"gemm_q8_0_ffn_up": 472727060}
 INT8_PEAK_TOPS = 5000.0      # MI355X dense int8 MFMA
 Q4_0, Q8_0, Q6_K = 2, 8, 14
 BLOCK_BYTES = {Q4_0: 18, Q8_0: 34, Q6_K: 210}
