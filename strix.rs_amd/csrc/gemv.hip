@@ -105,42 +105,52 @@ __global__ __launch_bounds__(1024) void gemv_flat_kernel(const GemvJobs J, int* 
 
 // Paired form: workgroup (x, p) serves jobs 2p (gate) and 2p + 1 (up) over the same rows and writes the product of the
 // activated gate dot and the up dot (gemv_body_flat, DUAL).
-// IND: 0 = the jobs' weights as given, 1 = experts read from device memory (J.ids), 2 = experts routed here: the first wave of
-// every workgroup runs the router (softmax + top route_k of the ne <= 64 logits, the arithmetic of topk_router_kernel) before the
-// workgroup requests its weights, which saves the routing launch in front of a decode token's expert FFN (3.2 us for about
-// 1.3 us of prologue); workgroup (0, 0) writes ids and weights out for the down launch.
+// IND: 0 = the jobs' weights as given, 1 = experts read from device memory (J.ids), 2 = experts routed here: every workgroup
+// runs the router (softmax + top route_k of the ne <= 64 logits, the arithmetic of topk_router_kernel) before it requests its
+// weights, which saves the routing launch in front of a decode token's expert FFN (2.9 us for less than 1 us of prologue);
+// workgroup (0, 0) writes ids and weights out for the down launch.
 template <class Ops, int PRE, int GL, int FQ, int IND = 0>
 __global__ __launch_bounds__(1024) void gemv_flat_dual_kernel(const GemvJobs J) {
     const GemvJob& jg = J.job[2 * blockIdx.y];
     const GemvJob& ju = J.job[2 * blockIdx.y + 1];
     if constexpr (IND == 2) {
-        __shared__ int r_ids[64];
-        __shared__ float r_w[64];
+        // Routing by the whole workgroup: every wave computes the 64 probabilities (the same bits everywhere), takes the rank
+        // contributions of 64 / waves experts, and after one barrier every wave adds the parts up and finds the expert whose
+        // rank is this workgroup's slot.  One wave doing all 64 comparisons alone costs the launch 0.6 us more.
+        __shared__ int r_part[16 * 64];
         __shared__ float r_sel[64];
-        if (threadIdx.x >= 64 && threadIdx.x < 576) {
-            // while the first wave routes, eight others pull the activation row through this CU's cache: the staging that
-            // follows the routing then finds it there instead of waiting for it after the routing
-            float keep = 0.f;
-            for (int i = threadIdx.x - 64; i < Ops::nb32(jg.nblk) * 8; i += 512) {
-                const float4 t = ((const float4*)jg.x)[i];
-                keep += t.x + t.y + t.z + t.w;
-            }
-            if (J.route_k < 0) r_sel[threadIdx.x & 63] = keep;   // (never: keeps the loads)
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;   // nwaves <= 16
+        // eight waves pull the activation row through this CU's cache meanwhile (used after the barrier, so nothing waits
+        // for it here): the staging that follows finds the row on its way or there
+        float4 pf = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (wave >= 1 && wave <= 8) {
+            const int i = threadIdx.x - 64;
+            if (i < Ops::nb32(jg.nblk) * 8) pf = ((const float4*)jg.x)[i];
         }
-        if (threadIdx.x < 64) {
-            float v[1];
-            v[0] = (int)threadIdx.x < J.ne ? J.logits[threadIdx.x] : -3.40282347e+38f;
-            topk_router_wave<1>(v, J.ne, J.route_k, r_ids, r_w, r_sel);
+        const bool live = lane < J.ne;
+        const float p = router_prob_lane(live ? J.logits[lane] : -3.40282347e+38f, live);
+        const int per = (64 + nwaves - 1) / nwaves;
+        r_part[wave * 64 + lane] = router_rank_part(p, min(wave * per, 64), min(wave * per + per, 64));
+        __syncthreads();
+        int rank = 0;
+        for (int w = 0; w < nwaves; w++) rank += r_part[w * 64 + lane];
+        const int slot = J.slot[2 * blockIdx.y];
+        const unsigned long long hit = __ballot(live && rank == slot);   // the ranks of the live lanes are a permutation
+        const int e = hit ? (int)__builtin_ctzll(hit) : 0;
+        if (blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {   // the routing itself, for the down launch and the caller
+#pragma clang fp contract(off)
+            if (live && rank < J.route_k) {
+                r_sel[rank] = p;
+                J.ids_out[rank] = lane;
+            }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            if (blockIdx.x == 0 && blockIdx.y == 0 && (int)threadIdx.x < J.route_k) {
-                J.ids_out[threadIdx.x] = r_ids[threadIdx.x];
-                J.w_out[threadIdx.x] = r_w[threadIdx.x];
-            }
+            float wsum = 0.f;   // in pick order, as the reference sums the chosen probabilities
+            for (int i = 0; i < J.route_k; i++) wsum += r_sel[i];
+            if (lane < J.route_k) J.w_out[lane] = r_sel[lane] / wsum;
         }
-        __syncthreads();
-        const int e = r_ids[J.slot[2 * blockIdx.y]];
+        if (J.route_k < 0) r_sel[lane] = pf.x + pf.y + pf.z + pf.w;   // (never: keeps the loads)
         gemv_body_flat<Ops, 1, PRE, GL, FQ, false, true>(job_weight_at<Ops>(J, 2 * blockIdx.y, e), jg.X(), jg.y, jg.N, jg.nblk, jg.N, 1,
                                                           blockIdx.x, jg.n_wgs, jg.magic_u, nullptr, 0,
                                                           job_weight_at<Ops>(J, 2 * blockIdx.y + 1, e), ju.y, jg.h, jg.act2);
@@ -568,7 +578,7 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
     const size_t upb = w0.type == kQ6_K ? 4 : (w0.type == kQ8_0 ? 2 : 1);
     const size_t rows = (w0.N + g.grid - 1) / g.grid;
     g.lds += rows * w0.nblk * upb / g.flat * 4;
-    if (g.lds + (ind && ind->logits ? 1024 : 0) > 160 * 1024) return SMX_OK;   // (in-launch routing keeps 768 bytes of LDS of its own)
+    if (g.lds + (ind && ind->logits ? 8192 : 0) > 160 * 1024) return SMX_OK;   // (in-launch routing keeps 4.3 KB of LDS of its own)
     const bool norm = prod && prod->kind == SMX_ACT_RMSNORM;
     const unsigned units = (unsigned)(w0.nblk * upb);
     const unsigned magic = (unsigned)(((1ull << 32) + units - 1) / units);

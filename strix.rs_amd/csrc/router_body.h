@@ -23,6 +23,38 @@ __device__ __forceinline__ double rb_lane_d(double v, int l) {
     const int lo = __builtin_amdgcn_readlane((int)b, l), hi = __builtin_amdgcn_readlane((int)(b >> 32), l);
     return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
 }
+// Up to 64 experts, one per lane: the softmax probability of this lane's expert (-1 for a lane past ne).  x: the expert's
+// logit (-FLT_MAX past ne).  Every cross-lane step is a DPP move or a lane read into a scalar register (no LDS round trips).
+__device__ __forceinline__ float router_prob_lane(float x, bool live) {
+#pragma clang fp contract(off)
+    // maximum and (double) sum over the wave: a DPP tree inside each 16-lane row, then the four rows in ascending order
+    float rm = x;
+    rm = fmaxf(rm, rb_dpp<0xB1>(rm));
+    rm = fmaxf(rm, rb_dpp<0x4E>(rm));
+    rm = fmaxf(rm, rb_dpp<0x141>(rm));
+    rm = fmaxf(rm, rb_dpp<0x140>(rm));
+    const float mx = fmaxf(fmaxf(rb_lane(rm, 0), rb_lane(rm, 16)), fmaxf(rb_lane(rm, 32), rb_lane(rm, 48)));
+    const float e = live ? det_expf(x - mx) : 0.f;
+    double rs = (double)e;
+    rs += rb_dpp_d<0xB1>(rs);
+    rs += rb_dpp_d<0x4E>(rs);
+    rs += rb_dpp_d<0x141>(rs);
+    rs += rb_dpp_d<0x140>(rs);
+    const double sum = ((rb_lane_d(rs, 0) + rb_lane_d(rs, 16)) + rb_lane_d(rs, 32)) + rb_lane_d(rs, 48);
+    return live ? e / (float)sum : -1.f;
+}
+// The part of a lane's rank that the experts j0 <= j < j1 contribute: how many of them precede this lane's expert in
+// (probability descending, index ascending) order.  The parts over all j add up to the rank; rank r < k is pick r.
+__device__ __forceinline__ int router_rank_part(float p, int j0, int j1) {
+    const int lane = threadIdx.x & 63;
+    int rank = 0;
+    for (int j = j0; j < j1; j++) {   // wave-uniform bounds
+        const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), j));
+        rank += (pj > p || (pj == p && j < lane)) ? 1 : 0;
+    }
+    return rank;
+}
+
 // The router's arithmetic, run by ONE wave: v[j] = logit of expert lane + 64 j (-FLT_MAX past ne); sel: 64 floats of LDS.
 template <int PL>
 __device__ __forceinline__ void topk_router_wave(float (&v)[PL], int ne, int k, int* __restrict__ ids, float* __restrict__ w,
@@ -31,26 +63,10 @@ __device__ __forceinline__ void topk_router_wave(float (&v)[PL], int ne, int k, 
     constexpr int kRouterPerLane = PL;
     const int lane = threadIdx.x & 63;
     if constexpr (PL == 1) {
-        // Up to 64 experts, one per lane: every cross-lane step is a DPP move or a lane read into a scalar register (no
-        // LDS round trips, which dominate the time of this one-wave kernel).  A lane's rank = the number
-        // of experts that precede it in (probability descending, index ascending) order; rank r < k is pick r.
+        // Up to 64 experts, one per lane.  A lane's rank = the number of experts that precede it in (probability descending,
+        // index ascending) order; rank r < k is pick r.
         const bool live = lane < ne;
-        const float x = v[0];
-        // maximum and (double) sum over the wave: a DPP tree inside each 16-lane row, then the four rows in ascending order
-        float rm = x;
-        rm = fmaxf(rm, rb_dpp<0xB1>(rm));
-        rm = fmaxf(rm, rb_dpp<0x4E>(rm));
-        rm = fmaxf(rm, rb_dpp<0x141>(rm));
-        rm = fmaxf(rm, rb_dpp<0x140>(rm));
-        const float mx = fmaxf(fmaxf(rb_lane(rm, 0), rb_lane(rm, 16)), fmaxf(rb_lane(rm, 32), rb_lane(rm, 48)));
-        const float e = live ? det_expf(x - mx) : 0.f;
-        double rs = (double)e;
-        rs += rb_dpp_d<0xB1>(rs);
-        rs += rb_dpp_d<0x4E>(rs);
-        rs += rb_dpp_d<0x141>(rs);
-        rs += rb_dpp_d<0x140>(rs);
-        const double sum = ((rb_lane_d(rs, 0) + rb_lane_d(rs, 16)) + rb_lane_d(rs, 32)) + rb_lane_d(rs, 48);
-        const float p = live ? e / (float)sum : -1.f;
+        const float p = router_prob_lane(v[0], live);
         int rank = 0;
 #pragma unroll
         for (int j = 0; j < 64; j++) {
