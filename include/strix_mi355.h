@@ -268,7 +268,9 @@ void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
  * groups of the GEMM's tile walk); for shapes served by the row-per-wavefront GEMV (rows that
  * are not a whole number of 16-byte unit groups, or longer than 16384 elements): "gemv_rpw" (rows per
  * wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4), "gemv_lpr" (lanes per row: 16, 32,
- * 64), "gemv_wpc" (workgroups per CU).  Results do not depend on them beyond fp32 summation order. */
+ * 64), "gemv_wpc" (workgroups per CU); "host_io" (host-pointer GEMV calls: 0 = the kernels read and write the context's
+ * pinned staging buffers themselves where that is the rule, 1 = a copy command each way, 2 = a copy command in, the result
+ * written by the kernel).  Results do not depend on them beyond fp32 summation order. */
 int smx_tune(smx_ctx* ctx, const char* knob, int value);
 
 /* ---- GGUF file -> resident weights: the loader side of the path, crates/strix-models/src/gguf.rs:104-238

@@ -149,10 +149,20 @@ int matmul_host(smx_ctx* c, const char* key, const float* xs, size_t m, size_t i
         if ((rc = ensure_host(c, c->hy, yb)) != SMX_OK) return rc;
         memcpy(c->hx.p, xs, xb);
     }
-    SMX_HIP(c, hipMemcpyAsync(c->xf32.p, pinned ? (const void*)c->hx.p : (const void*)xs, xb, hipMemcpyHostToDevice, c->stream));
-    rc = run_matmul_dev(c, *w, (const float*)c->xf32.p, m, (float*)c->yf32.p, force_gemm, nullptr, nullptr);
+    // Up to 4 rows on the GEMV kernels (plain loads of x, plain stores of y): the kernel reads the pinned staging and writes the
+    // pinned result itself.  A copy command each way costs more than the kernel (measured per call with one synchronisation:
+    // kernel alone 13 us, + host-to-device copy 16, + device-to-host copy 25; kernel on the pinned buffers 17).
+    const bool gemv_path = m <= 4 && !force_gemm && !skinny_serves(*w, m);
+    // (x: one row of up to 64 KB; every workgroup reads the whole row, and several long rows read over the bus by 256
+    // workgroups cost more than the copy command: Q8_0 2560 x 9728, 3 rows, 39 - 45 us against 34)
+    const bool x_direct = pinned && gemv_path && m == 1 && xb <= (size_t(64) << 10) && c->tune_host_io != 1 && c->tune_host_io != 2;
+    const bool y_direct = pinned && gemv_path && c->tune_host_io != 1;
+    if (!x_direct)
+        SMX_HIP(c, hipMemcpyAsync(c->xf32.p, pinned ? (const void*)c->hx.p : (const void*)xs, xb, hipMemcpyHostToDevice, c->stream));
+    rc = run_matmul_dev(c, *w, x_direct ? (const float*)c->hx.p : (const float*)c->xf32.p, m, y_direct ? (float*)c->hy.p : (float*)c->yf32.p,
+                        force_gemm, nullptr, nullptr);
     if (rc != SMX_OK) return rc;
-    SMX_HIP(c, hipMemcpyAsync(pinned ? (void*)c->hy.p : (void*)y, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
+    if (!y_direct) SMX_HIP(c, hipMemcpyAsync(pinned ? (void*)c->hy.p : (void*)y, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
     if (pinned) memcpy(y, c->hy.p, yb);
     return SMX_OK;
@@ -232,7 +242,15 @@ static int gemv_batch_host(smx_ctx* c, size_t n, const char* const* keys, const 
         xo += (w->K * 4 + 255) & ~size_t(255);
         yo += (w->N * 4 + 255) & ~size_t(255);
     }
-    if (pinned && xo) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, c->hx.p, xo, hipMemcpyHostToDevice, c->stream));
+    // small batches: the kernels read the pinned staging and write the pinned results themselves (see matmul_host)
+    const bool x_direct = pinned && xo <= (size_t(64) << 10) && c->tune_host_io != 1 && c->tune_host_io != 2;
+    const bool y_direct = pinned && c->tune_host_io != 1;
+    for (size_t i = 0; i < n; i++) {
+        if (!ws[i]) continue;
+        if (x_direct) xdev[i] = (float*)(c->hx.p + ((char*)xdev[i] - c->xf32.p));
+        if (y_direct) ydev[i] = (float*)(c->hy.p + yoff[i]);
+    }
+    if (pinned && xo && !x_direct) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, c->hx.p, xo, hipMemcpyHostToDevice, c->stream));
     // consecutive items of one format and row length share a launch (up to 8 per launch)
     for (size_t i = 0; i < n;) {
         if (!ws[i]) { i++; continue; }
@@ -256,7 +274,7 @@ static int gemv_batch_host(smx_ctx* c, size_t n, const char* const* keys, const 
         i = j;
     }
     if (pinned) {
-        if (yo) SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yo, hipMemcpyDeviceToHost, c->stream));
+        if (yo && !y_direct) SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yo, hipMemcpyDeviceToHost, c->stream));
     } else {
         for (size_t i = 0; i < n; i++)
             if (ws[i] && status[i] == SMX_OK)
@@ -416,12 +434,19 @@ int smx_gemv_fused(smx_ctx* c, const char* key, int act, const float* a, const f
     if ((rc = ensure_host(c, c->hy, yb)) != SMX_OK) return rc;
     memcpy(c->hx.p, a, w->K * 4);
     if (b) memcpy(c->hx.p + w->K * 4, b, w->K * 4);
-    SMX_HIP(c, hipMemcpyAsync(a_dev, c->hx.p, xb, hipMemcpyHostToDevice, c->stream));
+    // the kernel reads the pinned staging and writes the pinned result itself (see matmul_host)
+    const bool x_direct = xb <= (size_t(64) << 10) && c->tune_host_io != 1 && c->tune_host_io != 2, y_direct = c->tune_host_io != 1;
+    if (x_direct) {
+        a_dev = (float*)c->hx.p;
+        b_dev = b ? a_dev + w->K : nullptr;
+    } else {
+        SMX_HIP(c, hipMemcpyAsync(a_dev, c->hx.p, xb, hipMemcpyHostToDevice, c->stream));
+    }
     const float* xs[1] = {a_dev};
-    float* ys[1] = {(float*)c->yf32.p};
+    float* ys[1] = {y_direct ? (float*)c->hy.p : (float*)c->yf32.p};
     const ActProd prod = {act, b_dev, eps};
     if ((rc = launch_gemv_group(c, &w, xs, ys, 1, nullptr, &prod)) != SMX_OK) return rc;
-    SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
+    if (!y_direct) SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
     SMX_HIP(c, hipStreamSynchronize(c->stream));
     memcpy(y, c->hy.p, yb);
     return SMX_OK;

@@ -401,9 +401,12 @@ int smx_gemv_f32(smx_ctx* c, const char* key, const float* x, size_t in_len, flo
         if ((rc = ensure_host(c, c->hx, xb)) != SMX_OK) return rc;
         if ((rc = ensure_host(c, c->hy, yb)) != SMX_OK) return rc;
         std::memcpy(c->hx.p, x, xb);
-        SMX_HIP(c, hipMemcpyAsync(c->xf32.p, c->hx.p, xb, hipMemcpyHostToDevice, c->stream));
-        if ((rc = launch_gemv_f32(c, w, (const float*)c->xf32.p, (float*)c->yf32.p)) != SMX_OK) return rc;
-        SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
+        // the kernel reads the pinned staging and writes the pinned result itself (see smx_gemv)
+        const bool x_direct = xb <= (size_t(64) << 10) && c->tune_host_io != 1 && c->tune_host_io != 2, y_direct = c->tune_host_io != 1;
+        if (!x_direct) SMX_HIP(c, hipMemcpyAsync(c->xf32.p, c->hx.p, xb, hipMemcpyHostToDevice, c->stream));
+        if ((rc = launch_gemv_f32(c, w, x_direct ? (const float*)c->hx.p : (const float*)c->xf32.p,
+                                  y_direct ? (float*)c->hy.p : (float*)c->yf32.p)) != SMX_OK) return rc;
+        if (!y_direct) SMX_HIP(c, hipMemcpyAsync(c->hy.p, c->yf32.p, yb, hipMemcpyDeviceToHost, c->stream));
         SMX_HIP(c, hipStreamSynchronize(c->stream));
         std::memcpy(y, c->hy.p, yb);
         return SMX_OK;

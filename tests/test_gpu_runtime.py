@@ -144,6 +144,25 @@ def test_tuning_knobs_keep_results(accel, orc, synth, relerr, pkg):
         accel.tune("gemm_walk", walk)
         assert np.array_equal(accel.prefill_q8_gemm("t.tune", xs, 1100, 1000), base), walk
     accel.tune("gemm_walk", 0)
+    # host-pointer calls: the kernels working on the pinned buffers themselves, or copy commands in front and behind: same bits
+    raw6 = synth.make_weight(14, 300, 2560, seed=15)
+    assert accel.upload_q6_k("t.tune6", raw6, 2560, 300)
+    x1, x3 = synth.make_acts(1, 512, seed=16)[0], synth.make_acts(3, 512, seed=17)
+    x6 = synth.make_acts(1, 2560, seed=18)[0]
+    want = None
+    for mode in (0, 1, 2):
+        accel.tune("host_io", mode)
+        got = (accel.gemv("t.tune", x1, 1000), accel.gemv_rows("t.tune", x3, 1000), accel.gemv_f32("t.tune", x1, 1000),
+               accel.gemv("t.tune6", x6, 300), accel.gemv_f32("t.tune6", x6, 300),
+               accel.gemv_fused("t.tune", 1, x1, None, 1000, eps=1e-6),
+               *accel.gemv_batch([("t.tune", x1), ("t.tune6", x6), ("t.tune", x3[1])], [1000, 300, 1000]))
+        if want is None:
+            want = [np.array(g).copy() for g in got]
+            assert relerr(want[0], orc.matmul_q8_from_f32(2, raw, 512, 1000, x1.reshape(1, -1))[0]) <= 1e-5
+        for g, w_ in zip(got, want):
+            assert np.array_equal(np.array(g), w_), mode
+    accel.tune("host_io", 0)
+    accel.evict("t.tune6")
     with pytest.raises(pkg.SmxError):
         accel.tune("gemv_flat", 1)          # no knob re-routes a shape to another kernel
     with pytest.raises(pkg.SmxError):
