@@ -539,6 +539,60 @@ class Bench:
                 "note": "graph_us_per_token is cache-cold (weight sets rotate); one_weight_set_us_per_token re-reads one 274 MB "
                         "set, partly from the 256 MB Infinity Cache"}
 
+    def moe_prefill_timeline(self, name, ne, hidden, eff, k, m):
+        """Start and end of every workgroup of the two grouped GEMM launches of one MoE prefill layer call (Q8_0 experts, the
+        routing of moe_prefill_m512).  Runs only when named with --only, and needs a development build of the library with the
+        kernel's timeline compiled in:  python strix.rs_amd/build.py -DSMX_GEMM_TRACE  (rebuild without the flag afterwards)."""
+        import collections
+        import ctypes
+        acc, sy = self.acc, self.synth
+        try:
+            hook = acc._L.smx_debug_gemm_trace
+        except AttributeError:
+            return {"workload": name, "skipped": "the library was built without -DSMX_GEMM_TRACE"}
+        hook.argtypes = [ctypes.c_void_p]
+        gate, up, down = sy.make_moe_q8(ne, hidden, eff, seed=3000)
+        assert acc.upload_moe_q8(0, gate, up, down, hidden, eff, ne)
+        ids, w = sy.zipf_routing(m, ne, k, seed=5)
+        plan, slot_tok, wslot = sy.group_by_expert(ids, w, ne)
+        xs = sy.make_acts(m, hidden, seed=9)
+        xd, yd, tb = acc.dev_alloc(xs.nbytes), acc.dev_alloc(xs.nbytes), acc.dev_alloc(8192 * 32)
+        acc.h2d(xd, xs)
+        for _ in range(100):   # the clock the chip sustains under this load
+            acc.moe_layer_resident(0, xd, m, plan, slot_tok, wslot, yd)
+        acc.h2d(tb, np.zeros(8192 * 4, np.uint64))
+        assert hook(tb) == 0
+        acc.moe_layer_resident(0, xd, m, plan, slot_tok, wslot, yd)
+        acc.sync()
+        t = acc.d2h(np.empty(8192 * 4, np.uint64), tb).reshape(8192, 4).copy()
+        hook(None)
+        out = {"workload": name, "shape": {"experts": ne, "hidden": hidden, "eff": eff, "top_k": k, "M": m}, "launches": {}}
+        for lname, base in (("gate_up", 4096), ("down", 0)):
+            r = t[base:base + 4096]
+            r = r[r[:, 1] > 0]
+            t0 = r[:, 0].min()
+            st, en = (r[:, 0] - t0) / 100.0, (r[:, 1] - t0) / 100.0   # us on the 100 MHz clock
+            live = (r[:, 2] & 0xffffffff).astype(int)
+            hw, xcc = r[:, 3] & 0xffffffff, (r[:, 3] >> 32) & 0xf
+            cu = ((hw >> 8) & 0xf) | (((hw >> 12) & 1) << 4) | (((hw >> 13) & 7) << 5) | (xcc << 8)
+            rec = {"workgroups": int(len(r)), "makespan_us": float(en.max()), "compute_units": len(set(cu.tolist())), "classes": {}}
+            for cname, sel in (("more_than_64_tokens", live > 64), ("33_to_64_tokens", (live > 32) & (live <= 64)), ("up_to_32_tokens", live <= 32)):
+                if sel.any():
+                    d = en[sel] - st[sel]
+                    rec["classes"][cname] = {"tiles": int(sel.sum()), "duration_us_mean_min_max": [float(d.mean()), float(d.min()), float(d.max())],
+                                             "start_us_mean_max": [float(st[sel].mean()), float(st[sel].max())], "last_end_us": float(en[sel].max())}
+            last = collections.defaultdict(float)
+            for i in range(len(r)):
+                last[cu[i]] = max(last[cu[i]], en[i])
+            ends = np.array(list(last.values()))
+            rec["last_end_per_compute_unit_us_mean_min_max"] = [float(ends.mean()), float(ends.min()), float(ends.max())]
+            rec["workgroups_running_at_us"] = {str(x): int(((st <= x) & (en > x)).sum()) for x in range(10, int(en.max()), 10)}
+            rec["workgroups_not_started_at_us"] = {str(x): int((st > x).sum()) for x in range(10, int(en.max()), 10)}
+            out["launches"][lname] = rec
+        for p_ in (xd, yd, tb):
+            acc.dev_free(p_)
+        return out
+
     # ------------------------------------------------------------------ MoE
     def moe(self, name, ne, hidden, eff, k, m, layers, steps=None, warmup=None, ty=Q8_0):
         """Decode (m == 1): rotate over `layers` resident layers (320 MB each) so expert reads are
@@ -734,6 +788,8 @@ def main():
         ("moe_decode_q6_k", lambda: b.moe("moe_decode_q6_k", 64, 2048, 768, 8, 1, layers=4, ty=Q6_K)),
         ("moe_prefill_m512_q6_k", lambda: b.moe("moe_prefill_m512_q6_k", 64, 2048, 768, 8, 512, layers=1, ty=Q6_K)),
     ]
+    if "moe_prefill_timeline" in only:   # development builds only, never part of a default run
+        plans.append(("moe_prefill_timeline", lambda: b.moe_prefill_timeline("moe_prefill_timeline", 64, 2048, 768, 8, 512)))
     for name, fn in plans:
         if want(name):
             r = fn()

@@ -53,8 +53,27 @@ struct GemmFrag {
 
 constexpr int FMT_Q8 = 0, FMT_Q4 = 1, FMT_Q6 = 2;
 
+// Optional per-workgroup timeline (development builds only: -DSMX_GEMM_TRACE; compiled out of the library): start and end of
+// every workgroup of a launch on the constant 100 MHz clock, with its live tokens and the hardware unit it ran on.
+#ifdef SMX_GEMM_TRACE
+__device__ unsigned long long* g_gemm_trace = nullptr;   // [(grouped gate/up launch: 4096) + workgroup][4]
+#define SMX_GEMM_T0 const unsigned long long smx_t0 = wall_clock64()
+#define SMX_GEMM_T1(LIVE, OP)                                                                                                  \
+    do {                                                                                                                        \
+        if (threadIdx.x == 0 && g_gemm_trace && blockIdx.x < 4096) {                                                            \
+            unsigned long long* o_ = g_gemm_trace + ((size_t)(p.nops > 1 ? 4096 : 0) + blockIdx.x) * 4;                         \
+            o_[0] = smx_t0; o_[1] = wall_clock64(); o_[2] = (unsigned long long)(LIVE) | ((unsigned long long)(OP) << 32);      \
+            o_[3] = (unsigned long long)__builtin_amdgcn_s_getreg(63492) | ((unsigned long long)__builtin_amdgcn_s_getreg(63508) << 32); \
+        }                                                                                                                       \
+    } while (0)
+#else
+#define SMX_GEMM_T0 do { } while (0)
+#define SMX_GEMM_T1(LIVE, OP) do { } while (0)
+#endif
+
 template <int FMT, bool DUMP, int NW>
 __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmArgs p) {
+    SMX_GEMM_T0;
     constexpr bool Q4 = FMT == FMT_Q4, Q6 = FMT == FMT_Q6;
     static_assert(!Q6 || NW == 4, "the Q6_K staging map is written for 256 threads");
     constexpr int SUB = Q6 ? 2 : 1;  // scaled sub-blocks per 32-block
@@ -429,7 +448,15 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
             if (tok < M_end && row < N_end) out[(size_t)tok * p.ldo + col0 + (nt_base + nt) * 32 + col] = acc[nt][i];
         }
     }
+    SMX_GEMM_T1(live_tok, op_i);
 }
+
+#ifdef SMX_GEMM_TRACE
+// buf: device memory for 8192 x 4 u64 (or null to stop); the launches that follow write their workgroups' records
+extern "C" int smx_debug_gemm_trace(void* buf) {
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_gemm_trace), &buf, sizeof(buf)) == hipSuccess ? 0 : -1;
+}
+#endif
 
 // y[i] = sum over slices z (ascending) of part[z][i]
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4* __restrict__ part, float4* __restrict__ y,
