@@ -19,6 +19,9 @@ an empty launch, a kernel that only reads the weight bytes cache-cold (the floor
 and the int8 GEMM's compute phase alone (MFMA + the two FMAs per output of exact per-block rescaling).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--only name,...] [--no-cpu]
+
+One workload never runs by default: `--only moe_prefill_timeline` reads the per-workgroup timeline of the grouped GEMM
+launches from a development build of the library (python strix.rs_amd/build.py -DSMX_GEMM_TRACE).
 """
 import ctypes
 import argparse
