@@ -66,6 +66,7 @@ class Floors:
         L = ctypes.CDLL(path)
         dp = ctypes.POINTER(ctypes.c_double)
         L.sbk_empty_launch.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, dp]
+        L.sbk_empty_launch_graph.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, dp]
         L.sbk_read_floor.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int, dp]
         L.sbk_copy.argtypes = [ctypes.c_size_t, ctypes.c_int, dp]
         L.sbk_mfma_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, dp, dp, dp]
@@ -74,6 +75,12 @@ class Floors:
     def empty_launch(self, grid, block, launches=2000):
         d = ctypes.c_double()
         assert self.L.sbk_empty_launch(grid, block, launches, ctypes.byref(d)) == 1
+        return d.value
+
+    def empty_launch_graph(self, grid, block, launches=400):
+        """the same launches inside one replayed graph: the device-side cost of a dependent launch"""
+        d = ctypes.c_double()
+        assert self.L.sbk_empty_launch_graph(grid, block, launches, ctypes.byref(d)) == 1
         return d.value
 
     def read_floor(self, nbytes, cold=True, launches=400):
@@ -104,6 +111,7 @@ def machine_floors(log):
     out = {"workload": "machine_floors",
            "method": "HIP events around back-to-back launches on one stream, like every other workload here"}
     out["empty_launch_us"] = {f"{g}x{b}": f.empty_launch(g, b) for g, b in ((1, 64), (256, 256), (256, 1024), (512, 256), (1024, 256))}
+    out["empty_launch_in_a_graph_us"] = {f"{g}x{b}": f.empty_launch_graph(g, b) for g, b in ((1, 64), (256, 1024))}
     sizes = {"14MB_q4_0_9728x2560": 14008320, "26MB_q8_0_2560x9728": 26460160, "48MB_q6_k_15360x3840": 48384000,
              "112MB_eight_q4_0_9728x2560": 8 * 14008320}
     out["read_only_cold_us"] = {k: f.read_floor(v, True, 400 if v < 1e8 else 100) for k, v in sizes.items()}
@@ -888,6 +896,8 @@ def result_line(work, warmup, cpu):
         line["roofline"]["read_only_floor_us"] = floor_us
         line["roofline"]["kernel_over_floor"] = head["kernel_avg_us"] / floor_us
         line["roofline"]["empty_launch_us"] = floors["empty_launch_us"]["256x1024"]
+        if "empty_launch_in_a_graph_us" in floors:
+            line["roofline"]["empty_launch_in_a_graph_us"] = floors["empty_launch_in_a_graph_us"]["256x1024"]
         if best_gemm:
             ceil = floors["mfma_plus_rescale_fma"]["TOPS"]
             line["gemm"]["roofline"]["rescale_ceiling_TOPS"] = ceil

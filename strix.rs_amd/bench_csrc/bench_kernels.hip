@@ -2,7 +2,8 @@
 // path, timed the same way as the path itself (HIP events around back-to-back launches on one stream).
 // Nothing here is part of the product library and the product never loads it.
 //
-//   sbk_empty_launch   back-to-back launches of a kernel that does nothing: the fixed cost of a launch
+//   sbk_empty_launch   back-to-back launches of a kernel that does nothing: the fixed cost of a launch (and, as
+//                      sbk_empty_launch_graph, of a launch inside a replayed graph)
 //                      of a given grid (what a 14 MB GEMV pays before its first byte moves)
 //   sbk_read_floor     a kernel that only reads a buffer cache-cold (rotating buffers larger than the
 //                      Infinity Cache), one xor and one store per wave: the floor of a GEMV of that size
@@ -267,6 +268,36 @@ int sbk_empty_launch(unsigned grid, unsigned block, int launches, double* us_per
     if (us < 0 || hipGetLastError() != hipSuccess) return SBK_ERR;
     *us_per_launch = us / launches;
     return SBK_OK;
+}
+
+// The same launches captured as ONE graph and replayed: what a dependent launch costs the device when no host call sits
+// between two launches (the stream figure above is bound by how fast the host submits).
+int sbk_empty_launch_graph(unsigned grid, unsigned block, int launches, double* us_per_launch) {
+    if (!us_per_launch || grid == 0 || block == 0 || block > 1024 || launches <= 0) return SBK_ERR;
+    Timer t;
+    if (!t.ok) return SBK_ERR;
+    for (int i = 0; i < 20; i++) hipLaunchKernelGGL(empty_kernel, dim3(grid), dim3(block), 0, t.s, (int*)nullptr);
+    (void)hipStreamSynchronize(t.s);
+    hipGraph_t g = nullptr;
+    hipGraphExec_t ge = nullptr;
+    if (hipStreamBeginCapture(t.s, hipStreamCaptureModeThreadLocal) != hipSuccess) return SBK_ERR;
+    for (int i = 0; i < launches; i++) hipLaunchKernelGGL(empty_kernel, dim3(grid), dim3(block), 0, t.s, (int*)nullptr);
+    if (hipStreamEndCapture(t.s, &g) != hipSuccess || !g) return SBK_ERR;
+    int rc = SBK_ERR;
+    if (hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) == hipSuccess && ge) {
+        if (hipGraphLaunch(ge, t.s) == hipSuccess && hipStreamSynchronize(t.s) == hipSuccess) {   // first replay untimed
+            t.begin();
+            const bool ok = hipGraphLaunch(ge, t.s) == hipSuccess;
+            const double us = t.end_us();
+            if (ok && us >= 0) {
+                *us_per_launch = us / launches;
+                rc = SBK_OK;
+            }
+        }
+        (void)hipGraphExecDestroy(ge);
+    }
+    (void)hipGraphDestroy(g);
+    return rc;
 }
 
 // Reads `bytes` (a multiple of 16) per launch from one of `nbuf` distinct buffers in rotation (choose
