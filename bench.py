@@ -67,6 +67,7 @@ class Floors:
         dp = ctypes.POINTER(ctypes.c_double)
         L.sbk_empty_launch.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, dp]
         L.sbk_empty_launch_graph.argtypes = [ctypes.c_uint, ctypes.c_uint, ctypes.c_int, dp]
+        L.sbk_skeleton_graph.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_uint, ctypes.c_int, dp]
         L.sbk_read_floor.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_uint, ctypes.c_uint, ctypes.c_int, ctypes.c_int, dp]
         L.sbk_copy.argtypes = [ctypes.c_size_t, ctypes.c_int, dp]
         L.sbk_mfma_valu.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, dp, dp, dp]
@@ -81,6 +82,13 @@ class Floors:
         """the same launches inside one replayed graph: the device-side cost of a dependent launch"""
         d = ctypes.c_double()
         assert self.L.sbk_empty_launch_graph(grid, block, launches, ctypes.byref(d)) == 1
+        return d.value
+
+    def skeleton_graph(self, K, rows, grid=256, launches=400):
+        """a launch that only fetches the K-float activation its predecessor wrote and stores rows outputs per workgroup,
+        inside one replayed graph: the part of a dependent GEMV launch that is not weight traffic"""
+        d = ctypes.c_double()
+        assert self.L.sbk_skeleton_graph(K, rows, grid, launches, ctypes.byref(d)) == 1
         return d.value
 
     def read_floor(self, nbytes, cold=True, launches=400):
@@ -112,6 +120,7 @@ def machine_floors(log):
            "method": "HIP events around back-to-back launches on one stream, like every other workload here"}
     out["empty_launch_us"] = {f"{g}x{b}": f.empty_launch(g, b) for g, b in ((1, 64), (256, 256), (256, 1024), (512, 256), (1024, 256))}
     out["empty_launch_in_a_graph_us"] = {f"{g}x{b}": f.empty_launch_graph(g, b) for g, b in ((1, 64), (256, 1024))}
+    out["dependent_launch_skeleton_in_a_graph_us"] = {"2560_in_9728_out": f.skeleton_graph(2560, 38), "9728_in_9728_out": f.skeleton_graph(9728, 38)}
     sizes = {"14MB_q4_0_9728x2560": 14008320, "26MB_q8_0_2560x9728": 26460160, "48MB_q6_k_15360x3840": 48384000,
              "112MB_eight_q4_0_9728x2560": 8 * 14008320}
     out["read_only_cold_us"] = {k: f.read_floor(v, True, 400 if v < 1e8 else 100) for k, v in sizes.items()}

@@ -49,6 +49,21 @@ __global__ __launch_bounds__(1024) void empty_kernel(int* p) {
     if (p && threadIdx.x == 0xffffff) *p = 1;   // never true: the kernel has a body the compiler keeps
 }
 
+// The skeleton of a dependent GEMV launch: every workgroup fetches the K-float activation that the launch in front of it
+// wrote, meets at a barrier and stores `rows` outputs, which the next launch reads as its activation.
+__global__ __launch_bounds__(1024) void skeleton_kernel(const float* __restrict__ x, float* __restrict__ y, int K, int rows) {
+    __shared__ float red[1024];
+    float s = 0.f;
+    for (int i = threadIdx.x; i < K / 4; i += 1024) {
+        const float4 v = ((const float4*)x)[i];
+        s += v.x + v.y + v.z + v.w;
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    s = red[(threadIdx.x * 7) & 1023];
+    if ((int)threadIdx.x < rows) y[blockIdx.x * rows + threadIdx.x] = s * 0.f + 1.f;
+}
+
 // Workgroup b reads units [b * per_wg, (b + 1) * per_wg) of 16 bytes; wave w takes 64-unit loads
 // w, w + nw, ... of that slab, UNR loads requested before the first is used.  Lanes past the end re-read
 // the slab's last unit (no conditional loads).
@@ -297,6 +312,48 @@ int sbk_empty_launch_graph(unsigned grid, unsigned block, int launches, double* 
         (void)hipGraphExecDestroy(ge);
     }
     (void)hipGraphDestroy(g);
+    return rc;
+}
+
+// `launches` skeleton launches (grid workgroups x 1024 threads, K-float activation, rows outputs per workgroup; grid * rows
+// >= K), each reading what the one in front wrote, as one replayed graph: microseconds per launch.
+int sbk_skeleton_graph(int K, int rows, unsigned grid, int launches, double* us_per_launch) {
+    if (!us_per_launch || K <= 0 || K % 4 != 0 || rows <= 0 || rows > 1024 || grid == 0 || (size_t)grid * rows < (size_t)K || launches <= 0)
+        return SBK_ERR;
+    Timer t;
+    if (!t.ok) return SBK_ERR;
+    float *a = nullptr, *b = nullptr;
+    const size_t bytes = (size_t)grid * rows * 4;
+    if (hipMalloc(&a, bytes) != hipSuccess || hipMalloc(&b, bytes) != hipSuccess || hipMemset(a, 0, bytes) != hipSuccess ||
+        hipMemset(b, 0, bytes) != hipSuccess) {
+        if (a) (void)hipFree(a);
+        if (b) (void)hipFree(b);
+        return SBK_ERR;
+    }
+    auto launch = [&](int i) { hipLaunchKernelGGL(skeleton_kernel, dim3(grid), dim3(1024), 0, t.s, (i & 1) ? b : a, (i & 1) ? a : b, K, rows); };
+    for (int i = 0; i < 20; i++) launch(i);
+    (void)hipStreamSynchronize(t.s);
+    hipGraph_t g = nullptr;
+    hipGraphExec_t ge = nullptr;
+    int rc = SBK_ERR;
+    if (hipStreamBeginCapture(t.s, hipStreamCaptureModeThreadLocal) == hipSuccess) {
+        for (int i = 0; i < launches; i++) launch(i);
+        if (hipStreamEndCapture(t.s, &g) == hipSuccess && g && hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) == hipSuccess && ge) {
+            if (hipGraphLaunch(ge, t.s) == hipSuccess && hipStreamSynchronize(t.s) == hipSuccess) {
+                t.begin();
+                const bool ok = hipGraphLaunch(ge, t.s) == hipSuccess;
+                const double us = t.end_us();
+                if (ok && us >= 0) {
+                    *us_per_launch = us / launches;
+                    rc = SBK_OK;
+                }
+            }
+            (void)hipGraphExecDestroy(ge);
+        }
+        if (g) (void)hipGraphDestroy(g);
+    }
+    (void)hipFree(a);
+    (void)hipFree(b);
     return rc;
 }
 
