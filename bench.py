@@ -157,6 +157,7 @@ class Bench:
         self.synth = _load("strix_rs_amd_synth", os.path.join(pkg_dir, "synth.py"))
         self.acc = self.pkg.Mi355WeightAccel(0)
         self.steps, self.warmup = steps, warmup
+        self.settle_ms = 30.0   # untimed replays of a workload's graph before its timed region (not the headline's)
 
     def log(self, *a):
         print(*a, file=sys.stderr, flush=True)
@@ -185,7 +186,7 @@ class Bench:
         wall_ms = (time.perf_counter() - t0) * 1e3
         return ms, wall_ms
 
-    def _timed_queued(self, fn, steps, warmup, settle_ms=30.0):
+    def _timed_queued(self, fn, steps, warmup, settle_ms=None):
         """The K steps timed as ONE captured graph of the K calls, launched once between two events: the device runs them
         back to back however fast the host enqueued them.  This is the timed region of every decode workload.  A 5 us
         step is at the edge of what a Python caller submits per call (4.4-7.7 us per call across hosts; on a slow one a
@@ -201,6 +202,7 @@ class Bench:
         acc.sync()
         # settle_ms (workloads other than the headline): further untimed replays until the chip has run this load for that
         # long; under a bandwidth-heavy load it takes 20-30 ms to reach the clocks it then sustains (lm_head: 149 -> 141 us)
+        settle_ms = self.settle_ms if settle_ms is None else settle_ms
         t_settle = time.perf_counter()
         for _ in range(40):
             if (time.perf_counter() - t_settle) * 1e3 >= settle_ms:
@@ -260,7 +262,7 @@ class Bench:
         out["note"] = "host-pointer trait calls, PCIe and one sync per call included"
         return out
 
-    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False, trait=False, settle_ms=30.0):
+    def gemv(self, name, ty, N, K, m, min_total_bytes, steps=None, warmup=None, f32=False, trait=False, settle_ms=None):
         """m rows against rotating weight copies.  m <= 4: the dot4 GEMV (quantiser fused for m = 1); 5..64 rows of a
         Q8_0 / Q4_0 weight: the small-batch kernel on the matrix cores; f32: the fp32-activation GEMV (no quantiser)."""
         acc, sy = self.acc, self.synth
@@ -759,6 +761,7 @@ def main():
     ap.add_argument("--only", default="", help="comma-separated workload names (default: all)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-floors", action="store_true", help="skip the measurement-only kernels (empty launch, read floor, MFMA+FMA ceiling)")
+    ap.add_argument("--settle-ms", type=float, default=30.0, help="untimed graph replays of every workload but the headline until the chip has run it this long (0: one replay)")
     ap.add_argument("--no-trait", action="store_true", help="skip the host-pointer trait-call timing of the headline workload (keeps a kernel trace of the run to the timed launches)")
     ap.add_argument("--records", default=os.path.join(ROOT, "bench_workloads.json"), help="where the per-workload records are written")
     ap.add_argument("--no-headline", action="store_true", help="skip the headline GEMV when --only names other workloads")
@@ -770,6 +773,7 @@ def main():
     only = set(filter(None, a.only.split(",")))
     want = lambda n: not only or n in only
     b = Bench(a.steps, a.warmup)
+    b.settle_ms = a.settle_ms
     b.log("device:", b.acc.name())
     for kv in filter(None, a.tune.split(",")):
         knob, value = kv.split("=")
