@@ -123,7 +123,8 @@ def machine_floors(log):
     out["dependent_launch_skeleton_in_a_graph_us"] = {"2560_in_9728_out": f.skeleton_graph(2560, 38), "9728_in_9728_out": f.skeleton_graph(9728, 38)}
     sizes = {"14MB_q4_0_9728x2560": 14008320, "26MB_q8_0_2560x9728": 26460160, "48MB_q6_k_15360x3840": 48384000,
              "112MB_eight_q4_0_9728x2560": 8 * 14008320}
-    out["read_only_cold_us"] = {k: f.read_floor(v, True, 400 if v < 1e8 else 100) for k, v in sizes.items()}
+    # (the faster of two passes: the first measurement of a process may still run at rising clocks)
+    out["read_only_cold_us"] = {k: min(f.read_floor(v, True, 400 if v < 1e8 else 100) for _ in range(2)) for k, v in sizes.items()}
     out["read_only_cold_GBps"] = {k: sizes[k] / out["read_only_cold_us"][k] / 1e3 for k in sizes}
     out["read_only_hot_us"] = {"14MB_q4_0_9728x2560": f.read_floor(14008320, False)}
     us = f.copy(256 << 20)
