@@ -243,7 +243,11 @@ static int gemv_batch_host(smx_ctx* c, size_t n, const char* const* keys, const 
         yo += (w->N * 4 + 255) & ~size_t(255);
     }
     // small batches: the kernels read the pinned staging and write the pinned results themselves (see matmul_host)
-    const bool x_direct = pinned && xo <= (size_t(64) << 10) && c->tune_host_io != 1 && c->tune_host_io != 2;
+    // (every item's row is read by that item's workgroups only: rows of up to 64 KB each)
+    size_t x_longest = 0;
+    for (size_t i = 0; i < n; i++)
+        if (ws[i]) x_longest = std::max(x_longest, ws[i]->K * 4);
+    const bool x_direct = pinned && x_longest <= (size_t(64) << 10) && c->tune_host_io != 1 && c->tune_host_io != 2;
     const bool y_direct = pinned && c->tune_host_io != 1;
     for (size_t i = 0; i < n; i++) {
         if (!ws[i]) continue;
