@@ -238,7 +238,7 @@ int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nbl
         return launch_flat_fq<Ops, 1, PRE, GL, 1>(c, g, J, njobs, nblk, m);                          \
     }
         if constexpr (std::is_same<Ops, OpsQ4_0>::value || std::is_same<Ops, OpsQ8_0>::value) {
-            SMX_FLAT(3, 16) SMX_FLAT(3, 8)
+            SMX_FLAT(3, 16) SMX_FLAT(3, 8) SMX_FLAT(2, 16) SMX_FLAT(4, 16)
         } else if constexpr (kQ6) {
             SMX_FLAT(1, 16) SMX_FLAT(1, 8) SMX_FLAT(1, 4)
         }
@@ -316,6 +316,19 @@ int launch_type(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nbl
 // per 16 waves), persistent workgroups looping over chunks, lanes-per-row chosen to waste the fewest
 // lanes on short rows, and for weights with few, long rows the passes of a row are split over 2 or
 // 4 waves (K-split) so every SIMD has work.
+// Loads per round of the flat form (Q4_0 / Q8_0, one activation row, 16-lane groups).  A wave takes L = units of the
+// workgroup / 64 / 16 loads in rounds of PRE, each round one trip to memory; a last round of a single load costs as much as a
+// full one.  Measured (cold, in a graph): Q4_0 8192 x 2048 gate/up pair (L = 4) 7.56 / 6.79 / 7.66 us with 3 / 2 / 4 per round
+// and its single GEMV (L = 2) 4.16 / 4.10 / 4.19; Q8_0 8192 x 2048 single (L = 4) 5.68 / 5.23 / 5.37, pair (L = 8) 9.6 / 9.2 / 9.7;
+// Q4_0 14336 x 4096 single (L = 7) 7.98 / 7.85 / 7.72; Q4_0 9728 x 2560 single (L = 3) 4.89 / 5.11 / 4.95, pair (L = 6) 8.47 / 8.45 / 9.26.
+static int pick_flat_pre(size_t units_per_wg) {
+    const int L = (int)((((units_per_wg + 63) / 64) + 15) / 16);
+    if (L % 3 == 0) return 3;
+    if (L % 2 == 0) return 2;
+    if (L % 3 == 2) return 3;
+    return L >= 7 ? 4 : 3;   // 7 = 4 + 3; a single load either way
+}
+
 static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int mt, bool dump, int njobs) {
     Geom g;
     size_t tokb, units;
@@ -401,6 +414,7 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
             // Q6_K 15360 x 3840 (five load instructions per unit) 11.4 / 12.5 / 14.1 / 14.8 us with 1 / 2 / 3 / 4,
             // eight rows on Q8_0 2560 x 9728 14.1-14.6 / 14.8 / 15.8 us with 1 / 2 / 3
             g.flat_pre = type == kQ6_K ? 1 : (mt == 1 ? 3 : 1);
+            if (mt == 1 && type != kQ6_K && g.flat == 16) g.flat_pre = pick_flat_pre(rows * units);
             g.nt = 1024;
             g.grid = (unsigned)fwgs;
             g.lds = lds;
@@ -578,6 +592,7 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
     const size_t upb = w0.type == kQ6_K ? 4 : (w0.type == kQ8_0 ? 2 : 1);
     const size_t rows = (w0.N + g.grid - 1) / g.grid;
     g.lds += rows * w0.nblk * upb / g.flat * 4;
+    if (w0.type != kQ6_K && g.flat == 16) g.flat_pre = pick_flat_pre(2 * rows * w0.nblk * upb);   // both weights' units in one sequence
     if (g.lds + (ind && ind->logits ? 8192 : 0) > 160 * 1024) return SMX_OK;   // (in-launch routing keeps 4.3 KB of LDS of its own)
     const bool norm = prod && prod->kind == SMX_ACT_RMSNORM;
     const unsigned units = (unsigned)(w0.nblk * upb);
@@ -596,8 +611,8 @@ int launch_gemv_dual(smx_ctx* c, const Weight* const* wg, const Weight* const* w
     if (g.flat_pre == PRE && g.flat == GL)                                                                      \
         return ind ? (ind->logits ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 1, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1, 1>)) \
                    : (norm ? go(gemv_flat_dual_kernel<OPS, PRE, GL, 2>) : go(gemv_flat_dual_kernel<OPS, PRE, GL, 1>));
-    if (w0.type == kQ4_0) { SMX_DUAL(OpsQ4_0, 3, 16) SMX_DUAL(OpsQ4_0, 3, 8) }
-    else if (w0.type == kQ8_0) { SMX_DUAL(OpsQ8_0, 3, 16) SMX_DUAL(OpsQ8_0, 3, 8) }
+    if (w0.type == kQ4_0) { SMX_DUAL(OpsQ4_0, 3, 16) SMX_DUAL(OpsQ4_0, 3, 8) SMX_DUAL(OpsQ4_0, 2, 16) SMX_DUAL(OpsQ4_0, 4, 16) }
+    else if (w0.type == kQ8_0) { SMX_DUAL(OpsQ8_0, 3, 16) SMX_DUAL(OpsQ8_0, 3, 8) SMX_DUAL(OpsQ8_0, 2, 16) SMX_DUAL(OpsQ8_0, 4, 16) }
     else { SMX_DUAL(OpsQ6_K, 1, 16) SMX_DUAL(OpsQ6_K, 1, 8) SMX_DUAL(OpsQ6_K, 1, 4) }
 #undef SMX_DUAL
     return SMX_OK;   // no variant for this geometry: not served
