@@ -933,6 +933,12 @@ __device__ __forceinline__ void gemv_body_flat(const GemvW W, const GemvX X, flo
             c_t += 16;
         }
     };
+    // A long activation row (8192 elements or more) is several loads per thread on the first ten waves, and the weight loads
+    // of the waves that carry none of it would reach the CU's memory pipeline first and hold the row back behind cold HBM
+    // traffic (the staging barrier then fell 2.8 us after the launch instead of 1.4): there the waves meet once before the
+    // first weight request, so that the row's loads lead the queue.  Q4_0 / Q8_0 2560 x 9728 5.98 / 7.71 -> 5.4 / 7.3 us; on
+    // shorter rows the wait for the last wave to start costs more than it brings (cfg1 +0.15 us) and is left out.
+    if (MT == 1 && Ops::nb32(nblk) >= 256) __builtin_amdgcn_s_barrier();
     request();
     if (MT == 1) xs.store(smem, nblk, X);
     else if (kRowsF) xf.store(smem, tokb, nblk);

@@ -79,9 +79,12 @@ def test_flat_gemv_waits_for_the_activation_only(tmp_path):
            "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only", os.path.join(ROOT, "strix.rs_amd", "csrc", "gemv.hip"), "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True, timeout=900)
     ins = _kernel_lines(out.read_text(), "_ZN3smx16gemv_flat_kernelINS_7OpsQ4_0ELi1ELi3ELi16ELi1ELb0ELb0EEE")
-    barrier = next(i for i, l in enumerate(ins) if l.startswith("s_barrier"))
+    is_weight = lambda l: l.startswith(("global_load_ushort", "global_load_dwordx4 v")) and l.split()[-1] == "off"   # the activation's loads use the scalar base form
+    first_weight = next(i for i, l in enumerate(ins) if is_weight(l))
+    # the staging barrier: the first one behind the weight requests (a long row has the waves meet once in front of them)
+    barrier = next(i for i, l in enumerate(ins) if i > first_weight and l.startswith("s_barrier"))
     loads = [i for i, l in enumerate(ins[:barrier]) if l.startswith("global_load")]
-    weight_loads = [i for i in loads if ins[i].startswith(("global_load_ushort", "global_load_dwordx4 v")) and ins[i].split()[-1] == "off"]      # the activation's loads use the scalar base form
+    weight_loads = [i for i in loads if is_weight(ins[i])]
     assert len(weight_loads) == 6                      # three units: 16 bytes of quants + one f16 scale each
     last_weight = weight_loads[-1]
     assert any(i < weight_loads[0] for i in loads)     # the activation is requested first
