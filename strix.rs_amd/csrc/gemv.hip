@@ -406,7 +406,7 @@ static Geom pick_geom(const smx_ctx* c, QType type, size_t N, size_t nblk, int m
         for (;; rounds++) {
             fwgs = std::min(N, cus * rounds);
             rows = (N + fwgs - 1) / fwgs;                          // of the workgroup with the most rows
-            lds = tokb * (size_t)mt + rows * units / g.flat * 4 * mt;
+            lds = tokb * (size_t)mt + std::max<size_t>(rows * units / g.flat * 4 * mt, 128);   // (128: the rmsnorm reduction's sixteen wave sums)
             if (lds <= 128 * 1024 || fwgs == N) break;
         }
         if (rows * units < 65536 && lds <= 160 * 1024) {

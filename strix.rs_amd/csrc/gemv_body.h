@@ -709,7 +709,7 @@ struct FlatX {
         }
     }
 
-    // `tok`: the row's LDS area (also the scratch of the rmsnorm reduction); every thread of the
+    // `tok`: the row's LDS area (the rmsnorm reduction's scratch are the 128 bytes behind it); every thread of the
     // 1024-thread workgroup calls this.
     __device__ __forceinline__ void store(char* tok, int nblk, const GemvX& X) {
         const int nb32 = Ops::nb32(nblk);
@@ -745,12 +745,13 @@ struct FlatX {
                     ss += (double)v[j].w * (double)v[j].w;
                 }
                 ss = wave_sum_d(ss);
-                double* red = (double*)tok;
+                // the sixteen wave sums meet behind the row's own LDS area (where the group sums go once the weights are
+                // consumed): nothing the quantiser writes below touches them, so one barrier is enough
+                double* red = (double*)(tok + Ops::tok_bytes(nblk));
                 if ((i & 63) == 63) red[i >> 6] = ss;
                 __syncthreads();
                 double tot = 0.0;
                 for (int w = 0; w < 16; w++) tot += red[w];
-                __syncthreads();
                 const float rs = (float)(1.0 / sqrt(tot / (double)(nb32 * 32) + (double)X.eps));
                 if ((i & ~63) >= nb32 * 2) return;   // whole waves
                 float4 w4[4];
