@@ -265,7 +265,7 @@ void smx_graph_destroy(smx_ctx* ctx, smx_graph* g);
  * call it): launch-geometry overrides for sweeps; value 0 restores the built-in choice.  They shape
  * a kernel's launch, never which kernel a shape is served by.
  * Knobs: "gemm_splitk" (K slices of the GEMM), "gemm_tile_m" (tokens per GEMM tile: 64 or 128), "gemm_walk" (token-tile
- * groups of the GEMM's tile walk); for shapes served by the row-per-wavefront GEMV (rows that
+ * groups of the GEMM's tile walk), "gemm_narrow" (1: every weight strip of the GEMM 128 rows; 1 + n: the first n strips 96 rows); for shapes served by the row-per-wavefront GEMV (rows that
  * are not a whole number of 16-byte unit groups, or longer than 16384 elements): "gemv_rpw" (rows per
  * wavefront: 1, 2, 4), "gemv_ks" (wavefronts sharing a row: 1, 2, 4), "gemv_lpr" (lanes per row: 16, 32,
  * 64), "gemv_wpc" (workgroups per CU); "host_io" (host-pointer GEMV calls: 0 = the kernels read and write the context's

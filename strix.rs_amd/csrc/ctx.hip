@@ -569,6 +569,9 @@ int smx_tune(smx_ctx* c, const char* knob, int value) {
     } else if (k == "gemm_walk") {
         if (value > 64) return fail(c, SMX_ERR_ARG, "tune: gemm_walk must be 0..64");
         c->tune_gemm_walk = value;   // token-tile groups of the GEMM's tile walk (0: chosen from the L2 size)
+    } else if (k == "gemm_narrow") {
+        if (value > 1025) return fail(c, SMX_ERR_ARG, "tune: gemm_narrow must be 0 (rule), 1 (none) or 1 + the number of 96-row strips");
+        c->tune_gemm_narrow = value;
     } else if (k == "host_io") {
         if (value > 2) return fail(c, SMX_ERR_ARG, "tune: host_io must be 0 (kernels on the pinned buffers), 1 (copy commands both ways) or 2 (copy in, result direct)");
         c->tune_host_io = value;

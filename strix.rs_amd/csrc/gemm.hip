@@ -97,6 +97,17 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         t /= p.nops;
         const GemmTile tl = p.tiles[t];
         tok0 = tl.tok0; M_end = tl.tok_end; row0 = tl.row0; N_end = tl.row_end; col0 = tl.col0;
+    } else if (p.narrow) {
+        // mixed strips: the 128-row strips (rows from 96 * narrow on) strip by strip, then the 96-row strips (rows 0 ..), so
+        // that the launch's last, partly filled round of workgroups is made of the shorter tiles
+        const int full = (p.tiles_n - p.narrow) * p.tiles_m;
+        const bool nar = t >= full;
+        const int u = nar ? t - full : t;
+        const int tn = u / p.tiles_m, tm = u - tn * p.tiles_m;
+        tok0 = tm * p.tile_m; M_end = min(p.M, tok0 + p.tile_m);
+        row0 = nar ? tn * 96 : p.narrow * 96 + tn * BN;
+        N_end = nar ? row0 + 96 : p.N;
+        col0 = row0;
     } else {
         const int T = p.tiles_m * p.tiles_n;
         if (p.xcd_remap) t = (t & 7) * (T >> 3) + (t >> 3);
@@ -113,7 +124,9 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
     // 32 tokens and ONE row tile; <= 64 tokens: two waves per token half, two row tiles each.
     const int live_tok = M_end - tok0;
     const int tw = NW == 4 ? (live_tok <= 32 ? 0 : live_tok <= 64 ? (wave & 1) : wave) : wave;   // token sub-tile
-    const int nt_cnt = NW == 4 ? (live_tok <= 32 ? 1 : live_tok <= 64 ? 2 : 4) : 4;              // row tiles of this wave
+    const int live_rows = min(N_end - row0, BN);
+    const int full_cnt = (live_rows + 31) >> 5;   // a tile at the end of N, or a 96-row strip: only the row tiles that exist
+    const int nt_cnt = NW == 4 ? (live_tok <= 32 ? 1 : live_tok <= 64 ? 2 : full_cnt) : full_cnt;   // row tiles of this wave
     const int nt_base = NW == 4 ? (live_tok <= 32 ? wave : live_tok <= 64 ? (wave >> 1) * 2 : 0) : 0;
 
     const int nstage_total = (p.nb + KB - 1) / KB;
@@ -190,7 +203,7 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         } else if (!Q4) {
 #pragma unroll
             for (int ps = 0; ps < BG; ps++)
-                load_to_lds16(op.wquants, b_off[ps] + koff, sB + ps * NW * GRP);
+                if ((ps * NW + wave) * 8 < live_rows) load_to_lds16(op.wquants, b_off[ps] + koff, sB + ps * NW * GRP);
         } else {
             const int bq = min(blk0 + q_bi, p.nb - 1);
 #pragma unroll
@@ -551,13 +564,58 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     int Z = (dump || (m * w.N) % 4 != 0) ? 1 : (c->tune_gemm_splitk > 0 ? std::min(c->tune_gemm_splitk, nstages) : pick_splitk(slots, T, nstages));
     p.stages_per_slice = (nstages + Z - 1) / Z;
     Z = (nstages + p.stages_per_slice - 1) / p.stages_per_slice;
+    // Mixed strips.  When the tiles need several rounds of the chip's workgroup slots and the last round is partly filled,
+    // its idle slots cost up to a whole tile's time.  A tile of 96 weight rows runs three of the four row tiles (about 0.8
+    // of the time), so with the first `narrow` strips of N cut at 96 rows and dispatched last, the last round can be made
+    // of shorter tiles on more slots: 15360 rows x 2048 tokens = 1920 tiles = 3.75 rounds of 512 becomes 1536 tiles of
+    // 128 rows (3 rounds) and one round of 512 tiles of 96.  Chosen by the estimated makespan; taken when it saves 3 %.
+    if (Z == 1 && bm == 128 && !dump && c->tune_gemm_narrow != 1) {
+        const auto makespan = [&](int b) -> double {   // in 128-row tile times; -1: N does not split that way
+            if (96 * b > p.N) return -1.0;
+            const int a = (p.N - 96 * b + BN - 1) / BN;
+            const long full = (long)a * p.tiles_m, nar = (long)b * p.tiles_m;
+            const double c96 = 0.80;
+            const long q = full / slots, r = full % slots;
+            if (nar == 0) return (double)(q + (r ? 1 : 0));
+            // narrow tiles go to the slots that are free at q first, then in turn to whichever frees first
+            double t_a = (double)q, t_b = (double)q + 1.0;   // slots - r slots free at t_a, r slots at t_b
+            long n_a = slots - r, n_b = r, left = nar;
+            double end = r ? t_b : t_a;
+            while (left > 0) {
+                const bool use_a = n_b == 0 || (n_a > 0 && t_a <= t_b);
+                const long n = std::min(left, use_a ? n_a : n_b);
+                double& tt = use_a ? t_a : t_b;
+                if (n < (use_a ? n_a : n_b)) { end = std::max(end, tt + c96); break; }   // the rest of this group stays free
+                tt += c96;
+                end = std::max(end, tt);
+                left -= n;
+            }
+            return end;
+        };
+        int best_b = 0;
+        if (c->tune_gemm_narrow > 1) {
+            best_b = std::min(c->tune_gemm_narrow - 1, p.N / 96);
+        } else if (T > slots) {
+            double best = makespan(0);
+            const double need = 0.97 * best;
+            for (int b = 1; (long)b * p.tiles_m <= slots && 96 * b <= p.N; b++) {
+                const double t = makespan(b);
+                if (t > 0 && t < best && t <= need) { best = t; best_b = b; }
+            }
+        }
+        if (best_b > 0) {
+            p.narrow = best_b;
+            p.tiles_n = best_b + (p.N - 96 * best_b + BN - 1) / BN;
+        }
+    }
+    const int T_launch = p.tiles_m * p.tiles_n;
     p.op[0].out = y;
     if (Z > 1) {
         int rc = ensure(c, c->work, (size_t)Z * m * w.N * 4);
         if (rc != SMX_OK) return rc;
         p.op[0].out = (float*)c->work.p;
     }
-    const dim3 grid((unsigned)T, 1, (unsigned)Z);
+    const dim3 grid((unsigned)T_launch, 1, (unsigned)Z);
     {
         ProfScope ps(c, w.type == kQ4_0 ? "gemm_i8_q4_0" : w.type == kQ6_K ? "gemm_i8_q6_k" : "gemm_i8_q8_0");
         int rc;

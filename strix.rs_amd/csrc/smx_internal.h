@@ -79,7 +79,7 @@ struct smx_ctx {
     hipEvent_t htab_done = nullptr;  // recorded after the last copy out of htab (null: htab is free)
 
     // tuning overrides (0 = automatic)
-    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_tile_m = 0, tune_gemm_walk = 0, tune_host_io = 0;
+    int tune_gemv_rpw = 0, tune_gemv_ks = 0, tune_gemv_wpc = 0, tune_gemv_lpr = 0, tune_gemm_splitk = 0, tune_gemm_tile_m = 0, tune_gemm_walk = 0, tune_host_io = 0, tune_gemm_narrow = 0;
 
     // dynamic-LDS limit already raised on this context's device, per kernel (see set_dyn_lds): a fixed
     // open-addressing table, so that a launch never allocates host memory
@@ -196,6 +196,7 @@ struct GemmArgs {
     int xcd_remap;
     int walk_gm;            // dense tiling: token tiles per group of the tile walk (see launch_gemm)
     int nops;               // grouped launches: operands per tile (workgroup x serves tile x / nops, operand x % nops)
+    int narrow;             // dense tiling: the first `narrow` weight strips have 96 rows and are dispatched last (see launch_gemm)
 };
 
 // ---- launchers (all enqueue on c->stream; return SMX_OK or an error) ----

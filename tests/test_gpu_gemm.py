@@ -80,6 +80,27 @@ def test_gemm_64_token_tiles(accel, orc, synth, relerr, ty, M, N, K):
     accel.evict("t.t64")
 
 
+@pytest.mark.parametrize("ty,M,N,K", [(8, 200, 416, 512), (2, 130, 1000, 640), (14, 150, 330, 512), (8, 129, 96, 256), (8, 300, 100, 96)])
+def test_gemm_96_row_strips(accel, orc, synth, relerr, ty, M, N, K):
+    """A launch whose last round of workgroups would be partly filled cuts the first weight strips at 96 rows; the knob
+    forces any number of them on any shape (N a whole number of strips or ragged, one strip only, more asked for than fit).
+    Same integers, same fp32 association per output: bit-equal to the plain tiling."""
+    raw = synth.make_weight(ty, N, K, seed=M + N)
+    assert getattr(accel, UPLOAD[ty])("t.n96", raw, K, N)
+    xs = synth.make_acts(M, K, seed=N)
+    ref = orc.matmul_q8_from_f32(ty, raw, K, N, xs)
+    accel.tune("gemm_splitk", 1)
+    accel.tune("gemm_narrow", 1)
+    plain = accel.prefill_q8_gemm("t.n96", xs, M, N)
+    assert relerr(plain, ref) <= TOL
+    for n in (1, 2, 3, 1000):
+        accel.tune("gemm_narrow", 1 + n)
+        assert np.array_equal(accel.prefill_q8_gemm("t.n96", xs, M, N), plain), n
+    accel.tune("gemm_narrow", 0)
+    accel.tune("gemm_splitk", 0)
+    accel.evict("t.n96")
+
+
 def test_gemm_declines_and_errors(accel, synth, pkg):
     assert accel.prefill_q8_gemm("t.absent", np.zeros((2, 64), np.float32), 2, 8) is None
     raw = synth.make_weight(8, 8, 256, seed=1)
