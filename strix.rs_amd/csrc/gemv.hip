@@ -244,6 +244,11 @@ int launch_flat(smx_ctx* c, const Geom& g, const GemvJobs& J, int njobs, int nbl
         }
 #undef SMX_FLAT
     } else if constexpr (!(kQ6 && MT == 8)) {
+        if constexpr (MT <= 4 && !kQ6) {   // fp32 rows quantised by the kernel, two loads per round
+            if constexpr (MT == 2 && std::is_same<Ops, OpsQ8_0>::value) {
+                if (g.rowsf && g.flat == 16 && g.flat_pre == 2) return launch_flat_fq<Ops, MT, 2, 16, 1>(c, g, J, njobs, nblk, m);
+            }
+        }
         // several rows arrive quantised
         constexpr int PRE = 1;
         if (g.flat_pre == PRE) {
@@ -462,6 +467,10 @@ int launch_gemv(smx_ctx* c, const Weight& w, const float* x, size_t m, float* y,
     // 2..4 rows of at most 49152 values in all: the flat kernel quantises them itself (up to three half blocks per thread), which
     // saves the quantiser launch; longer rows are quantised once for all workgroups by their own launch
     g.rowsf = mt > 1 && mt <= 4 && g.flat && !dump && (size_t)mt * w.K <= 49152;
+    // Two rows of a Q8_0 weight (a unit is one 16-byte load there): two loads per round.  Measured with 1 / 2 / 3 / 4 per round:
+    // 2560 x 9728 9.60 / 9.15 / 9.15 / 9.45 us, 9728 x 2560 8.30 / 7.64 / 7.48 / 7.96, 4096 x 4096 6.76 / 6.14 / 6.63 / 6.58.  Q4_0 and three
+    // or four rows (bound by the staging of the rows and the LDS reads of four rows per unit) lose 0 .. 8 % with more than one.
+    if (g.rowsf && w.type == kQ8_0 && mt == 2 && g.flat == 16) g.flat_pre = 2;
     if (mt > 1 && !g.rowsf) {
         // each of the persistent workgroups would repeat the quantiser for all m rows: do it once instead
         int rc;
