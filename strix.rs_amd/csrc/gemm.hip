@@ -97,25 +97,24 @@ __global__ __launch_bounds__(64 * NW, NW == 8 ? 1 : 2) void gemm_i8_kernel(GemmA
         t /= p.nops;
         const GemmTile tl = p.tiles[t];
         tok0 = tl.tok0; M_end = tl.tok_end; row0 = tl.row0; N_end = tl.row_end; col0 = tl.col0;
-    } else if (p.narrow) {
-        // mixed strips: the 128-row strips (rows from 96 * narrow on) strip by strip, then the 96-row strips (rows 0 ..), so
-        // that the launch's last, partly filled round of workgroups is made of the shorter tiles
-        const int full = (p.tiles_n - p.narrow) * p.tiles_m;
-        const bool nar = t >= full;
-        const int u = nar ? t - full : t;
-        const int tn = u / p.tiles_m, tm = u - tn * p.tiles_m;
+    } else {
+        // The first `narrow` strips of N are 96 rows high and dispatched last (see launch_gemm); each part (128-row strips,
+        // 96-row strips) is walked on its own.
+        const int full_strips = p.tiles_n - p.narrow;
+        const int t_full = full_strips * p.tiles_m;
+        const bool nar = t >= t_full;   // never without narrow strips
+        if (nar) t -= t_full;
+        const int ns = nar ? p.narrow : full_strips;
+        const int T = ns * p.tiles_m;
+        if (p.xcd_remap & (nar ? 2 : 1)) t = (t & 7) * (T >> 3) + (t >> 3);
+        // logical order: token-tile group (walk_gm token tiles), weight strip, token tile inside the group
+        const int per_group = p.walk_gm * ns;
+        const int grp = t / per_group, in_grp = t - grp * per_group;
+        const int tn = in_grp / p.walk_gm, tm = grp * p.walk_gm + (in_grp - tn * p.walk_gm);
         tok0 = tm * p.tile_m; M_end = min(p.M, tok0 + p.tile_m);
         row0 = nar ? tn * 96 : p.narrow * 96 + tn * BN;
         N_end = nar ? row0 + 96 : p.N;
         col0 = row0;
-    } else {
-        const int T = p.tiles_m * p.tiles_n;
-        if (p.xcd_remap) t = (t & 7) * (T >> 3) + (t >> 3);
-        // logical order: token-tile group (walk_gm token tiles), weight strip, token tile inside the group
-        const int per_group = p.walk_gm * p.tiles_n;
-        const int grp = t / per_group, in_grp = t - grp * per_group;
-        const int tn = in_grp / p.walk_gm, tm = grp * p.walk_gm + (in_grp - tn * p.walk_gm);
-        tok0 = tm * p.tile_m; row0 = tn * BN; col0 = row0; M_end = min(p.M, tok0 + p.tile_m); N_end = p.N;
     }
     const GemmOperand op = p.op[op_i];
     // Wave roles.  A full tile gives each wave 32 tokens x 128 rows (4 row tiles).  A tile with few live
@@ -568,7 +567,10 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
     // its idle slots cost up to a whole tile's time.  A tile of 96 weight rows runs three of the four row tiles (about 0.8
     // of the time), so with the first `narrow` strips of N cut at 96 rows and dispatched last, the last round can be made
     // of shorter tiles on more slots: 15360 rows x 2048 tokens = 1920 tiles = 3.75 rounds of 512 becomes 1536 tiles of
-    // 128 rows (3 rounds) and one round of 512 tiles of 96.  Chosen by the estimated makespan; taken when it saves 3 %.
+    // 128 rows (3 rounds) and one round of 512 tiles of 96.  Chosen by the estimated makespan; taken when it saves 3 %, for
+    // Q6_K weights only: measured at that shape Q6_K 598 -> 575 us per launch, Q8_0 339.6 -> 337 and Q4_0 350.7 -> 349 (inside
+    // the spread between machines, with 2.5 % more vector instructions per launch: a partly filled round runs faster
+    // already, a workgroup alone on a CU has its SIMDs to itself).  The knob forces any number of strips for any format.
     if (Z == 1 && bm == 128 && !dump && c->tune_gemm_narrow != 1) {
         const auto makespan = [&](int b) -> double {   // in 128-row tile times; -1: N does not split that way
             if (96 * b > p.N) return -1.0;
@@ -595,7 +597,7 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
         int best_b = 0;
         if (c->tune_gemm_narrow > 1) {
             best_b = std::min(c->tune_gemm_narrow - 1, p.N / 96);
-        } else if (T > slots) {
+        } else if (T > slots && w.type == kQ6_K) {
             double best = makespan(0);
             const double need = 0.97 * best;
             for (int b = 1; (long)b * p.tiles_m <= slots && 96 * b <= p.N; b++) {
@@ -606,6 +608,7 @@ int launch_gemm(smx_ctx* c, const Weight& w, const int8_t* xq, const float* xd, 
         if (best_b > 0) {
             p.narrow = best_b;
             p.tiles_n = best_b + (p.N - 96 * best_b + BN - 1) / BN;
+            p.xcd_remap = (((p.tiles_n - best_b) * p.tiles_m) % 8 == 0 ? 1 : 0) | ((best_b * p.tiles_m) % 8 == 0 ? 2 : 0);
         }
     }
     const int T_launch = p.tiles_m * p.tiles_n;
